@@ -1,0 +1,131 @@
+/*
+ * phyai_fp8.h - C ABI of the MI355X (gfx950) W8A8 fp8 quantized-linear library.
+ *
+ * Every entry point is `extern "C"`, takes raw device pointers, sizes and a HIP
+ * stream (passed as `void*`, i.e. a `hipStream_t`), enqueues work on that stream
+ * and returns without synchronising.  None of them allocates device memory;
+ * scratch space is a caller-owned workspace sized by
+ * phyai_fp8_linear_workspace_bytes().  Return value: 0 on success, a negative
+ * PHYAI_FP8_E* code otherwise; phyai_fp8_last_error() gives the message of the
+ * calling thread's last failure.
+ *
+ * The reference has no native fp8 code: on this path it runs torch tensor ops,
+ * torch._scaled_mm and a flashinfer activation kernel.  Each declaration below
+ * names the reference lines (paths relative to the reference checkout) whose
+ * arithmetic it replaces.
+ *
+ * Layouts.  Activations x: [M, K] bf16, K contiguous, row stride ldx elements.
+ * Codes xq: [M, K] e4m3fn bytes, dense.  Weights w: [N, K] e4m3fn bytes, dense,
+ * K contiguous (the layout Fp8Spec.allocate registers, quant/fp8.py:74-79).
+ * Scales: x_scale [M] fp32, w_scale [N] fp32.  bias: [N] bf16 or NULL.
+ * out: bf16, row stride ldo elements, [M, N] (or [M, N/2] for gated epilogues,
+ * where gate = columns [0, N/2) and up = columns [N/2, N), mlp/dense_mlp.py:11-15).
+ */
+#ifndef PHYAI_FP8_H
+#define PHYAI_FP8_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define PHYAI_FP8_ABI_VERSION 1
+
+enum {
+    PHYAI_FP8_OK = 0,
+    PHYAI_FP8_EINVAL = -1,      /* bad pointer / size / alignment                 */
+    PHYAI_FP8_EUNSUPPORTED = -2, /* shape outside what the kernels handle          */
+    PHYAI_FP8_EWORKSPACE = -3,  /* workspace missing or too small                 */
+    PHYAI_FP8_ELAUNCH = -4      /* HIP reported a launch error                    */
+};
+
+/* Epilogue applied to (acc * x_scale[m] * w_scale[n] + bias[n]).
+ * mlp/dense_mlp.py:87-124 (activation table), :256-265 (where it is applied). */
+enum {
+    PHYAI_FP8_EPI_NONE = 0,
+    PHYAI_FP8_EPI_GEGLU_TANH = 1, /* gelu_tanh(gate) * up  -> [M, N/2]             */
+    PHYAI_FP8_EPI_GEGLU_ERF = 2,  /* gelu_erf(gate) * up   -> [M, N/2]             */
+    PHYAI_FP8_EPI_SWIGLU = 3,     /* silu(gate) * up       -> [M, N/2]             */
+    PHYAI_FP8_EPI_GELU_TANH = 4,  /* plain fc1 -> gelu_tanh -> [M, N]              */
+    PHYAI_FP8_EPI_GELU_ERF = 5    /* plain fc1 -> gelu (erf) -> [M, N]             */
+};
+
+int phyai_fp8_abi_version(void);
+const char *phyai_fp8_last_error(void);
+
+/*
+ * Per-token dynamic activation quantizer.
+ * Replaces Fp8Spec.quantize_activation, PER_CHANNEL/BLOCK branch
+ * (layers/quant/fp8.py:150-155): bf16 absmax per row floored at bf16(1e-12),
+ * scale = fp32(bf16(amax/448)), codes = e4m3fn_rne(fp32(x) / scale).
+ * Bit-exact with that expression.  Requires K % 8 == 0 and 16-byte aligned rows.
+ */
+int phyai_fp8_quant_rowwise(const void *x, int64_t M, int64_t K, int64_t ldx,
+                            void *xq, float *x_scale, void *stream);
+
+/*
+ * Static per-tensor activation quantizer.
+ * Replaces Fp8Spec.quantize_activation, PER_TENSOR branch
+ * (layers/quant/fp8.py:142-148): codes = e4m3fn(clamp(fp32(x)/input_scale[0], +-448)).
+ * input_scale is a device pointer to one fp32.
+ */
+int phyai_fp8_quant_static(const void *x, int64_t M, int64_t K, int64_t ldx,
+                           const float *input_scale, void *xq, void *stream);
+
+/*
+ * Offline per-output-channel weight quantizer: w_scale[n] = absmax_k(W[n,:])/448
+ * in fp32 (floored at FLT_MIN), wq = e4m3fn(clamp(W/w_scale, +-448)).
+ * The reference has no such function (TODO at layers/quant/fp8.py:80-83; its
+ * model-optimizer package is empty); the rule is the benchmark's definition.
+ */
+int phyai_fp8_weight_quant_rowwise(const void *w, int64_t N, int64_t K, int64_t ldw,
+                                   void *wq, float *w_scale, void *stream);
+
+/*
+ * Bytes of workspace phyai_fp8_linear / phyai_fp8_gemm need for this shape.
+ * The workspace must be 256-byte aligned and its first
+ * PHYAI_FP8_WORKSPACE_HEADER_BYTES must be zero before the first call that uses
+ * it; every call leaves them zero again.  Two calls that may run concurrently
+ * must not share a workspace.
+ */
+#define PHYAI_FP8_WORKSPACE_HEADER_BYTES 16384
+size_t phyai_fp8_linear_workspace_bytes(int64_t M, int64_t N, int64_t K, int epilogue);
+
+/*
+ * fp8 x fp8 GEMM on already-quantized activations with fused
+ * dequant-scale-bias-activation epilogue, bf16 out.
+ * Replaces the torch._scaled_mm call of TorchKernel._fp8_per_channel
+ * (layers/linear/backends/torch.py:166-175) and, for epilogue != NONE, the
+ * following activation launch of DenseMLP.forward (mlp/dense_mlp.py:256-265).
+ * Per-tensor layers (torch.py:123-153) pass x_scale_is_scalar = 1 and a pointer
+ * to the single input scale.  Requires K % 16 == 0 and N % 16 == 0
+ * (the same gate as TorchKernel.can_handle, torch.py:91).
+ */
+int phyai_fp8_gemm(const void *xq, const float *x_scale, int x_scale_is_scalar,
+                   const void *w, const float *w_scale, const void *bias,
+                   void *out, int64_t ldo, int64_t M, int64_t N, int64_t K,
+                   int epilogue, void *workspace, size_t workspace_bytes, void *stream);
+
+/*
+ * The whole quantized linear: per-token quantization of bf16 x followed by the
+ * GEMM above, as one call.  Replaces TorchKernel._fp8_per_channel
+ * (layers/linear/backends/torch.py:155-176) end to end.
+ */
+int phyai_fp8_linear(const void *x, int64_t ldx, const void *w, const float *w_scale,
+                     const void *bias, void *out, int64_t ldo, int64_t M, int64_t N,
+                     int64_t K, int epilogue, void *workspace, size_t workspace_bytes,
+                     void *stream);
+
+/*
+ * Test hook: run the device fp32 -> e4m3fn cast used by the quantizers over n
+ * values (device pointers), so that it can be compared exhaustively with the
+ * CPU cast.  Not part of the reference surface.
+ */
+int phyai_fp8_debug_cast_e4m3(const float *v, int64_t n, void *codes, void *stream);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* PHYAI_FP8_H */

@@ -1,0 +1,74 @@
+"""ctypes loader for ``libphyai_fp8.so`` (the gfx950 HIP kernels behind a C ABI).
+
+There is no fallback: if the shared library is missing or does not export the
+symbols the header declares, importing the ops fails loudly.
+"""
+
+from __future__ import annotations
+
+import ctypes
+import os
+import subprocess
+
+_PKG = os.path.dirname(os.path.abspath(__file__))
+LIB_PATH = os.path.join(_PKG, "lib", "libphyai_fp8.so")
+CSRC_DIR = os.path.join(_PKG, "csrc")
+ABI_VERSION = 1
+
+# name -> (restype, argtypes); mirrors include/phyai_fp8.h one to one.
+_i64, _vp, _int, _sz = ctypes.c_int64, ctypes.c_void_p, ctypes.c_int, ctypes.c_size_t
+SIGNATURES: dict[str, tuple[object, list[object]]] = {
+    "phyai_fp8_abi_version": (_int, []),
+    "phyai_fp8_last_error": (ctypes.c_char_p, []),
+    "phyai_fp8_quant_rowwise": (_int, [_vp, _i64, _i64, _i64, _vp, _vp, _vp]),
+    "phyai_fp8_quant_static": (_int, [_vp, _i64, _i64, _i64, _vp, _vp, _vp]),
+    "phyai_fp8_weight_quant_rowwise": (_int, [_vp, _i64, _i64, _i64, _vp, _vp, _vp]),
+    "phyai_fp8_linear_workspace_bytes": (_sz, [_i64, _i64, _i64, _int]),
+    "phyai_fp8_gemm": (_int, [_vp, _vp, _int, _vp, _vp, _vp, _vp, _i64, _i64, _i64, _i64, _int, _vp, _sz, _vp]),
+    "phyai_fp8_linear": (_int, [_vp, _i64, _vp, _vp, _vp, _vp, _i64, _i64, _i64, _i64, _int, _vp, _sz, _vp]),
+    "phyai_fp8_debug_cast_e4m3": (_int, [_vp, _i64, _vp, _vp]),
+}
+
+
+class Fp8LibraryError(RuntimeError):
+    """The native library is missing, stale, or a call into it failed."""
+
+
+_lib: ctypes.CDLL | None = None
+
+
+def build(verbose: bool = False) -> str:
+    """Compile the HIP sources for gfx950 with hipcc (``make -C phyai_amd/csrc``)."""
+    out = None if verbose else subprocess.DEVNULL
+    subprocess.check_call(["make", "-C", CSRC_DIR, "-j8"], stdout=out, stderr=out)
+    return LIB_PATH
+
+
+def load() -> ctypes.CDLL:
+    global _lib
+    if _lib is not None:
+        return _lib
+    if not os.path.exists(LIB_PATH):
+        raise Fp8LibraryError(
+            f"{LIB_PATH} not found: build it with `make -C {CSRC_DIR}` "
+            "(or phyai_amd._lib.build()); there is no non-HIP fallback"
+        )
+    lib = ctypes.CDLL(LIB_PATH)
+    for name, (res, args) in SIGNATURES.items():
+        try:
+            fn = getattr(lib, name)
+        except AttributeError as e:
+            raise Fp8LibraryError(f"{LIB_PATH} does not export {name}; rebuild it") from e
+        fn.restype = res
+        fn.argtypes = args
+    got = lib.phyai_fp8_abi_version()
+    if got != ABI_VERSION:
+        raise Fp8LibraryError(f"{LIB_PATH} has ABI version {got}, expected {ABI_VERSION}; rebuild it")
+    _lib = lib
+    return lib
+
+
+def check(rc: int, what: str) -> None:
+    if rc != 0:
+        msg = load().phyai_fp8_last_error()
+        raise Fp8LibraryError(f"{what} failed (rc={rc}): {msg.decode() if msg else ''}")

@@ -1,0 +1,170 @@
+// extern "C" boundary of the fp8 linear library: argument validation, workspace
+// carving and kernel selection.  No allocation, no synchronisation.
+#include <hip/hip_runtime.h>
+#include <stdarg.h>
+#include <stdio.h>
+
+#include "../../include/phyai_fp8.h"
+#include "fp8_device.h"
+#include "launch.h"
+
+namespace {
+
+thread_local char g_err[256] = "";
+
+int fail(int code, const char* fmt, ...) {
+    va_list ap;
+    va_start(ap, fmt);
+    vsnprintf(g_err, sizeof(g_err), fmt, ap);
+    va_end(ap);
+    return code;
+}
+
+int check_launch(const char* what) {
+    hipError_t e = hipGetLastError();
+    if (e != hipSuccess) return fail(PHYAI_FP8_ELAUNCH, "%s: %s", what, hipGetErrorString(e));
+    return PHYAI_FP8_OK;
+}
+
+bool aligned(const void* p, size_t a) { return (reinterpret_cast<uintptr_t>(p) & (a - 1)) == 0; }
+
+size_t align_up(size_t v, size_t a) { return (v + a - 1) / a * a; }
+
+constexpr int64_t kMaxElems = (int64_t)1 << 31;  // kernels index rows with 32-bit offsets
+
+int check_epilogue(int epilogue, int64_t N) {
+    if (epilogue < PHYAI_FP8_EPI_NONE || epilogue > PHYAI_FP8_EPI_GELU_ERF)
+        return fail(PHYAI_FP8_EINVAL, "unknown epilogue %d", epilogue);
+    if (phyai::epi_is_gated(epilogue) && (N % 32) != 0)
+        return fail(PHYAI_FP8_EUNSUPPORTED, "gated epilogue needs N %% 32 == 0 (gate/up halves of 16-aligned width), got N=%lld", (long long)N);
+    return 0;
+}
+
+// Workspace layout of phyai_fp8_linear: [GEMM region][xq codes][x_scale].
+struct LinearCarve {
+    size_t gemm_bytes, xq_off, xs_off, total;
+};
+LinearCarve carve(int64_t M, int64_t N, int64_t K, int epilogue) {
+    LinearCarve c;
+    c.gemm_bytes = align_up(phyai::gemm_workspace_bytes(M, N, K, epilogue), 256);
+    c.xq_off = c.gemm_bytes;
+    c.xs_off = c.xq_off + align_up((size_t)(M > 0 ? M : 0) * (size_t)(K > 0 ? K : 0), 256);
+    c.total = c.xs_off + align_up((size_t)(M > 0 ? M : 0) * sizeof(float), 256);
+    return c;
+}
+
+int check_quant_args(const char* fn, const void* x, int64_t M, int64_t K, int64_t ldx, const void* xq) {
+    if (M < 0 || K <= 0) return fail(PHYAI_FP8_EINVAL, "%s: bad shape M=%lld K=%lld", fn, (long long)M, (long long)K);
+    if (M == 0) return 0;
+    if (!x || !xq) return fail(PHYAI_FP8_EINVAL, "%s: null pointer", fn);
+    if (K % 8 != 0) return fail(PHYAI_FP8_EUNSUPPORTED, "%s: K=%lld must be a multiple of 8", fn, (long long)K);
+    if (ldx < K || ldx % 8 != 0) return fail(PHYAI_FP8_EINVAL, "%s: row stride %lld must be >= K and a multiple of 8", fn, (long long)ldx);
+    if (!aligned(x, 16) || !aligned(xq, 8)) return fail(PHYAI_FP8_EINVAL, "%s: x must be 16-byte and xq 8-byte aligned", fn);
+    if (M * ldx >= kMaxElems * 4 || M >= kMaxElems) return fail(PHYAI_FP8_EUNSUPPORTED, "%s: tensor too large", fn);
+    return 0;
+}
+
+}  // namespace
+
+extern "C" {
+
+int phyai_fp8_abi_version(void) { return PHYAI_FP8_ABI_VERSION; }
+
+const char* phyai_fp8_last_error(void) { return g_err; }
+
+int phyai_fp8_quant_rowwise(const void* x, int64_t M, int64_t K, int64_t ldx, void* xq,
+                            float* x_scale, void* stream) {
+    if (int rc = check_quant_args("phyai_fp8_quant_rowwise", x, M, K, ldx, xq)) return rc;
+    if (M == 0) return PHYAI_FP8_OK;
+    if (!x_scale) return fail(PHYAI_FP8_EINVAL, "phyai_fp8_quant_rowwise: null x_scale");
+    phyai::launch_quant_rowwise(x, M, K, ldx, xq, x_scale, static_cast<hipStream_t>(stream));
+    return check_launch("phyai_fp8_quant_rowwise");
+}
+
+int phyai_fp8_quant_static(const void* x, int64_t M, int64_t K, int64_t ldx,
+                           const float* input_scale, void* xq, void* stream) {
+    if (int rc = check_quant_args("phyai_fp8_quant_static", x, M, K, ldx, xq)) return rc;
+    if (M == 0) return PHYAI_FP8_OK;
+    if (!input_scale) return fail(PHYAI_FP8_EINVAL, "phyai_fp8_quant_static: null input_scale");
+    phyai::launch_quant_static(x, M, K, ldx, input_scale, xq, static_cast<hipStream_t>(stream));
+    return check_launch("phyai_fp8_quant_static");
+}
+
+int phyai_fp8_weight_quant_rowwise(const void* w, int64_t N, int64_t K, int64_t ldw, void* wq,
+                                   float* w_scale, void* stream) {
+    if (int rc = check_quant_args("phyai_fp8_weight_quant_rowwise", w, N, K, ldw, wq)) return rc;
+    if (N == 0) return PHYAI_FP8_OK;
+    if (!w_scale) return fail(PHYAI_FP8_EINVAL, "phyai_fp8_weight_quant_rowwise: null w_scale");
+    phyai::launch_weight_quant(w, N, K, ldw, wq, w_scale, static_cast<hipStream_t>(stream));
+    return check_launch("phyai_fp8_weight_quant_rowwise");
+}
+
+size_t phyai_fp8_linear_workspace_bytes(int64_t M, int64_t N, int64_t K, int epilogue) {
+    return carve(M, N, K, epilogue).total;
+}
+
+int phyai_fp8_gemm(const void* xq, const float* x_scale, int x_scale_is_scalar, const void* w,
+                   const float* w_scale, const void* bias, void* out, int64_t ldo, int64_t M,
+                   int64_t N, int64_t K, int epilogue, void* workspace, size_t workspace_bytes,
+                   void* stream) {
+    if (M < 0 || N <= 0 || K <= 0)
+        return fail(PHYAI_FP8_EINVAL, "phyai_fp8_gemm: bad shape M=%lld N=%lld K=%lld", (long long)M, (long long)N, (long long)K);
+    if (int rc = check_epilogue(epilogue, N)) return rc;
+    if (K % 16 != 0 || N % 16 != 0)
+        return fail(PHYAI_FP8_EUNSUPPORTED, "phyai_fp8_gemm: K=%lld and N=%lld must be multiples of 16", (long long)K, (long long)N);
+    if (M == 0) return PHYAI_FP8_OK;
+    if (!xq || !x_scale || !w || !w_scale || !out) return fail(PHYAI_FP8_EINVAL, "phyai_fp8_gemm: null pointer");
+    if (!aligned(xq, 16) || !aligned(w, 16)) return fail(PHYAI_FP8_EINVAL, "phyai_fp8_gemm: xq and w must be 16-byte aligned");
+    const int64_t n_out = phyai::epi_is_gated(epilogue) ? N / 2 : N;
+    if (ldo < n_out) return fail(PHYAI_FP8_EINVAL, "phyai_fp8_gemm: ldo=%lld < output width %lld", (long long)ldo, (long long)n_out);
+    if (M * K >= kMaxElems || N * K >= kMaxElems || M * ldo >= kMaxElems * 2)
+        return fail(PHYAI_FP8_EUNSUPPORTED, "phyai_fp8_gemm: operand larger than 2^31 elements");
+    if (workspace && !aligned(workspace, 256)) return fail(PHYAI_FP8_EINVAL, "phyai_fp8_gemm: workspace must be 256-byte aligned");
+
+    phyai::GemmProblem g;
+    g.xq = static_cast<const uint8_t*>(xq);
+    g.x_scale = x_scale;
+    g.x_scale_is_scalar = x_scale_is_scalar ? 1 : 0;
+    g.w = static_cast<const uint8_t*>(w);
+    g.w_scale = w_scale;
+    g.bias = static_cast<const uint16_t*>(bias);
+    g.out = static_cast<uint16_t*>(out);
+    g.ldo = ldo;
+    g.M = (int)M; g.N = (int)N; g.K = (int)K;
+    g.epilogue = epilogue;
+    g.workspace = workspace;
+    g.workspace_bytes = workspace_bytes;
+    const int rc = phyai::launch_gemm(g, static_cast<hipStream_t>(stream));
+    if (rc == -3)
+        return fail(PHYAI_FP8_EWORKSPACE, "phyai_fp8_gemm: workspace of %zu bytes is too small, need %zu",
+                    workspace ? workspace_bytes : (size_t)0, phyai::gemm_workspace_bytes(M, N, K, epilogue));
+    if (rc != 0) return fail(PHYAI_FP8_EUNSUPPORTED, "phyai_fp8_gemm: no kernel for this problem (rc=%d)", rc);
+    return check_launch("phyai_fp8_gemm");
+}
+
+int phyai_fp8_linear(const void* x, int64_t ldx, const void* w, const float* w_scale,
+                     const void* bias, void* out, int64_t ldo, int64_t M, int64_t N, int64_t K,
+                     int epilogue, void* workspace, size_t workspace_bytes, void* stream) {
+    if (M < 0 || N <= 0 || K <= 0)
+        return fail(PHYAI_FP8_EINVAL, "phyai_fp8_linear: bad shape M=%lld N=%lld K=%lld", (long long)M, (long long)N, (long long)K);
+    if (M == 0) return PHYAI_FP8_OK;
+    const LinearCarve c = carve(M, N, K, epilogue);
+    if (!workspace || workspace_bytes < c.total)
+        return fail(PHYAI_FP8_EWORKSPACE, "phyai_fp8_linear: workspace of %zu bytes is too small, need %zu",
+                    workspace ? workspace_bytes : (size_t)0, c.total);
+    if (!aligned(workspace, 256)) return fail(PHYAI_FP8_EINVAL, "phyai_fp8_linear: workspace must be 256-byte aligned");
+    uint8_t* ws = static_cast<uint8_t*>(workspace);
+    void* xq = ws + c.xq_off;
+    float* xs = reinterpret_cast<float*>(ws + c.xs_off);
+    if (int rc = phyai_fp8_quant_rowwise(x, M, K, ldx, xq, xs, stream)) return rc;
+    return phyai_fp8_gemm(xq, xs, 0, w, w_scale, bias, out, ldo, M, N, K, epilogue, workspace,
+                          c.gemm_bytes, stream);
+}
+
+int phyai_fp8_debug_cast_e4m3(const float* v, int64_t n, void* codes, void* stream) {
+    if (n < 0 || (n > 0 && (!v || !codes))) return fail(PHYAI_FP8_EINVAL, "phyai_fp8_debug_cast_e4m3: bad arguments");
+    phyai::launch_debug_cast(v, n, codes, static_cast<hipStream_t>(stream));
+    return check_launch("phyai_fp8_debug_cast_e4m3");
+}
+
+}  // extern "C"

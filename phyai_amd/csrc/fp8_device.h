@@ -1,0 +1,82 @@
+// Device-side helpers shared by the gfx950 fp8 kernels: bf16 <-> fp32, the
+// e4m3fn encoder, wavefront reductions and the epilogue activations.
+#pragma once
+
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+namespace phyai {
+
+constexpr int kWave = 64;          // CDNA wavefront width
+constexpr float kFp8Max = 448.0f;  // largest finite e4m3fn
+constexpr uint32_t kAmaxFloorBf16 = 0x2B8D;  // bf16(1e-12): clamp_min floor of the row absmax
+
+typedef int v8i __attribute__((ext_vector_type(8)));
+typedef int v4i __attribute__((ext_vector_type(4)));
+typedef float v16f __attribute__((ext_vector_type(16)));
+typedef float v4f __attribute__((ext_vector_type(4)));
+
+__device__ __forceinline__ float bf16_bits_to_f32(uint32_t h) { return __uint_as_float(h << 16); }
+
+// fp32 -> bf16 bits, round to nearest even, NaN -> 0x7FC0.
+__device__ __forceinline__ uint32_t f32_to_bf16_bits(float f) {
+    uint32_t u = __float_as_uint(f);
+    uint32_t r = (u + 0x7FFFu + ((u >> 16) & 1u)) >> 16;
+    return (f != f) ? 0x7FC0u : r;
+}
+
+// Two fp32 -> two e4m3fn codes (OCP, round to nearest even) in the low 16 bits.
+// The hardware convert is used for the in-range part; values at or beyond 480
+// and NaN take the NaN code with the input's sign, which is what a software
+// RNE cast without saturation gives.
+__device__ __forceinline__ uint32_t e4m3_pack2(float a, float b) {
+    uint32_t w = (uint32_t)__builtin_amdgcn_cvt_pk_fp8_f32(a, b, 0, false);
+    uint32_t ua = __float_as_uint(a), ub = __float_as_uint(b);
+    if ((ua & 0x7FFFFFFFu) >= 0x43F00000u) w = (w & 0xFF00u) | ((ua >> 24) & 0x80u) | 0x7Fu;
+    if ((ub & 0x7FFFFFFFu) >= 0x43F00000u) w = (w & 0x00FFu) | ((((ub >> 24) & 0x80u) | 0x7Fu) << 8);
+    return w & 0xFFFFu;
+}
+
+__device__ __forceinline__ uint32_t wave_max_u32(uint32_t v) {
+#pragma unroll
+    for (int off = 32; off >= 1; off >>= 1) {
+        uint32_t o = (uint32_t)__shfl_xor((int)v, off, kWave);
+        v = o > v ? o : v;
+    }
+    return v;
+}
+
+// ---- epilogue activations (fp32 math) ------------------------------------
+__device__ __forceinline__ float gelu_tanh_f(float v) {
+    const float k0 = 0.7978845608028654f, k1 = 0.044715f;
+    float u = k0 * (v + k1 * v * v * v);
+    // tanh(u) = 1 - 2 / (exp(2u) + 1); exact limits at +-inf, no cancellation blow-up
+    float t = 1.0f - 2.0f * __builtin_amdgcn_rcpf(__expf(2.0f * u) + 1.0f);
+    return 0.5f * v * (1.0f + t);
+}
+__device__ __forceinline__ float gelu_erf_f(float v) { return 0.5f * v * (1.0f + erff(v * 0.70710678118654752f)); }
+__device__ __forceinline__ float silu_f(float v) { return v * __builtin_amdgcn_rcpf(1.0f + __expf(-v)); }
+
+enum Epilogue : int {
+    EPI_NONE = 0,
+    EPI_GEGLU_TANH = 1,
+    EPI_GEGLU_ERF = 2,
+    EPI_SWIGLU = 3,
+    EPI_GELU_TANH = 4,
+    EPI_GELU_ERF = 5,
+};
+__host__ __device__ constexpr bool epi_is_gated(int e) { return e >= EPI_GEGLU_TANH && e <= EPI_SWIGLU; }
+
+template <int EPI>
+__device__ __forceinline__ float apply_act(float v) {
+    if constexpr (EPI == EPI_GEGLU_TANH || EPI == EPI_GELU_TANH) return gelu_tanh_f(v);
+    else if constexpr (EPI == EPI_GEGLU_ERF || EPI == EPI_GELU_ERF) return gelu_erf_f(v);
+    else if constexpr (EPI == EPI_SWIGLU) return silu_f(v);
+    else return v;
+}
+
+// Round an fp32 value through bf16 (the reference materialises the GEMM output
+// as a bf16 tensor before the activation kernel reads it).
+__device__ __forceinline__ float round_bf16(float v) { return bf16_bits_to_f32(f32_to_bf16_bits(v)); }
+
+}  // namespace phyai

@@ -1,0 +1,369 @@
+// LDS-staged fp8 x fp8 MFMA GEMM (NT: A = xq [M,K], B = w [N,K], both K-contiguous)
+// with the dequant-scale-bias-activation epilogue fused, bf16 out.
+//
+// Workgroup = 256 threads = 4 wavefronts arranged WAVES_M x WAVES_N over a
+// BM x BN output tile; K is consumed in 128-byte slabs, double-buffered in LDS.
+// Global -> LDS: each thread moves 16 bytes per pass, 8 threads cover one
+// 128-byte row slab (one cache line), 32 rows per pass.  LDS rows are 128 bytes;
+// the 16-byte chunk index is XOR-ed with (row & 7) so that both the 128-bit
+// stores and the MFMA operand reads (32 rows x the same logical chunk) spread
+// over all banks.
+// MFMA: v_mfma_f32_32x32x64_f8f6f4 (fp8 e4m3 x fp8 e4m3, fp32 accumulate).  Lane l
+// supplies row (l % 32) of the 32x64 operand block and 32 consecutive K bytes
+// starting at 32 * (l / 32); A and B use the same K split, so the dot products
+// line up.  Accumulator register r of lane l is C[8*(r/4) + 4*(l/32) + r%4][l%32].
+//
+// Gated epilogues pair column n (gate) with column n + N/2 (up).  The B tile of
+// a gated kernel is therefore gathered from two row ranges of w: within each
+// wavefront's WN columns the first WN/2 are gate columns and the second WN/2 the
+// matching up columns, so the pair sits in the same lane of two accumulators.
+//
+// Split-K (grid.z > 1): each split stores its fp32 accumulators to the
+// workspace in fragment order; the last split to arrive at the tile's counter
+// (device-scope atomic) sums all partials in split order - a fixed order, so
+// results are reproducible - and runs the epilogue.  It then resets the
+// counter, which keeps the workspace header zero between calls.
+#include "fp8_device.h"
+#include "launch.h"
+
+namespace phyai {
+
+constexpr int BK = 128;  // bytes (= fp8 elements) of K per LDS slab
+
+struct TileArgs {
+    const uint8_t* __restrict__ a;   // xq
+    const uint8_t* __restrict__ b;   // w
+    const float* __restrict__ a_scale;
+    const float* __restrict__ b_scale;
+    const uint16_t* __restrict__ bias;
+    uint16_t* __restrict__ out;
+    float* __restrict__ partials;
+    int* __restrict__ counters;
+    int64_t ldo;
+    int M, N, K;
+    int a_scale_scalar;
+    int k_tiles_per_split;  // in BK slabs
+};
+
+__device__ __forceinline__ v8i lds_frag(const uint8_t* buf, int row, int ks, int h) {
+    const int c0 = ks * 4 + h * 2;
+    const int sw = row & 7;
+    const uint8_t* r = buf + row * BK;
+    const v4i lo = *reinterpret_cast<const v4i*>(r + ((c0 ^ sw) << 4));
+    const v4i hi = *reinterpret_cast<const v4i*>(r + (((c0 + 1) ^ sw) << 4));
+    v8i f;
+    f[0] = lo[0]; f[1] = lo[1]; f[2] = lo[2]; f[3] = lo[3];
+    f[4] = hi[0]; f[5] = hi[1]; f[6] = hi[2]; f[7] = hi[3];
+    return f;
+}
+
+template <int BM, int BN, int WAVES_M, int WAVES_N, int EPI, bool SPLITK>
+__global__ __launch_bounds__(256) void gemm_fp8_tile_kernel(const TileArgs p) {
+    static_assert(WAVES_M * WAVES_N == 4, "4 wavefronts per workgroup");
+    constexpr bool GATED = epi_is_gated(EPI);
+    constexpr int WM = BM / WAVES_M, WN = BN / WAVES_N;
+    constexpr int TM = WM / 32, TN = WN / 32;
+    static_assert(TM >= 1 && TN >= 1, "wave tile must hold a 32x32 block");
+    static_assert(!GATED || (TN % 2 == 0), "gated epilogue needs gate/up block pairs per wave");
+    constexpr int PA = BM / 32, PB = BN / 32;  // loader passes
+    constexpr int TILE_BYTES = (BM + BN) * BK;
+
+    __shared__ __attribute__((aligned(16))) uint8_t lds[2 * TILE_BYTES];
+    __shared__ int s_last;
+
+    const int tid = threadIdx.x;
+    const int lane = tid & 63, wave = tid >> 6;
+    const int wm = wave / WAVES_N, wn = wave % WAVES_N;
+    const int l32 = lane & 31, h = lane >> 5;
+
+    const int m0 = blockIdx.y * BM;
+    // Gated: a tile spans BN/2 gate columns and the BN/2 up columns that pair with them.
+    const int half_n = p.N / 2;
+    const int n0 = GATED ? blockIdx.x * (BN / 2) : blockIdx.x * BN;
+
+    // ---- loader geometry: thread -> (row within pass, 16-byte chunk) ----------
+    const int lrow = tid >> 3, lchunk = tid & 7;
+    int a_off[PA], b_off[PB];
+#pragma unroll
+    for (int i = 0; i < PA; ++i) {
+        int r = m0 + i * 32 + lrow;
+        r = r < p.M ? r : p.M - 1;
+        a_off[i] = r * p.K;
+    }
+#pragma unroll
+    for (int i = 0; i < PB; ++i) {
+        const int jj = i * 32 + lrow;  // column within the tile
+        int r;
+        if constexpr (GATED) {
+            const int w_ = jj / WN, j = jj % WN;
+            const int up = j / (WN / 2);
+            int g = n0 + w_ * (WN / 2) + j % (WN / 2);
+            g = g < half_n ? g : half_n - 1;
+            r = up * half_n + g;
+        } else {
+            r = n0 + jj;
+            r = r < p.N ? r : p.N - 1;
+        }
+        b_off[i] = r * p.K;
+    }
+
+    const int k_begin = SPLITK ? blockIdx.z * p.k_tiles_per_split * BK : 0;
+    int k_end = SPLITK ? k_begin + p.k_tiles_per_split * BK : p.K;
+    k_end = k_end < p.K ? k_end : p.K;
+    const int n_slabs = (k_end - k_begin + BK - 1) / BK;
+
+    uint4 ra[PA], rb[PB];
+    auto load_global = [&](int slab) {
+        const int k = k_begin + slab * BK + lchunk * 16;
+        const bool ok = k < k_end;
+#pragma unroll
+        for (int i = 0; i < PA; ++i)
+            ra[i] = ok ? *reinterpret_cast<const uint4*>(p.a + a_off[i] + k) : make_uint4(0, 0, 0, 0);
+#pragma unroll
+        for (int i = 0; i < PB; ++i)
+            rb[i] = ok ? *reinterpret_cast<const uint4*>(p.b + b_off[i] + k) : make_uint4(0, 0, 0, 0);
+    };
+    auto store_lds = [&](int buf) {
+        uint8_t* base = lds + buf * TILE_BYTES;
+        const int sw = (lchunk ^ (lrow & 7)) << 4;
+#pragma unroll
+        for (int i = 0; i < PA; ++i)
+            *reinterpret_cast<uint4*>(base + (i * 32 + lrow) * BK + sw) = ra[i];
+#pragma unroll
+        for (int i = 0; i < PB; ++i)
+            *reinterpret_cast<uint4*>(base + BM * BK + (i * 32 + lrow) * BK + sw) = rb[i];
+    };
+
+    v16f acc[TM][TN];
+#pragma unroll
+    for (int i = 0; i < TM; ++i)
+#pragma unroll
+        for (int j = 0; j < TN; ++j)
+#pragma unroll
+            for (int r = 0; r < 16; ++r) acc[i][j][r] = 0.f;
+
+    if (n_slabs > 0) {
+        load_global(0);
+        store_lds(0);
+    }
+    __syncthreads();
+
+    for (int s = 0; s < n_slabs; ++s) {
+        const int cur = s & 1;
+        if (s + 1 < n_slabs) load_global(s + 1);
+        const uint8_t* abuf = lds + cur * TILE_BYTES;
+        const uint8_t* bbuf = abuf + BM * BK;
+#pragma unroll
+        for (int ks = 0; ks < 2; ++ks) {
+            v8i fa[TM], fb[TN];
+#pragma unroll
+            for (int i = 0; i < TM; ++i) fa[i] = lds_frag(abuf, wm * WM + i * 32 + l32, ks, h);
+#pragma unroll
+            for (int j = 0; j < TN; ++j) fb[j] = lds_frag(bbuf, wn * WN + j * 32 + l32, ks, h);
+#pragma unroll
+            for (int i = 0; i < TM; ++i)
+#pragma unroll
+                for (int j = 0; j < TN; ++j)
+                    acc[i][j] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(
+                        fa[i], fb[j], acc[i][j], 0, 0, 0, 0, 0, 0);
+        }
+        if (s + 1 < n_slabs) store_lds(cur ^ 1);
+        __syncthreads();
+    }
+
+    // ---- split-K: publish partials, last arriver reduces -----------------------
+    if constexpr (SPLITK) {
+        const int S = gridDim.z;
+        const int tile = blockIdx.y * gridDim.x + blockIdx.x;
+        constexpr int FRAG = TM * TN * 16;  // floats per thread
+        float* mine = p.partials + ((size_t)tile * S + blockIdx.z) * (FRAG * 256);
+#pragma unroll
+        for (int i = 0; i < TM; ++i)
+#pragma unroll
+            for (int j = 0; j < TN; ++j)
+#pragma unroll
+                for (int r = 0; r < 16; ++r) mine[((i * TN + j) * 16 + r) * 256 + tid] = acc[i][j][r];
+        __threadfence();
+        __syncthreads();
+        if (tid == 0) {
+            const int old = __hip_atomic_fetch_add(p.counters + tile, 1, __ATOMIC_ACQ_REL,
+                                                   __HIP_MEMORY_SCOPE_AGENT);
+            s_last = (old == S - 1);
+        }
+        __syncthreads();
+        if (!s_last) return;
+        __threadfence();
+        const float* all = p.partials + (size_t)tile * S * (FRAG * 256);
+#pragma unroll
+        for (int i = 0; i < TM; ++i)
+#pragma unroll
+            for (int j = 0; j < TN; ++j)
+#pragma unroll
+                for (int r = 0; r < 16; ++r) acc[i][j][r] = 0.f;
+        for (int z = 0; z < S; ++z) {
+            const float* pz = all + (size_t)z * (FRAG * 256);
+#pragma unroll
+            for (int i = 0; i < TM; ++i)
+#pragma unroll
+                for (int j = 0; j < TN; ++j)
+#pragma unroll
+                    for (int r = 0; r < 16; ++r)
+                        acc[i][j][r] += __builtin_nontemporal_load(pz + ((i * TN + j) * 16 + r) * 256 + tid);
+        }
+        if (tid == 0)
+            __hip_atomic_store(p.counters + tile, 0, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    }
+
+    // ---- epilogue ------------------------------------------------------------
+    constexpr int TNO = GATED ? TN / 2 : TN;  // output column blocks per wave
+#pragma unroll
+    for (int j = 0; j < TNO; ++j) {
+        int n_gate, n_out;
+        if constexpr (GATED) {
+            n_out = n0 + wn * (WN / 2) + j * 32 + l32;  // column in [0, N/2)
+            n_gate = n_out;
+        } else {
+            n_out = n0 + wn * WN + j * 32 + l32;
+            n_gate = n_out;
+        }
+        const int n_lim = GATED ? half_n : p.N;
+        const bool n_ok = n_out < n_lim;
+        const int n_safe = n_ok ? n_gate : 0;
+        const float sg = p.b_scale[n_safe];
+        const float bg = p.bias ? bf16_bits_to_f32(p.bias[n_safe]) : 0.f;
+        float su = 0.f, bu = 0.f;
+        if constexpr (GATED) {
+            su = p.b_scale[half_n + n_safe];
+            bu = p.bias ? bf16_bits_to_f32(p.bias[half_n + n_safe]) : 0.f;
+        }
+#pragma unroll
+        for (int i = 0; i < TM; ++i) {
+#pragma unroll
+            for (int r = 0; r < 16; ++r) {
+                const int m = m0 + wm * WM + i * 32 + 8 * (r / 4) + 4 * h + (r % 4);
+                if (m < p.M && n_ok) {
+                    const float sa = p.a_scale[p.a_scale_scalar ? 0 : m];
+                    float v = acc[i][j][r] * (sa * sg) + bg;
+                    if constexpr (GATED) {
+                        const float u = acc[i][j + TN / 2][r] * (sa * su) + bu;
+                        v = apply_act<EPI>(round_bf16(v)) * round_bf16(u);
+                    } else if constexpr (EPI != EPI_NONE) {
+                        v = apply_act<EPI>(round_bf16(v));
+                    }
+                    p.out[(int64_t)m * p.ldo + n_out] = (uint16_t)f32_to_bf16_bits(v);
+                }
+            }
+        }
+    }
+}
+
+// ---- host side ---------------------------------------------------------------
+
+constexpr size_t kHeaderBytes = 16384;  // split-K tile counters (4096 ints)
+
+struct TileConfig {
+    int bm, bn;
+    int splits;
+};
+
+static int ceil_div(int a, int b) { return (a + b - 1) / b; }
+
+// Tile shape and split count.  Small M is weight-streaming bound: use the
+// smallest M tile and split K until there are enough workgroups to keep every
+// CU pulling weight bytes.  Large M is MFMA bound: big square tiles, no split.
+static TileConfig pick_config(int M, int N, int K, int epilogue) {
+    const bool gated = epi_is_gated(epilogue);
+    TileConfig c;
+    if (M <= 64) {
+        c.bm = 64;
+        c.bn = gated ? 128 : 64;
+    } else {
+        c.bm = 128;
+        c.bn = 128;
+    }
+    const int n_eff = gated ? N / 2 : N;
+    const int bn_eff = gated ? c.bn / 2 : c.bn;
+    const int tiles = ceil_div(M, c.bm) * ceil_div(n_eff, bn_eff);
+    const int slabs = ceil_div(K, BK);
+    int s = 1;
+    if (tiles < 256) {
+        s = ceil_div(512, tiles);
+        const int max_s = slabs / 2 > 0 ? slabs / 2 : 1;  // at least 2 slabs per split
+        if (s > max_s) s = max_s;
+        if (s > 32) s = 32;
+        if (tiles > 4096) s = 1;
+    }
+    // every split must own at least one slab
+    const int per = ceil_div(slabs, s);
+    s = ceil_div(slabs, per);
+    c.splits = s;
+    return c;
+}
+
+static size_t partial_bytes(const TileConfig& c, int M, int N, int epilogue) {
+    if (c.splits <= 1) return 0;
+    const bool gated = epi_is_gated(epilogue);
+    const int n_eff = gated ? N / 2 : N;
+    const int bn_eff = gated ? c.bn / 2 : c.bn;
+    const size_t tiles = (size_t)ceil_div(M, c.bm) * ceil_div(n_eff, bn_eff);
+    return tiles * c.splits * (size_t)c.bm * c.bn * sizeof(float);
+}
+
+size_t gemm_workspace_bytes(int64_t M, int64_t N, int64_t K, int epilogue) {
+    if (M <= 0 || N <= 0 || K <= 0) return kHeaderBytes;
+    const TileConfig c = pick_config((int)M, (int)N, (int)K, epilogue);
+    return kHeaderBytes + partial_bytes(c, (int)M, (int)N, epilogue);
+}
+
+template <int BM, int BN, int WAVES_M, int WAVES_N, int EPI>
+static void launch_one(const TileArgs& a, dim3 grid, bool split, hipStream_t st) {
+    if (split)
+        hipLaunchKernelGGL((gemm_fp8_tile_kernel<BM, BN, WAVES_M, WAVES_N, EPI, true>), grid, dim3(256), 0, st, a);
+    else
+        hipLaunchKernelGGL((gemm_fp8_tile_kernel<BM, BN, WAVES_M, WAVES_N, EPI, false>), grid, dim3(256), 0, st, a);
+}
+
+template <int EPI>
+static int launch_epi(const TileArgs& a, const TileConfig& c, dim3 grid, hipStream_t st) {
+    constexpr bool GATED = epi_is_gated(EPI);
+    const bool split = c.splits > 1;
+    if (c.bm == 64) {
+        if constexpr (GATED) launch_one<64, 128, 2, 2, EPI>(a, grid, split, st);
+        else launch_one<64, 64, 2, 2, EPI>(a, grid, split, st);
+    } else {
+        launch_one<128, 128, 2, 2, EPI>(a, grid, split, st);
+    }
+    return 0;
+}
+
+int launch_gemm(const GemmProblem& g, hipStream_t st) {
+    if (g.M == 0 || g.N == 0) return 0;
+    const TileConfig c = pick_config(g.M, g.N, g.K, g.epilogue);
+    const bool gated = epi_is_gated(g.epilogue);
+    const int n_eff = gated ? g.N / 2 : g.N;
+    const int bn_eff = gated ? c.bn / 2 : c.bn;
+    const size_t need = kHeaderBytes + partial_bytes(c, g.M, g.N, g.epilogue);
+    if (c.splits > 1 && (g.workspace == nullptr || g.workspace_bytes < need)) return -3;
+
+    TileArgs a;
+    a.a = g.xq; a.b = g.w; a.a_scale = g.x_scale; a.b_scale = g.w_scale; a.bias = g.bias;
+    a.out = g.out; a.ldo = g.ldo; a.M = g.M; a.N = g.N; a.K = g.K;
+    a.a_scale_scalar = g.x_scale_is_scalar;
+    a.counters = static_cast<int*>(g.workspace);
+    a.partials = g.workspace ? reinterpret_cast<float*>(static_cast<uint8_t*>(g.workspace) + kHeaderBytes) : nullptr;
+    const int slabs = ceil_div(g.K, BK);
+    a.k_tiles_per_split = ceil_div(slabs, c.splits);
+    const dim3 grid(ceil_div(n_eff, bn_eff), ceil_div(g.M, c.bm), c.splits);
+
+    switch (g.epilogue) {
+    case EPI_NONE: return launch_epi<EPI_NONE>(a, c, grid, st);
+    case EPI_GEGLU_TANH: return launch_epi<EPI_GEGLU_TANH>(a, c, grid, st);
+    case EPI_GEGLU_ERF: return launch_epi<EPI_GEGLU_ERF>(a, c, grid, st);
+    case EPI_SWIGLU: return launch_epi<EPI_SWIGLU>(a, c, grid, st);
+    case EPI_GELU_TANH: return launch_epi<EPI_GELU_TANH>(a, c, grid, st);
+    case EPI_GELU_ERF: return launch_epi<EPI_GELU_ERF>(a, c, grid, st);
+    default: return -2;
+    }
+}
+
+}  // namespace phyai

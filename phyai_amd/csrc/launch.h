@@ -1,0 +1,36 @@
+// Host-side launch functions implemented by the kernel translation units and
+// called from the C ABI layer.
+#pragma once
+#include <hip/hip_runtime.h>
+#include <stddef.h>
+#include <stdint.h>
+
+namespace phyai {
+
+int launch_quant_rowwise(const void* x, int64_t M, int64_t K, int64_t ldx, void* xq, float* xs,
+                         hipStream_t st);
+int launch_weight_quant(const void* w, int64_t N, int64_t K, int64_t ldw, void* wq, float* ws,
+                        hipStream_t st);
+int launch_quant_static(const void* x, int64_t M, int64_t K, int64_t ldx, const float* input_scale,
+                        void* xq, hipStream_t st);
+int launch_debug_cast(const float* v, int64_t n, void* codes, hipStream_t st);
+
+struct GemmProblem {
+    const uint8_t* xq;      // [M, K]
+    const float* x_scale;   // [M] or [1]
+    int x_scale_is_scalar;
+    const uint8_t* w;       // [N, K]
+    const float* w_scale;   // [N]
+    const uint16_t* bias;   // [N] bf16 or null
+    uint16_t* out;          // [M, N_out] bf16
+    int64_t ldo;
+    int M, N, K;
+    int epilogue;
+    void* workspace;        // header (counters) + split-K partials
+    size_t workspace_bytes;
+};
+
+size_t gemm_workspace_bytes(int64_t M, int64_t N, int64_t K, int epilogue);
+int launch_gemm(const GemmProblem& p, hipStream_t st);
+
+}  // namespace phyai

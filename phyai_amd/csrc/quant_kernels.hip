@@ -1,0 +1,207 @@
+// Activation / weight quantizers for gfx950.
+//
+// One workgroup per row.  Each thread keeps its slice of the row in registers
+// (CHUNKS x 8 bf16 = CHUNKS 128-bit loads), so the row is read from HBM once:
+// pass 1 reduces |x| to the row maximum across the wavefront (cross-lane
+// shuffles) and then across wavefronts through LDS; pass 2 divides, converts to
+// e4m3fn and stores 8 codes per 64-bit store.
+#include "fp8_device.h"
+#include "launch.h"
+
+namespace phyai {
+
+enum QuantMode : int {
+    QUANT_ACT_DYNAMIC = 0,  // bf16 amax floored at bf16(1e-12); scale = fp32(bf16(amax/448)); no clamp
+    QUANT_WEIGHT = 1,       // fp32 amax/448 floored at FLT_MIN; clamp to +-448
+};
+
+template <int THREADS>
+__device__ __forceinline__ uint32_t block_max_u32(uint32_t v, uint32_t* smem) {
+    v = wave_max_u32(v);
+    if constexpr (THREADS > kWave) {
+        constexpr int NW = THREADS / kWave;
+        const int wave = threadIdx.x / kWave, lane = threadIdx.x % kWave;
+        if (lane == 0) smem[wave] = v;
+        __syncthreads();
+        uint32_t r = smem[0];
+#pragma unroll
+        for (int i = 1; i < NW; ++i) r = smem[i] > r ? smem[i] : r;
+        v = r;
+    }
+    return v;
+}
+
+__device__ __forceinline__ uint32_t absmax8(uint4 q, uint32_t m) {
+    const uint32_t w[4] = {q.x, q.y, q.z, q.w};
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+        uint32_t lo = w[i] & 0x7FFFu, hi = (w[i] >> 16) & 0x7FFFu;
+        m = lo > m ? lo : m;
+        m = hi > m ? hi : m;
+    }
+    return m;
+}
+
+template <int MODE>
+__device__ __forceinline__ uint2 encode8(uint4 q, float s) {
+    const uint32_t w[4] = {q.x, q.y, q.z, q.w};
+    uint32_t c[4];
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+        float a = bf16_bits_to_f32(w[i] & 0xFFFFu) / s;
+        float b = bf16_bits_to_f32(w[i] >> 16) / s;
+        if constexpr (MODE == QUANT_WEIGHT) {
+            a = fminf(fmaxf(a, -kFp8Max), kFp8Max);
+            b = fminf(fmaxf(b, -kFp8Max), kFp8Max);
+        }
+        c[i] = e4m3_pack2(a, b);
+    }
+    return make_uint2(c[0] | (c[1] << 16), c[2] | (c[3] << 16));
+}
+
+// Row absmax as bf16 bits.  |bf16| bit patterns order like the values they
+// encode, so an unsigned max over (bits & 0x7FFF) is the bf16 amax; a NaN in the
+// row has the largest pattern and therefore wins, as torch.amax propagates it.
+template <int MODE>
+__device__ __forceinline__ float scale_from_amax_bits(uint32_t amax_bits) {
+    if constexpr (MODE == QUANT_ACT_DYNAMIC) {
+        amax_bits = amax_bits < kAmaxFloorBf16 ? kAmaxFloorBf16 : amax_bits;
+        return bf16_bits_to_f32(f32_to_bf16_bits(bf16_bits_to_f32(amax_bits) / kFp8Max));
+    } else {
+        float s = bf16_bits_to_f32(amax_bits) / kFp8Max;
+        return s >= 1.17549435e-38f ? s : 1.17549435e-38f;
+    }
+}
+
+template <int THREADS, int CHUNKS, int MODE>
+__global__ __launch_bounds__(THREADS) void quant_rows_reg_kernel(
+    const uint16_t* __restrict__ x, int64_t ldx, int K, uint8_t* __restrict__ xq,
+    float* __restrict__ scale) {
+    __shared__ uint32_t smem[THREADS / kWave];
+    const int64_t row = blockIdx.x;
+    const uint16_t* xr = x + row * ldx;
+    uint4 v[CHUNKS];
+    uint32_t m = 0;
+#pragma unroll
+    for (int c = 0; c < CHUNKS; ++c) {
+        const int k = (c * THREADS + threadIdx.x) * 8;
+        v[c] = make_uint4(0, 0, 0, 0);
+        if (k < K) v[c] = *reinterpret_cast<const uint4*>(xr + k);
+        m = absmax8(v[c], m);
+    }
+    m = block_max_u32<THREADS>(m, smem);
+    const float s = scale_from_amax_bits<MODE>(m);
+    if (threadIdx.x == 0) scale[row] = s;
+    uint8_t* qr = xq + row * (int64_t)K;
+#pragma unroll
+    for (int c = 0; c < CHUNKS; ++c) {
+        const int k = (c * THREADS + threadIdx.x) * 8;
+        if (k < K) *reinterpret_cast<uint2*>(qr + k) = encode8<MODE>(v[c], s);
+    }
+}
+
+// Rows too long for the register-resident form: two passes over global memory
+// (the second one hits L2).
+template <int MODE>
+__global__ __launch_bounds__(256) void quant_rows_loop_kernel(
+    const uint16_t* __restrict__ x, int64_t ldx, int K, uint8_t* __restrict__ xq,
+    float* __restrict__ scale) {
+    __shared__ uint32_t smem[256 / kWave];
+    const int64_t row = blockIdx.x;
+    const uint16_t* xr = x + row * ldx;
+    uint32_t m = 0;
+    for (int k = threadIdx.x * 8; k < K; k += 256 * 8)
+        m = absmax8(*reinterpret_cast<const uint4*>(xr + k), m);
+    m = block_max_u32<256>(m, smem);
+    const float s = scale_from_amax_bits<MODE>(m);
+    if (threadIdx.x == 0) scale[row] = s;
+    uint8_t* qr = xq + row * (int64_t)K;
+    for (int k = threadIdx.x * 8; k < K; k += 256 * 8)
+        *reinterpret_cast<uint2*>(qr + k) = encode8<MODE>(*reinterpret_cast<const uint4*>(xr + k), s);
+}
+
+// Static per-tensor quantizer: clamp(fp32(x)/s, +-448) -> e4m3fn.  torch.clamp
+// lets NaN through, and so do fminf/fmaxf here only if ordered the other way,
+// hence the explicit NaN test.
+__global__ __launch_bounds__(256) void quant_static_kernel(
+    const uint16_t* __restrict__ x, int64_t ldx, int64_t M, int K,
+    const float* __restrict__ input_scale, uint8_t* __restrict__ xq) {
+    const float s = *input_scale;
+    const int64_t chunks_per_row = K / 8;
+    const int64_t total = M * chunks_per_row;
+    for (int64_t i = blockIdx.x * 256 + threadIdx.x; i < total; i += (int64_t)gridDim.x * 256) {
+        const int64_t row = i / chunks_per_row;
+        const int k = (int)(i % chunks_per_row) * 8;
+        const uint4 q = *reinterpret_cast<const uint4*>(x + row * ldx + k);
+        const uint32_t w[4] = {q.x, q.y, q.z, q.w};
+        uint32_t c[4];
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+            float a = bf16_bits_to_f32(w[j] & 0xFFFFu) / s;
+            float b = bf16_bits_to_f32(w[j] >> 16) / s;
+            a = (a != a) ? a : fminf(fmaxf(a, -kFp8Max), kFp8Max);
+            b = (b != b) ? b : fminf(fmaxf(b, -kFp8Max), kFp8Max);
+            c[j] = e4m3_pack2(a, b);
+        }
+        *reinterpret_cast<uint2*>(xq + row * (int64_t)K + k) =
+            make_uint2(c[0] | (c[1] << 16), c[2] | (c[3] << 16));
+    }
+}
+
+__global__ __launch_bounds__(256) void debug_cast_kernel(const float* __restrict__ v, int64_t n,
+                                                         uint8_t* __restrict__ codes) {
+    for (int64_t i = blockIdx.x * 256 + threadIdx.x; i < n; i += (int64_t)gridDim.x * 256)
+        codes[i] = (uint8_t)(e4m3_pack2(v[i], 0.0f) & 0xFFu);
+}
+
+template <int MODE>
+static int launch_quant_rows(const void* x, int64_t M, int64_t K, int64_t ld, void* xq,
+                             float* scale, hipStream_t st) {
+    if (M == 0) return 0;
+    const uint16_t* xp = static_cast<const uint16_t*>(x);
+    uint8_t* qp = static_cast<uint8_t*>(xq);
+    const dim3 grid((unsigned)M);
+    const int k = (int)K;
+#define PHYAI_QL(T, C) \
+    hipLaunchKernelGGL((quant_rows_reg_kernel<T, C, MODE>), grid, dim3(T), 0, st, xp, ld, k, qp, scale)
+    if (K <= 512) PHYAI_QL(64, 1);
+    else if (K <= 1024) PHYAI_QL(128, 1);
+    else if (K <= 2048) PHYAI_QL(256, 1);
+    else if (K <= 4096) PHYAI_QL(256, 2);
+    else if (K <= 8192) PHYAI_QL(256, 4);
+    else if (K <= 16384) PHYAI_QL(256, 8);
+    else if (K <= 32768) PHYAI_QL(256, 16);
+    else hipLaunchKernelGGL((quant_rows_loop_kernel<MODE>), grid, dim3(256), 0, st, xp, ld, k, qp, scale);
+#undef PHYAI_QL
+    return 0;
+}
+
+int launch_quant_rowwise(const void* x, int64_t M, int64_t K, int64_t ldx, void* xq, float* xs,
+                         hipStream_t st) {
+    return launch_quant_rows<QUANT_ACT_DYNAMIC>(x, M, K, ldx, xq, xs, st);
+}
+int launch_weight_quant(const void* w, int64_t N, int64_t K, int64_t ldw, void* wq, float* ws,
+                        hipStream_t st) {
+    return launch_quant_rows<QUANT_WEIGHT>(w, N, K, ldw, wq, ws, st);
+}
+int launch_quant_static(const void* x, int64_t M, int64_t K, int64_t ldx, const float* input_scale,
+                        void* xq, hipStream_t st) {
+    if (M == 0) return 0;
+    int64_t total = M * (K / 8);
+    int blocks = (int)((total + 255) / 256);
+    if (blocks > 4096) blocks = 4096;
+    hipLaunchKernelGGL(quant_static_kernel, dim3(blocks), dim3(256), 0, st,
+                       static_cast<const uint16_t*>(x), ldx, M, (int)K, input_scale,
+                       static_cast<uint8_t*>(xq));
+    return 0;
+}
+int launch_debug_cast(const float* v, int64_t n, void* codes, hipStream_t st) {
+    if (n == 0) return 0;
+    int blocks = (int)((n + 255) / 256);
+    if (blocks > 8192) blocks = 8192;
+    hipLaunchKernelGGL(debug_cast_kernel, dim3(blocks), dim3(256), 0, st, v, n,
+                       static_cast<uint8_t*>(codes));
+    return 0;
+}
+
+}  // namespace phyai

@@ -1,0 +1,289 @@
+"""Flat tensor ops over the HIP kernels, in the reference kernel package's style:
+plain functions over device tensors with keyword-only optional pre-allocated
+outputs, inputs flattened to 2-D, ``RuntimeError("phyai_amd.ops.<op>: ...")`` on
+bad arguments, and an empty-input fast path (compare
+``phyai-kernel/phyai_kernel/triton/ada_rms_norm.py:196-221,267-288`` and
+``rms_norm.py:348-353`` in the reference).
+
+The ops enqueue on the current torch stream and never synchronise, so they can
+be recorded into a HIP graph once their workspace exists (see
+:func:`reserve_workspace`).
+"""
+
+from __future__ import annotations
+
+import torch
+
+from phyai_amd import _lib
+
+EPI_NONE = 0
+EPI_GEGLU_TANH = 1
+EPI_GEGLU_ERF = 2
+EPI_SWIGLU = 3
+EPI_GELU_TANH = 4
+EPI_GELU_ERF = 5
+_GATED = (EPI_GEGLU_TANH, EPI_GEGLU_ERF, EPI_SWIGLU)
+EPILOGUES = {
+    None: EPI_NONE, "none": EPI_NONE,
+    "geglu_tanh": EPI_GEGLU_TANH, "geglu_erf": EPI_GEGLU_ERF, "swiglu": EPI_SWIGLU,
+    "gelu_tanh": EPI_GELU_TANH, "gelu": EPI_GELU_ERF, "gelu_erf": EPI_GELU_ERF,
+}
+
+WORKSPACE_HEADER_BYTES = 16384
+
+
+def _err(op: str, msg: str) -> RuntimeError:
+    return RuntimeError(f"phyai_amd.ops.{op}: {msg}")
+
+
+def _stream_ptr() -> int:
+    return torch.cuda.current_stream().cuda_stream
+
+
+def _epi(op: str, epilogue) -> int:
+    if isinstance(epilogue, int) and not isinstance(epilogue, bool):
+        if epilogue not in range(6):
+            raise _err(op, f"unknown epilogue {epilogue!r}")
+        return epilogue
+    try:
+        return EPILOGUES[epilogue]
+    except KeyError:
+        raise _err(op, f"unknown epilogue {epilogue!r}; expected one of {sorted(k for k in EPILOGUES if k)}") from None
+
+
+def _as_rows(op: str, x: torch.Tensor, name: str, dtype: torch.dtype) -> torch.Tensor:
+    if not isinstance(x, torch.Tensor):
+        raise _err(op, f"{name} must be a Tensor, got {type(x)!r}")
+    if not x.is_cuda:
+        raise _err(op, f"{name} must live on the GPU, got device={x.device}")
+    if x.dtype != dtype:
+        raise _err(op, f"{name} must be {dtype}, got {x.dtype}")
+    if x.dim() < 1:
+        raise _err(op, f"{name} must have at least one dim")
+    x2 = x.reshape(-1, x.shape[-1])
+    if x2.stride(-1) != 1 or (x2.shape[0] > 1 and x2.stride(0) % 8 != 0) or x2.data_ptr() % 16 != 0:
+        x2 = x2.contiguous()
+    return x2
+
+
+# ---- workspace --------------------------------------------------------------
+# One zero-initialised scratch tensor per (device, stream), grown on demand
+# outside graph capture.  The kernels keep its header zero between calls.
+_workspaces: dict[tuple[int, int], torch.Tensor] = {}
+
+
+def workspace_bytes(M: int, N: int, K: int, epilogue=EPI_NONE) -> int:
+    return int(_lib.load().phyai_fp8_linear_workspace_bytes(M, N, K, _epi("workspace_bytes", epilogue)))
+
+
+def reserve_workspace(nbytes: int, device: torch.device | None = None) -> torch.Tensor:
+    """Make sure the current stream's workspace on ``device`` holds ``nbytes``."""
+    dev = torch.device("cuda", torch.cuda.current_device()) if device is None else torch.device(device)
+    idx = dev.index if dev.index is not None else torch.cuda.current_device()
+    key = (idx, _stream_ptr())
+    ws = _workspaces.get(key)
+    if ws is None or ws.numel() < nbytes:
+        if torch.cuda.is_current_stream_capturing():
+            raise _err(
+                "reserve_workspace",
+                f"workspace of {nbytes} bytes needed while a graph is being captured; "
+                "run the op once (or call reserve_workspace) before capture",
+            )
+        size = max(int(nbytes), 1 << 20)
+        size = (size + 0xFFFFF) & ~0xFFFFF
+        ws = torch.zeros(size, dtype=torch.uint8, device=torch.device("cuda", idx))
+        _workspaces[key] = ws
+    return ws
+
+
+def _workspace_for(M: int, N: int, K: int, epi: int, device: torch.device) -> torch.Tensor:
+    return reserve_workspace(workspace_bytes(M, N, K, epi), device)
+
+
+# ---- quantizers ---------------------------------------------------------------
+
+def fp8_quant_rowwise(x: torch.Tensor, *, out: torch.Tensor | None = None,
+                      scale_out: torch.Tensor | None = None) -> tuple[torch.Tensor, torch.Tensor]:
+    """Per-token dynamic e4m3fn quantization of bf16 ``x[..., K]``.
+
+    Returns ``(codes[..., K] float8_e4m3fn, scale[..., 1] float32)``, bit-exact
+    with ``Fp8Spec.quantize_activation`` (reference ``layers/quant/fp8.py:150-155``).
+    """
+    op = "fp8_quant_rowwise"
+    x2 = _as_rows(op, x, "x", torch.bfloat16)
+    M, K = x2.shape
+    if K % 8 != 0:
+        raise _err(op, f"last dim {K} must be a multiple of 8")
+    if out is None:
+        out = torch.empty(x.shape, dtype=torch.float8_e4m3fn, device=x.device)
+    elif out.shape != x.shape or out.dtype != torch.float8_e4m3fn or not out.is_contiguous():
+        raise _err(op, "out must be a contiguous float8_e4m3fn tensor shaped like x")
+    sshape = (*x.shape[:-1], 1)
+    if scale_out is None:
+        scale_out = torch.empty(sshape, dtype=torch.float32, device=x.device)
+    elif scale_out.shape != sshape or scale_out.dtype != torch.float32 or not scale_out.is_contiguous():
+        raise _err(op, f"scale_out must be a contiguous float32 tensor of shape {sshape}")
+    if M == 0:
+        return out, scale_out
+    rc = _lib.load().phyai_fp8_quant_rowwise(x2.data_ptr(), M, K, x2.stride(0) if M > 1 else K,
+                                              out.data_ptr(), scale_out.data_ptr(), _stream_ptr())
+    _lib.check(rc, op)
+    return out, scale_out
+
+
+def fp8_quant_static(x: torch.Tensor, input_scale: torch.Tensor, *,
+                     out: torch.Tensor | None = None) -> torch.Tensor:
+    """Static per-tensor quantization (reference ``layers/quant/fp8.py:142-148``)."""
+    op = "fp8_quant_static"
+    x2 = _as_rows(op, x, "x", torch.bfloat16)
+    M, K = x2.shape
+    if K % 8 != 0:
+        raise _err(op, f"last dim {K} must be a multiple of 8")
+    if not (isinstance(input_scale, torch.Tensor) and input_scale.is_cuda and input_scale.dtype == torch.float32
+            and input_scale.numel() == 1):
+        raise _err(op, "input_scale must be a one-element float32 GPU tensor")
+    if out is None:
+        out = torch.empty(x.shape, dtype=torch.float8_e4m3fn, device=x.device)
+    elif out.shape != x.shape or out.dtype != torch.float8_e4m3fn or not out.is_contiguous():
+        raise _err(op, "out must be a contiguous float8_e4m3fn tensor shaped like x")
+    if M == 0:
+        return out
+    rc = _lib.load().phyai_fp8_quant_static(x2.data_ptr(), M, K, x2.stride(0) if M > 1 else K,
+                                             input_scale.data_ptr(), out.data_ptr(), _stream_ptr())
+    _lib.check(rc, op)
+    return out
+
+
+def fp8_weight_quant(w: torch.Tensor, *, out: torch.Tensor | None = None,
+                     scale_out: torch.Tensor | None = None) -> tuple[torch.Tensor, torch.Tensor]:
+    """Offline per-output-channel weight quantization: ``(codes [N,K], scale [N])``."""
+    op = "fp8_weight_quant"
+    if w.dim() != 2:
+        raise _err(op, f"w must be 2-D (N, K), got shape {tuple(w.shape)}")
+    w2 = _as_rows(op, w, "w", torch.bfloat16)
+    N, K = w2.shape
+    if K % 8 != 0:
+        raise _err(op, f"K={K} must be a multiple of 8")
+    if out is None:
+        out = torch.empty((N, K), dtype=torch.float8_e4m3fn, device=w.device)
+    if scale_out is None:
+        scale_out = torch.empty((N,), dtype=torch.float32, device=w.device)
+    if N == 0:
+        return out, scale_out
+    rc = _lib.load().phyai_fp8_weight_quant_rowwise(w2.data_ptr(), N, K, w2.stride(0) if N > 1 else K,
+                                                     out.data_ptr(), scale_out.data_ptr(), _stream_ptr())
+    _lib.check(rc, op)
+    return out, scale_out
+
+
+# ---- GEMM / linear --------------------------------------------------------------
+
+def _check_weight(op: str, weight: torch.Tensor, weight_scale: torch.Tensor, K: int) -> tuple[int, int]:
+    if not (isinstance(weight, torch.Tensor) and weight.is_cuda and weight.dim() == 2):
+        raise _err(op, "weight must be a 2-D GPU tensor (N, K)")
+    if weight.dtype not in (torch.float8_e4m3fn, torch.uint8):
+        raise _err(op, f"weight must be float8_e4m3fn, got {weight.dtype}")
+    if not weight.is_contiguous():
+        raise _err(op, "weight must be contiguous (N, K) with K innermost")
+    N, Kw = weight.shape
+    if Kw != K:
+        raise _err(op, f"weight K={Kw} does not match activation K={K}")
+    if K % 16 != 0 or N % 16 != 0:
+        raise _err(op, f"K={K} and N={N} must be multiples of 16")
+    if not (weight_scale.is_cuda and weight_scale.dtype == torch.float32 and weight_scale.numel() == N
+            and weight_scale.is_contiguous()):
+        raise _err(op, f"weight_scale must be a contiguous float32 GPU tensor with {N} elements")
+    return N, K
+
+
+def _check_bias(op: str, bias: torch.Tensor | None, N: int) -> int:
+    if bias is None:
+        return 0
+    if not (bias.is_cuda and bias.dtype == torch.bfloat16 and bias.numel() == N and bias.is_contiguous()):
+        raise _err(op, f"bias must be a contiguous bfloat16 GPU tensor with {N} elements")
+    return bias.data_ptr()
+
+
+def _out_for(op: str, lead: tuple[int, ...], n_out: int, out: torch.Tensor | None, device) -> torch.Tensor:
+    shape = (*lead, n_out)
+    if out is None:
+        return torch.empty(shape, dtype=torch.bfloat16, device=device)
+    if tuple(out.shape) != shape or out.dtype != torch.bfloat16 or not out.is_contiguous():
+        raise _err(op, f"out must be a contiguous bfloat16 tensor of shape {shape}")
+    return out
+
+
+def fp8_gemm(xq: torch.Tensor, x_scale: torch.Tensor, weight: torch.Tensor, weight_scale: torch.Tensor,
+             bias: torch.Tensor | None = None, *, epilogue=None, out: torch.Tensor | None = None) -> torch.Tensor:
+    """``bf16(act((xq @ weight.T) * x_scale * weight_scale + bias))`` on quantized inputs.
+
+    ``x_scale`` has one element per token row, or a single element (static
+    per-tensor scale).  Replaces the ``torch._scaled_mm`` call at reference
+    ``layers/linear/backends/torch.py:166-175`` (and ``:145-152``).
+    """
+    op = "fp8_gemm"
+    epi = _epi(op, epilogue)
+    if not (isinstance(xq, torch.Tensor) and xq.is_cuda and xq.dtype in (torch.float8_e4m3fn, torch.uint8)):
+        raise _err(op, "xq must be a float8_e4m3fn GPU tensor")
+    x2 = xq.reshape(-1, xq.shape[-1])
+    if not x2.is_contiguous():
+        x2 = x2.contiguous()
+    M, K = x2.shape
+    N, _ = _check_weight(op, weight, weight_scale, K)
+    if epi in _GATED and N % 32 != 0:
+        raise _err(op, f"gated epilogue needs N % 32 == 0, got {N}")
+    xs = x_scale.reshape(-1)
+    if not (xs.is_cuda and xs.dtype == torch.float32 and xs.numel() in (1, M) and xs.is_contiguous()):
+        raise _err(op, f"x_scale must be float32 with 1 or {M} elements")
+    scalar = 1 if (xs.numel() == 1 and M != 1) else 0
+    bias_ptr = _check_bias(op, bias, N)
+    n_out = N // 2 if epi in _GATED else N
+    out = _out_for(op, tuple(xq.shape[:-1]), n_out, out, xq.device)
+    if M == 0:
+        return out
+    ws = _workspace_for(M, N, K, epi, xq.device)
+    rc = _lib.load().phyai_fp8_gemm(x2.data_ptr(), xs.data_ptr(), scalar, weight.data_ptr(),
+                                     weight_scale.data_ptr(), bias_ptr, out.data_ptr(), n_out, M, N, K, epi,
+                                     ws.data_ptr(), ws.numel(), _stream_ptr())
+    _lib.check(rc, op)
+    return out
+
+
+def fp8_linear(x: torch.Tensor, weight: torch.Tensor, weight_scale: torch.Tensor,
+               bias: torch.Tensor | None = None, *, epilogue=None, out: torch.Tensor | None = None) -> torch.Tensor:
+    """The whole W8A8 linear on bf16 ``x[..., K]``: per-token quantization, fp8 MFMA
+    GEMM, per-channel dequantization, bias and optional activation, bf16 out.
+
+    Replaces ``TorchKernel._fp8_per_channel`` (reference
+    ``layers/linear/backends/torch.py:155-176``) and, with a gated ``epilogue``,
+    the activation launch that follows it in ``DenseMLP.forward``
+    (``layers/mlp/dense_mlp.py:256-261``).
+    """
+    op = "fp8_linear"
+    epi = _epi(op, epilogue)
+    x2 = _as_rows(op, x, "x", torch.bfloat16)
+    M, K = x2.shape
+    N, _ = _check_weight(op, weight, weight_scale, K)
+    if epi in _GATED and N % 32 != 0:
+        raise _err(op, f"gated epilogue needs N % 32 == 0, got {N}")
+    bias_ptr = _check_bias(op, bias, N)
+    n_out = N // 2 if epi in _GATED else N
+    out = _out_for(op, tuple(x.shape[:-1]), n_out, out, x.device)
+    if M == 0:
+        return out
+    ws = _workspace_for(M, N, K, epi, x.device)
+    rc = _lib.load().phyai_fp8_linear(x2.data_ptr(), x2.stride(0) if M > 1 else K, weight.data_ptr(),
+                                       weight_scale.data_ptr(), bias_ptr, out.data_ptr(), n_out, M, N, K, epi,
+                                       ws.data_ptr(), ws.numel(), _stream_ptr())
+    _lib.check(rc, op)
+    return out
+
+
+def debug_cast_e4m3(v: torch.Tensor) -> torch.Tensor:
+    """Device fp32 -> e4m3fn cast used by the quantizers, exposed for exhaustive tests."""
+    if not (v.is_cuda and v.dtype == torch.float32 and v.is_contiguous()):
+        raise _err("debug_cast_e4m3", "v must be a contiguous float32 GPU tensor")
+    out = torch.empty(v.shape, dtype=torch.uint8, device=v.device)
+    rc = _lib.load().phyai_fp8_debug_cast_e4m3(v.data_ptr(), v.numel(), out.data_ptr(), _stream_ptr())
+    _lib.check(rc, "debug_cast_e4m3")
+    return out

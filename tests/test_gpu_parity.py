@@ -1,0 +1,325 @@
+"""GPU parity: the HIP kernels, called through the C ABI, against the CPU oracle.
+
+Quantizer codes and scales must be bit-exact.  GEMM outputs must satisfy
+max|out - ref| <= 1e-2 * max|ref| and cosine >= 0.9999 against the fp32
+dequantized matmul (the tolerance the benchmark definition states); cases whose
+sums are exact in fp32 must be bit-exact.
+"""
+
+from __future__ import annotations
+
+import numpy as np
+import pytest
+import torch
+
+from conftest import seeded
+from oracle import cport, ref
+
+pytestmark = pytest.mark.gpu
+
+TOL_MAXABS = 1e-2
+TOL_COS = 0.9999
+
+
+def _ops():
+    from phyai_amd import ops
+    return ops
+
+
+def _bits(t: torch.Tensor) -> np.ndarray:
+    return t.detach().cpu().contiguous().view(torch.uint16).numpy()
+
+
+def _codes(t: torch.Tensor) -> np.ndarray:
+    return t.detach().cpu().contiguous().view(torch.uint8).numpy()
+
+
+def assert_close_to_ref(out: torch.Tensor, ref_f32: torch.Tensor, what=""):
+    o = out.detach().float().cpu().reshape(-1).double()
+    r = ref_f32.detach().float().cpu().reshape(-1).double()
+    assert torch.isfinite(o).all(), f"{what}: non-finite output"
+    scale = r.abs().max().item()
+    err = (o - r).abs().max().item()
+    cos = (o @ r / (o.norm() * r.norm()).clamp_min(1e-30)).item() if scale > 0 else 1.0
+    assert err <= TOL_MAXABS * scale + 1e-30, f"{what}: max abs err {err:.4g} > 1e-2*{scale:.4g}"
+    assert cos >= TOL_COS, f"{what}: cosine {cos:.6f} < {TOL_COS}"
+
+
+# ---------------------------------------------------------------------------
+# device cast
+# ---------------------------------------------------------------------------
+
+def test_device_cast_matches_oracle_dense_sweep(dev):
+    """Every fp32 pattern on a 2^-12-relative grid below 512 (both signs, several
+    sub-grid tails incl. exact ties) through the device cast vs the C oracle."""
+    ops = _ops()
+    hi = (np.arange(0, 0x44000000 >> 12, dtype=np.uint32) << 12)
+    for tail in (0, 1, 0x7FF, 0x800, 0x801, 0xFFF):
+        for sgn in (0, 0x80000000):
+            b = (hi | np.uint32(tail) | np.uint32(sgn)).astype(np.uint32)
+            v = b.view(np.float32)
+            want = cport.f32_to_e4m3(v)
+            got = ops.debug_cast_e4m3(torch.from_numpy(v.copy()).to(dev)).cpu().numpy()
+            bad = np.nonzero(got != want)[0]
+            assert bad.size == 0, (
+                f"tail={tail:#x} sign={sgn:#x}: {bad.size} mismatches, first at bits "
+                f"{b[bad[0]]:#010x} ({v[bad[0]]!r}): device {got[bad[0]]:#04x} oracle {want[bad[0]]:#04x}")
+
+
+def test_device_cast_special_values(dev):
+    ops = _ops()
+    v = np.array([0.0, -0.0, 448.0, -448.0, 463.9, 464.0, 465.0, 479.9, 480.0, 1e9, -1e9,
+                  np.inf, -np.inf, 2.0 ** -9, 2.0 ** -10, 1.5 * 2.0 ** -10, 2.0 ** -6, 1e-30], np.float32)
+    want = cport.f32_to_e4m3(v)
+    got = ops.debug_cast_e4m3(torch.from_numpy(v).to(dev)).cpu().numpy()
+    assert (got == want).all(), list(zip(v.tolist(), got.tolist(), want.tolist()))
+    nan = ops.debug_cast_e4m3(torch.tensor([float("nan")], device=dev)).cpu().numpy()
+    assert (nan & 0x7F) == 0x7F
+
+
+# ---------------------------------------------------------------------------
+# quantizer
+# ---------------------------------------------------------------------------
+
+QUANT_SHAPES = [(1, 16), (3, 8), (8, 64), (50, 1024), (50, 2048), (50, 4096), (7, 520), (33, 1000),
+                (5, 8192), (3, 16384), (2, 32768), (2, 40000), (816, 2048)]
+
+
+@pytest.mark.parametrize("M,K", QUANT_SHAPES)
+def test_quant_rowwise_bit_exact(dev, M, K):
+    ops = _ops()
+    x = seeded((M, K), seed=100 + M + K)
+    q, s = ops.fp8_quant_rowwise(x.to(dev))
+    wq, ws = cport.quant_rowwise(_bits(x))
+    assert q.shape == (M, K) and s.shape == (M, 1) and s.dtype == torch.float32
+    np.testing.assert_array_equal(s.cpu().numpy().reshape(-1).view(np.uint32), ws.view(np.uint32))
+    np.testing.assert_array_equal(_codes(q), wq)
+    tq, ts = ref.quant_rowwise(x)
+    np.testing.assert_array_equal(_codes(q), _codes(tq))
+    assert torch.equal(s.cpu(), ts)
+
+
+def test_quant_rowwise_edge_rows(dev):
+    """All-zero row, +-0, subnormal bf16, power-of-two amax, bf16 max, an outlier row."""
+    ops = _ops()
+    K = 256
+    x = seeded((8, K), seed=7)
+    x[0] = 0
+    x[1] = 0; x[1, 0] = -0.0; x[1, 5] = 1e-38
+    x[2] = torch.full((K,), 9.2e-41).bfloat16(); x[2, 3] = -9.2e-41
+    x[3, 17] = 64.0; x[3] = x[3].clamp(-64, 64)
+    x[4, 0] = torch.finfo(torch.bfloat16).max
+    x[5, 100] = 2000.0
+    x[6] = x[6] * 1e-20
+    x[7] = -x[7].abs()
+    q, s = ops.fp8_quant_rowwise(x.to(dev))
+    wq, ws = cport.quant_rowwise(_bits(x))
+    np.testing.assert_array_equal(s.cpu().numpy().reshape(-1).view(np.uint32), ws.view(np.uint32))
+    np.testing.assert_array_equal(_codes(q), wq)
+    tq, ts = ref.quant_rowwise(x)
+    np.testing.assert_array_equal(_codes(q), _codes(tq))
+
+
+def test_quant_rowwise_all_bf16_values(dev):
+    """Every finite bf16 bit pattern as x, against a sweep of row maxima."""
+    ops = _ops()
+    allbits = np.arange(0, 1 << 16, dtype=np.uint16)
+    finite = allbits[(allbits & 0x7F80) != 0x7F80]
+    K = 65536
+    rows = []
+    for amax in (1.0, 3.140625, 448.0, 0.0078125, 1e-20, 3e38, 17.5, 2.0 ** -100):
+        row = np.zeros(K, np.uint16)
+        vals = torch.from_numpy(finite.copy()).view(torch.bfloat16).float()
+        keep = finite[(vals.abs() <= amax).numpy()]
+        row[: keep.size] = keep
+        row[-1] = torch.tensor([amax]).bfloat16().view(torch.uint16).item()
+        rows.append(row)
+    xb = np.stack(rows)
+    x = torch.from_numpy(xb).view(torch.bfloat16)
+    q, s = ops.fp8_quant_rowwise(x.to(dev))
+    wq, ws = cport.quant_rowwise(xb)
+    np.testing.assert_array_equal(s.cpu().numpy().reshape(-1).view(np.uint32), ws.view(np.uint32))
+    np.testing.assert_array_equal(_codes(q), wq)
+
+
+def test_quant_rowwise_strided_and_batched(dev):
+    ops = _ops()
+    x = seeded((4, 6, 128), seed=3).to(dev)
+    q, s = ops.fp8_quant_rowwise(x)
+    assert q.shape == (4, 6, 128) and s.shape == (4, 6, 1)
+    tq, ts = ref.quant_rowwise(x.cpu())
+    np.testing.assert_array_equal(_codes(q), _codes(tq))
+    big = seeded((10, 512), seed=4).to(dev)
+    view = big[:, 128:384]
+    q2, s2 = ops.fp8_quant_rowwise(view)
+    tq2, ts2 = ref.quant_rowwise(view.cpu())
+    np.testing.assert_array_equal(_codes(q2), _codes(tq2))
+    assert torch.equal(s2.cpu(), ts2)
+
+
+def test_quant_rowwise_empty(dev):
+    ops = _ops()
+    q, s = ops.fp8_quant_rowwise(torch.empty((0, 64), dtype=torch.bfloat16, device=dev))
+    assert q.shape == (0, 64) and s.shape == (0, 1)
+
+
+def test_quant_static_bit_exact(dev):
+    ops = _ops()
+    x = seeded((33, 256), seed=11, scale=3.0)
+    for sc in (1.0, 0.01, 0.37):
+        scale = torch.tensor([sc], dtype=torch.float32)
+        q = ops.fp8_quant_static(x.to(dev), scale.to(dev))
+        np.testing.assert_array_equal(_codes(q), _codes(ref.quant_static(x, scale)))
+        np.testing.assert_array_equal(_codes(q), cport.quant_static(_bits(x), sc))
+
+
+@pytest.mark.parametrize("N,K", [(64, 128), (256, 1024), (100, 72)])
+def test_weight_quant_bit_exact(dev, N, K):
+    ops = _ops()
+    w = seeded((N, K), seed=N + K, scale=0.02)
+    w[1] = 0
+    q, s = ops.fp8_weight_quant(w.to(dev))
+    wq, ws = cport.weight_quant(_bits(w))
+    np.testing.assert_array_equal(s.cpu().numpy().view(np.uint32), ws.view(np.uint32))
+    np.testing.assert_array_equal(_codes(q), wq)
+    tq, ts = ref.weight_quant(w)
+    np.testing.assert_array_equal(_codes(q), _codes(tq))
+    assert torch.equal(s.cpu(), ts)
+
+
+# ---------------------------------------------------------------------------
+# GEMM
+# ---------------------------------------------------------------------------
+
+def _problem(M, N, K, seed, bias=True):
+    x = seeded((M, K), seed=seed)
+    w = seeded((N, K), seed=seed + 1, scale=0.02)
+    b = seeded((N,), seed=seed + 2, scale=0.01) if bias else None
+    wq, ws = ref.weight_quant(w)
+    return x, wq, ws, b
+
+
+def test_gemm_exact_integer_layout(dev):
+    """Small-integer codes and power-of-two scales: every product and partial sum
+    is exact in fp32, so any accumulation order gives the same bits.  A wrong
+    lane/row mapping, a dropped K slab or a transposed operand changes the result."""
+    ops = _ops()
+    g = torch.Generator().manual_seed(5)
+    for (M, N, K) in [(64, 64, 128), (50, 96, 256), (128, 256, 384), (200, 144, 1040), (33, 2560, 1024)]:
+        xi = torch.randint(-4, 5, (M, K), generator=g).float()
+        wi = torch.randint(-4, 5, (N, K), generator=g).float()
+        xq = xi.to(torch.float8_e4m3fn)
+        wq = wi.to(torch.float8_e4m3fn)
+        xs = torch.full((M, 1), 0.5)
+        ws = torch.full((N,), 0.25)
+        want = ((xi @ wi.t()) * 0.125).bfloat16()
+        got = ops.fp8_gemm(xq.to(dev), xs.to(dev), wq.to(dev), ws.to(dev))
+        assert torch.equal(got.cpu(), want), f"{(M, N, K)}: {(got.cpu().float() - want.float()).abs().max()}"
+
+
+def test_gemm_row_col_identity(dev):
+    """x = one-hot rows, w = distinct per-row values: out[m, n] must be w[n, k(m)]."""
+    ops = _ops()
+    M, N, K = 64, 128, 128
+    xq = torch.zeros(M, K)
+    for m in range(M):
+        xq[m, (m * 7) % K] = 1.0
+    w = ((torch.arange(N)[:, None] * 3 + torch.arange(K)[None, :]) % 15 - 7).float()
+    got = ops.fp8_gemm(xq.to(torch.float8_e4m3fn).to(dev), torch.ones(M, 1, device=dev),
+                       w.to(torch.float8_e4m3fn).to(dev), torch.ones(N, device=dev))
+    want = (xq @ w.t()).bfloat16()
+    assert torch.equal(got.cpu(), want)
+
+
+GEMM_SHAPES = [
+    (50, 4096, 1024),    # config 1
+    (50, 2560, 1024), (50, 1024, 2048), (50, 1024, 4096),   # expert qkv / o / down
+    (1, 256, 1024), (7, 48, 80), (64, 64, 128), (65, 80, 144), (130, 272, 528),
+    (816, 2048, 2048), (300, 1024, 4096),
+]
+
+
+@pytest.mark.parametrize("M,N,K", GEMM_SHAPES)
+def test_linear_matches_oracle(dev, M, N, K):
+    ops = _ops()
+    x, wq, ws, b = _problem(M, N, K, seed=M + N + K)
+    got = ops.fp8_linear(x.to(dev), wq.to(dev), ws.to(dev), b.to(dev))
+    xq, xs = ref.quant_rowwise(x)
+    want_f32 = ref.gemm_f32(xq, xs, wq, ws, b)
+    assert got.shape == (M, N) and got.dtype == torch.bfloat16
+    assert_close_to_ref(got, want_f32, f"linear {M}x{N}x{K}")
+    # much tighter than the stated tolerance: bf16 rounding noise only
+    rel = (got.cpu().float() - want_f32).norm() / want_f32.norm()
+    assert rel < 4e-3, f"relative Frobenius error {rel:.3g}"
+
+
+@pytest.mark.parametrize("M,N,K", [(50, 512, 256), (9, 64, 128)])
+def test_linear_matches_c_oracle_small(dev, M, N, K):
+    ops = _ops()
+    x, wq, ws, b = _problem(M, N, K, seed=1)
+    got = ops.fp8_linear(x.to(dev), wq.to(dev), ws.to(dev), b.to(dev))
+    q, s = cport.quant_rowwise(_bits(x))
+    _, f32 = cport.linear(q, s, _codes(wq), ws.numpy(), _bits(b), 0, want_f32=True)
+    assert_close_to_ref(got, torch.from_numpy(f32), "c-oracle")
+
+
+@pytest.mark.parametrize("epi_name,epi", [("geglu_tanh", 1), ("geglu_erf", 2), ("swiglu", 3),
+                                          ("gelu_tanh", 4), ("gelu", 5)])
+@pytest.mark.parametrize("M,N,K", [(50, 8192, 1024), (70, 192, 272), (816, 1024, 512)])
+def test_linear_epilogues(dev, epi_name, epi, M, N, K):
+    ops = _ops()
+    x, wq, ws, b = _problem(M, N, K, seed=epi * 1000 + M)
+    got = ops.fp8_linear(x.to(dev), wq.to(dev), ws.to(dev), b.to(dev), epilogue=epi_name)
+    xq, xs = ref.quant_rowwise(x)
+    y = ref.gemm_f32(xq, xs, wq, ws, b)
+    want = ref.epilogue(y, epi).float()
+    n_out = N // 2 if epi in ref.GATED else N
+    assert got.shape == (M, n_out)
+    assert_close_to_ref(got, want, f"{epi_name} {M}x{N}x{K}")
+
+
+def test_linear_no_bias_and_batched(dev):
+    ops = _ops()
+    x = seeded((2, 25, 1024), seed=9)
+    w = seeded((2560, 1024), seed=10, scale=0.02)
+    wq, ws = ref.weight_quant(w)
+    got = ops.fp8_linear(x.to(dev), wq.to(dev), ws.to(dev))
+    assert got.shape == (2, 25, 2560)
+    xq, xs = ref.quant_rowwise(x)
+    assert_close_to_ref(got, ref.gemm_f32(xq, xs, wq, ws), "batched")
+
+
+def test_linear_zero_weight_gives_bias(dev):
+    """The reference's own exact case (tests/layers/linear/test_kernel_torch.py:199-215)."""
+    ops = _ops()
+    N, K = 32, 64
+    wq = torch.zeros(N, K, dtype=torch.float8_e4m3fn, device=dev)
+    ws = torch.ones(N, device=dev)
+    bias = torch.ones(N, dtype=torch.bfloat16, device=dev)
+    x = torch.zeros(4, K, dtype=torch.bfloat16, device=dev)
+    y = ops.fp8_linear(x, wq, ws, bias)
+    assert torch.equal(y, bias.expand(4, N))
+
+
+def test_gemm_scalar_x_scale(dev):
+    ops = _ops()
+    x, wq, ws, b = _problem(40, 128, 256, seed=21)
+    scale = torch.tensor([0.05])
+    xq = ref.quant_static(x, scale)
+    got = ops.fp8_gemm(xq.to(dev), scale.to(dev), wq.to(dev), ws.to(dev), b.to(dev))
+    want = ref.gemm_f32(xq, scale.expand(40, 1), wq, ws, b)
+    assert_close_to_ref(got, want, "per-tensor")
+
+
+def test_linear_repeatable_and_workspace_stays_clean(dev):
+    """Split-K path: same bits on every call (fixed reduction order) and the
+    counters in the workspace header return to zero."""
+    ops = _ops()
+    x, wq, ws, b = _problem(50, 1024, 4096, seed=33)
+    xd, wd, sd, bd = x.to(dev), wq.to(dev), ws.to(dev), b.to(dev)
+    first = ops.fp8_linear(xd, wd, sd, bd).clone()
+    for _ in range(5):
+        assert torch.equal(ops.fp8_linear(xd, wd, sd, bd), first)
+    torch.cuda.synchronize()
+    for w in ops._workspaces.values():
+        assert int(w[: ops.WORKSPACE_HEADER_BYTES].max().item()) == 0
