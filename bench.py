@@ -1,0 +1,249 @@
+#!/usr/bin/env python3
+"""Benchmark of the W8A8 fp8 linear hot path on one MI355X.
+
+Workload (the configuration the metric is quoted on): the Pi0.5 action-expert
+linear set.  18 layers x {qkv 1024->2560, o 2048->1024, gate_up 1024->8192 with
+fused GeGLU-tanh, down 4096->1024}, M = 50 action tokens, bf16 activations
+~N(0,1), fp8 e4m3fn weights ~N(0,0.02) with per-output-channel scales, every
+layer with its own weight tensors (311 MB of fp8 weights per denoise step), and
+10 flow-matching steps recorded in ONE hipGraph.  A bench "step" is one replay of
+that graph (what the engine launches per action chunk); `value` is the p50 time
+of one denoise step (replay time / 10) in microseconds.
+
+Printed JSON (one line):
+  value / ms_per_step  whole-path numbers (quantizer + GEMM + epilogue, graph replay)
+  roofline             the GEMM kernel alone: algorithmic bytes of one layer's four
+                       linears / their measured average launch durations (HIP events
+                       around graph replays that contain only those GEMM launches,
+                       distinct weights per launch so they stream from HBM)
+  cpu_baseline         torch CPU dequantize + matmul form of the same layer set on
+                       this box's host cores (a reported baseline, not the target)
+  extra                prefix-prefill set (M = 816) in TFLOP/s against dense fp8 peak
+
+Inputs are resident in HBM before the timed region starts.
+"""
+
+from __future__ import annotations
+
+import argparse
+import json
+import os
+import statistics
+import sys
+import time
+
+import torch
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+if ROOT not in sys.path:
+    sys.path.insert(0, ROOT)
+
+HBM_PEAK_GBS = 8000.0       # MI355X HBM3E
+FP8_PEAK_TFLOPS = 5000.0    # MI355X dense fp8 MFMA
+
+# (name, N, K, epilogue) per layer
+EXPERT_SET = [("qkv", 2560, 1024, None), ("o", 1024, 2048, None),
+              ("gate_up", 8192, 1024, "geglu_tanh"), ("down", 1024, 4096, None)]
+PREFILL_SET = [("qkv", 2560, 2048, None), ("o", 2048, 2048, None),
+               ("gate_up", 32768, 2048, "geglu_tanh"), ("down", 2048, 16384, None)]
+
+
+def algorithmic_bytes(M: int, N: int, K: int, epilogue, bias: bool = False) -> int:
+    """bf16 X in + fp8 W + fp32 weight scales (+ bf16 bias) + bf16 out (half width if gated)."""
+    n_out = N // 2 if epilogue in ("geglu_tanh", "geglu_erf", "swiglu") else N
+    return 2 * M * K + N * K + 4 * N + (2 * N if bias else 0) + 2 * M * n_out
+
+
+def make_layers(dev, shapes, M, n_layers, seed0=0):
+    """Seeded synthetic tensors, generated on the CPU and copied to the device so that
+    the CPU baseline sees the same bits.  Weights are quantized on the device by the
+    library's own weight quantizer (bit-exact with the oracle's)."""
+    from phyai_amd import ops
+
+    layers = []
+    seed = seed0
+    for li in range(n_layers):
+        layer = {}
+        for name, N, K, epi in shapes:
+            g = torch.Generator().manual_seed(seed)
+            seed += 1
+            w = (torch.randn(N, K, generator=g) * 0.02).to(torch.bfloat16)
+            x = torch.randn(M, K, generator=g).to(torch.bfloat16)
+            wq, ws = ops.fp8_weight_quant(w.to(dev))
+            n_out = N // 2 if epi else N
+            layer[name] = dict(w=wq, ws=ws, x=x.to(dev), epi=epi, N=N, K=K,
+                               out=torch.empty(M, n_out, dtype=torch.bfloat16, device=dev),
+                               w_bf16_cpu=w if li == 0 else None, x_cpu=x if li == 0 else None)
+        layers.append(layer)
+    return layers
+
+
+def run_layers(layers, shapes):
+    from phyai_amd import ops
+
+    for layer in layers:
+        for name, _, _, _ in shapes:
+            t = layer[name]
+            ops.fp8_linear(t["x"], t["w"], t["ws"], None, epilogue=t["epi"], out=t["out"])
+
+
+def time_replays(graph, n, warmup):
+    """HIP events around each replay, on the stream the replays are launched on."""
+    for _ in range(warmup):
+        graph.replay()
+    torch.cuda.synchronize()
+    evs = [(torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)) for _ in range(n)]
+    t0 = time.perf_counter()
+    for a, b in evs:
+        a.record()
+        graph.replay()
+        b.record()
+    torch.cuda.synchronize()
+    wall = time.perf_counter() - t0
+    return [a.elapsed_time(b) for a, b in evs], wall
+
+
+def gemm_only_times(dev, layers, shapes, M, reps=8, iters=30):
+    """Average launch duration of the GEMM kernel per shape: a graph holding only
+    pre-quantized GEMM launches (reps passes over the distinct per-layer weights)."""
+    from phyai_amd import ops
+    from phyai_amd.runtime import HipGraph
+
+    out = {}
+    for name, N, K, epi in shapes:
+        pre = []
+        for layer in layers:
+            t = layer[name]
+            xq, xs = ops.fp8_quant_rowwise(t["x"])
+            pre.append((xq, xs, t))
+
+        def fn():
+            for _ in range(reps):
+                for xq, xs, t in pre:
+                    ops.fp8_gemm(xq, xs, t["w"], t["ws"], None, epilogue=t["epi"], out=t["out"])
+
+        g = HipGraph()
+        g.capture(fn, {})
+        ts, _ = time_replays(g, iters, 3)
+        launches = reps * len(pre)
+        out[name] = statistics.median(ts) * 1e3 / launches  # us per launch
+    return out
+
+
+def cpu_baseline(layers, shapes, M, budget_s=12.0):
+    """torch CPU dequantize + matmul (+ quantizer, + GeGLU) on layer 0's tensors."""
+    from oracle import ref
+
+    items = []
+    for name, N, K, epi in shapes:
+        t = layers[0][name]
+        wq, ws = ref.weight_quant(t["w_bf16_cpu"])
+        items.append((t["x_cpu"], wq, ws, {None: 0, "geglu_tanh": 1}[epi]))
+
+    def layer_once():
+        for x, wq, ws, epi in items:
+            ref.linear(x, wq, ws, None, epi)
+
+    layer_once()
+    ts = []
+    t_end = time.perf_counter() + budget_s
+    while time.perf_counter() < t_end or len(ts) < 3:
+        t0 = time.perf_counter()
+        layer_once()
+        ts.append(time.perf_counter() - t0)
+    return statistics.median(ts), len(ts)
+
+
+def main() -> int:
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=200)
+    ap.add_argument("--warmup", type=int, default=20)
+    ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--no-prefill", action="store_true")
+    args = ap.parse_args()
+    if args.gpus != 1 or int(os.environ.get("WORLD_SIZE", "1")) != 1:
+        print("bench.py: this path is built and measured on ONE GPU (TP=1, no collectives); "
+              "run with --gpus 1", file=sys.stderr)
+        return 2
+    if not torch.cuda.is_available():
+        print("bench.py: no GPU visible", file=sys.stderr)
+        return 2
+
+    from phyai_amd.runtime import HipGraph
+
+    dev = torch.device("cuda", 0)
+    torch.cuda.set_device(dev)
+    M, n_layers, denoise_steps = 50, 18, 10
+
+    layers = make_layers(dev, EXPERT_SET, M, n_layers)
+
+    def chunk():
+        for _ in range(denoise_steps):
+            run_layers(layers, EXPERT_SET)
+
+    graph = HipGraph()
+    graph.capture(chunk, {})
+    torch.cuda.synchronize()
+    ts_ms, wall = time_replays(graph, args.steps, args.warmup)
+    ms_per_step = wall * 1e3 / args.steps
+    p50_replay_ms = statistics.median(ts_ms)
+    value_us = p50_replay_ms * 1e3 / denoise_steps
+
+    # ---- roofline of the dominant kernel (the small-M GEMM) --------------------
+    per_launch_us = gemm_only_times(dev, layers, EXPERT_SET, M)
+    layer_bytes = sum(algorithmic_bytes(M, N, K, epi) for _, N, K, epi in EXPERT_SET)
+    layer_us = sum(per_launch_us.values())
+    achieved = layer_bytes / (layer_us * 1e-6) / 1e9
+    roofline = {
+        "bound": "hbm", "achieved": round(achieved, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
+        "frac": round(achieved / HBM_PEAK_GBS, 4), "traffic": None,
+        "kernel": "gemm_fp8_tile_kernel (M=50, four expert shapes)",
+        "bytes_per_layer": layer_bytes,
+        "per_shape": {name: {"us": round(per_launch_us[name], 3),
+                             "GB/s": round(algorithmic_bytes(M, N, K, epi) / per_launch_us[name] / 1e3, 1)}
+                      for name, N, K, epi in EXPERT_SET},
+        "whole_path_frac": round(layer_bytes * n_layers / (value_us * 1e-6) / 1e9 / HBM_PEAK_GBS, 4),
+    }
+
+    # ---- prefix prefill (M = 816): MFMA-bound regime -----------------------------
+    extra = {}
+    if not args.no_prefill:
+        pl = make_layers(dev, PREFILL_SET, 816, 4, seed0=10_000)
+        pg = HipGraph()
+        pg.capture(lambda: run_layers(pl, PREFILL_SET), {})
+        pts, _ = time_replays(pg, 30, 3)
+        p_layer_us = statistics.median(pts) * 1e3 / len(pl)
+        flops = sum(2 * 816 * N * K for _, N, K, _ in PREFILL_SET)
+        extra["prefill_M816"] = {"us_per_layer": round(p_layer_us, 2),
+                                 "TFLOP/s": round(flops / (p_layer_us * 1e-6) / 1e12, 1),
+                                 "frac_fp8_peak": round(flops / (p_layer_us * 1e-6) / 1e12 / FP8_PEAK_TFLOPS, 4)}
+        del pl, pg
+
+    cpu = None
+    if not args.no_cpu_baseline:
+        threads = torch.get_num_threads()
+        layer_s, n_iter = cpu_baseline(layers, EXPERT_SET, M)
+        cpu = {"value": round(layer_s * 1e6 * n_layers, 1), "unit": "us per denoise step", "cores": threads,
+               "kind": "port",
+               "sample": f"torch CPU dequantize+matmul incl. quantizer and GeGLU on 1 of {n_layers} layers "
+                         f"(4 linears, M={M}), p50 of {n_iter} passes, scaled x{n_layers}"}
+
+    line = {
+        "metric": "p50 us per Pi0.5 expert denoise-step linears (fp8 W8A8)",
+        "value": round(value_us, 2), "unit": "us", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
+        "ms_per_step": round(ms_per_step, 4), "higher_is_better": False, "scaling": "weak",
+        "vs_baseline": None, "dtype": "fp8_e4m3fn x fp8_e4m3fn -> fp32 acc -> bf16", "data": "synthetic",
+        "config": {"workload": "action-expert linear set: 18 layers x {qkv 1024->2560, o 2048->1024, "
+                               "gate_up 1024->8192 + GeGLU, down 4096->1024}, M=50, distinct weights per layer",
+                   "step": "one hipGraph replay = 10 denoise steps = 720 quantized linears",
+                   "denoise_steps_per_replay": denoise_steps, "cache_policy":
+                   "311 MB of weights per denoise step cycle through HBM; nothing is pinned in cache"},
+        "roofline": roofline, "cpu_baseline": cpu, "extra": extra,
+    }
+    print(json.dumps(line))
+    return 0
+
+
+if __name__ == "__main__":
+    sys.exit(main())

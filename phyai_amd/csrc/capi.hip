@@ -46,7 +46,13 @@ struct LinearCarve {
 };
 LinearCarve carve(int64_t M, int64_t N, int64_t K, int epilogue) {
     LinearCarve c;
-    c.gemm_bytes = align_up(phyai::gemm_workspace_bytes(M, N, K, epilogue), 256);
+    {
+        const int64_t n_out = phyai::epi_is_gated(epilogue) ? N / 2 : N;
+        // worst case over output strides: the widest of the kernels that may be chosen
+        size_t a = phyai::gemm_workspace_bytes(M, N, K, epilogue, n_out);
+        size_t b = phyai::gemm_workspace_bytes(M, N, K, epilogue, 1);
+        c.gemm_bytes = align_up(a > b ? a : b, 256);
+    }
     c.xq_off = c.gemm_bytes;
     c.xs_off = c.xq_off + align_up((size_t)(M > 0 ? M : 0) * (size_t)(K > 0 ? K : 0), 256);
     c.total = c.xs_off + align_up((size_t)(M > 0 ? M : 0) * sizeof(float), 256);
@@ -137,7 +143,7 @@ int phyai_fp8_gemm(const void* xq, const float* x_scale, int x_scale_is_scalar, 
     const int rc = phyai::launch_gemm(g, static_cast<hipStream_t>(stream));
     if (rc == -3)
         return fail(PHYAI_FP8_EWORKSPACE, "phyai_fp8_gemm: workspace of %zu bytes is too small, need %zu",
-                    workspace ? workspace_bytes : (size_t)0, phyai::gemm_workspace_bytes(M, N, K, epilogue));
+                    workspace ? workspace_bytes : (size_t)0, phyai::gemm_workspace_bytes(M, N, K, epilogue, ldo));
     if (rc != 0) return fail(PHYAI_FP8_EUNSUPPORTED, "phyai_fp8_gemm: no kernel for this problem (rc=%d)", rc);
     return check_launch("phyai_fp8_gemm");
 }

@@ -1,0 +1,287 @@
+// Weight-streaming fp8 GEMM for at most 64 token rows (the M = 50 action-chunk regime).
+//
+// At these sizes a whole weight matrix (2-8 MB) is less than what the chip holds
+// in flight, so the kernel is built around latency, not throughput:
+//
+//  * No cross-workgroup reduction.  A workgroup owns 16*NT output columns over the
+//    WHOLE K range; its eight wavefronts split K between them (wavefront w takes
+//    the 128-byte K steps w, w+8, w+16, ...) and meet once, in LDS, to add their
+//    partial sums in wavefront order (fixed order: reproducible results).  A
+//    device-wide split-K would need three dependent trips to memory (publish
+//    partials, bump a counter, read partials back); this needs none.
+//  * Few output columns (N = 1024) would leave most CUs idle, and every workgroup has to
+//    read the activations of all its token rows, so such shapes are also split along M
+//    (grid.y): a workgroup then owns 16*NT columns x 16*MB token rows.  Workgroups that
+//    share a weight tile differ only in blockIdx.y, and with a multiple of 8 tiles they land
+//    on the same XCD, so the tile comes from HBM once and from that XCD's L2 afterwards.
+//  * Every lane requests all of its bytes first - weights and quantized
+//    activations, straight from global memory into VGPRs in MFMA operand layout -
+//    together with the scales and bias the epilogue will want, and only then
+//    starts to compute.  Nothing is staged through LDS before the MFMAs, so there
+//    is no barrier between the loads and the math.
+//  * v_mfma_f32_16x16x128_f8f6f4: lane l supplies operand row (l % 16) and 32 of
+//    the 128 K bytes of a step.  Which 32 is free as long as both operands agree;
+//    lane group q = l / 16 takes bytes [16q, 16q+16) and [64+16q, 64+16q+16), so
+//    one 128-bit load instruction reads 64 contiguous bytes of each of 16 rows.
+//    w is the "A" operand (rows = output columns n), x the "B" operand (columns =
+//    token rows m): accumulator register r of lane l is
+//    out[m = 16*mb + l%16][n = n0 + 4*(l/16) + r].
+//  * Gated epilogues (GeGLU / SwiGLU): the 16 operand rows of a tile are 8 gate
+//    columns and the 8 up columns that pair with them, so gate and up of one output
+//    sit 32 lanes apart in the same accumulator and meet in the LDS reduction.
+//  * After the reduction one thread owns four consecutive output columns of one
+//    token: scale, bias, activation, one 64-bit bf16x4 store.
+#include "fp8_device.h"
+#include "launch.h"
+#include <stdio.h>
+#include <stdlib.h>
+
+namespace phyai {
+
+struct SkinnyArgs {
+    const uint8_t* __restrict__ xq;  // [M, K]
+    const uint8_t* __restrict__ w;   // [N, K]
+    const float* __restrict__ x_scale;
+    const float* __restrict__ w_scale;
+    const uint16_t* __restrict__ bias;
+    uint16_t* __restrict__ out;
+    int64_t ldo;
+    int M, N, K;
+    int x_scale_scalar;
+    int rounds;  // K steps are consumed in rounds of SK_WAVES * KPW
+};
+
+constexpr int SK_WAVES = 8;
+constexpr int SK_THREADS = SK_WAVES * kWave;
+
+__device__ __forceinline__ v8i join(v4i lo, v4i hi) {
+    v8i f;
+    f[0] = lo[0]; f[1] = lo[1]; f[2] = lo[2]; f[3] = lo[3];
+    f[4] = hi[0]; f[5] = hi[1]; f[6] = hi[2]; f[7] = hi[3];
+    return f;
+}
+
+// MB: 16-row token blocks per workgroup (grid.y workgroups cover M); NT: 16-row weight
+// tiles per workgroup; KPW: K steps per wavefront per round.
+template <int MB, int NT, int KPW, int EPI>
+__global__ __launch_bounds__(SK_THREADS) void gemm_fp8_skinny_kernel(const SkinnyArgs p) {
+    constexpr bool GATED = epi_is_gated(EPI);
+    constexpr int COLS_PER_TILE = GATED ? 8 : 16;  // output columns per 16-row weight tile
+
+    __shared__ v4f red[SK_WAVES][NT][MB][kWave];
+
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const int l16 = lane & 15, q = lane >> 4;
+    const int half_n = p.N / 2;
+    const int n_out_total = GATED ? half_n : p.N;
+    const int col0 = blockIdx.x * (COLS_PER_TILE * NT);  // first output column of the workgroup
+    const int total_steps = p.K >> 7;
+    const int m_base = blockIdx.y * (MB * 16);
+
+    // ---- epilogue role of this thread and its operands (requested first) ---------
+    // thread -> (tile e_nt, token block e_mb, lane position e_lane); it finishes token
+    // m = 16*e_mb + e_lane%16 and output columns e_n .. e_n+3.
+    const int e_lane = tid & 63;
+    const int e_mb = (tid >> 6) % MB;
+    const int e_nt = (tid >> 6) / MB;
+    const int e_q = e_lane >> 4;
+    const bool e_role = (e_nt < NT) && (!GATED || e_q < 2);
+    const int e_m = m_base + e_mb * 16 + (e_lane & 15);
+    const int e_n = col0 + (e_nt < NT ? e_nt : 0) * COLS_PER_TILE + 4 * e_q;
+    const bool e_live = e_role && e_m < p.M && e_n < n_out_total;
+    const int e_n_safe = e_live ? e_n : 0;
+    const v4f sw4 = *reinterpret_cast<const v4f*>(p.w_scale + e_n_safe);
+    v4f su4 = v4f{0.f, 0.f, 0.f, 0.f};
+    if constexpr (GATED) su4 = *reinterpret_cast<const v4f*>(p.w_scale + half_n + e_n_safe);
+    uint2 bw2 = make_uint2(0, 0), bu2 = make_uint2(0, 0);
+    if (p.bias) {
+        bw2 = *reinterpret_cast<const uint2*>(p.bias + e_n_safe);
+        if constexpr (GATED) bu2 = *reinterpret_cast<const uint2*>(p.bias + half_n + e_n_safe);
+    }
+    const float sa = p.x_scale[(p.x_scale_scalar || !e_live) ? 0 : e_m];
+
+    // ---- operand row pointers ---------------------------------------------------------
+    const uint8_t* wrow[NT];
+#pragma unroll
+    for (int nt = 0; nt < NT; ++nt) {
+        int r;
+        if constexpr (GATED) {
+            const int g = col0 + nt * 8 + (l16 & 7);
+            r = (l16 < 8 ? 0 : half_n) + (g < half_n ? g : half_n - 1);
+        } else {
+            r = col0 + nt * 16 + l16;
+            r = r < p.N ? r : p.N - 1;
+        }
+        wrow[nt] = p.w + (size_t)r * p.K + q * 16;
+    }
+    const uint8_t* xrow[MB];
+#pragma unroll
+    for (int mb = 0; mb < MB; ++mb) {
+        int r = m_base + mb * 16 + l16;
+        r = r < p.M ? r : p.M - 1;  // rows past M only feed outputs that are never stored
+        xrow[mb] = p.xq + (size_t)r * p.K + q * 16;
+    }
+
+    v4f acc[NT][MB];
+#pragma unroll
+    for (int nt = 0; nt < NT; ++nt)
+#pragma unroll
+        for (int mb = 0; mb < MB; ++mb) acc[nt][mb] = v4f{0.f, 0.f, 0.f, 0.f};
+
+    for (int rnd = 0; rnd < p.rounds; ++rnd) {
+        v4i wlo[KPW][NT], whi[KPW][NT], xlo[KPW][MB], xhi[KPW][MB];
+        bool live[KPW];
+        // ---- 1. request every byte of this round ------------------------------------
+#pragma unroll
+        for (int j = 0; j < KPW; ++j) {
+            const int s = (rnd * KPW + j) * SK_WAVES + wave;  // wave-uniform
+            live[j] = s < total_steps;
+            const int off = (live[j] ? s : total_steps - 1) << 7;
+#pragma unroll
+            for (int nt = 0; nt < NT; ++nt) {
+                wlo[j][nt] = *reinterpret_cast<const v4i*>(wrow[nt] + off);
+                whi[j][nt] = *reinterpret_cast<const v4i*>(wrow[nt] + off + 64);
+            }
+#pragma unroll
+            for (int mb = 0; mb < MB; ++mb) {
+                xlo[j][mb] = *reinterpret_cast<const v4i*>(xrow[mb] + off);
+                xhi[j][mb] = *reinterpret_cast<const v4i*>(xrow[mb] + off + 64);
+            }
+        }
+        // ---- 2. MFMA ---------------------------------------------------------------------
+#pragma unroll
+        for (int j = 0; j < KPW; ++j) {
+#pragma unroll
+            for (int nt = 0; nt < NT; ++nt) {
+                v8i a = join(wlo[j][nt], whi[j][nt]);
+                if (!live[j]) a = v8i{0, 0, 0, 0, 0, 0, 0, 0};  // a step past K adds nothing
+#pragma unroll
+                for (int mb = 0; mb < MB; ++mb)
+                    acc[nt][mb] = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(
+                        a, join(xlo[j][mb], xhi[j][mb]), acc[nt][mb], 0, 0, 0, 0, 0, 0);
+            }
+        }
+    }
+
+    // ---- 3. add the eight wavefronts' partial sums, in wavefront order -------------------
+#pragma unroll
+    for (int nt = 0; nt < NT; ++nt)
+#pragma unroll
+        for (int mb = 0; mb < MB; ++mb) red[wave][nt][mb][lane] = acc[nt][mb];
+    __syncthreads();
+    if (!e_role) return;
+    v4f g = red[0][e_nt][e_mb][e_lane];
+#pragma unroll
+    for (int w = 1; w < SK_WAVES; ++w) g += red[w][e_nt][e_mb][e_lane];
+    v4f u = v4f{0.f, 0.f, 0.f, 0.f};
+    if constexpr (GATED) {
+        u = red[0][e_nt][e_mb][e_lane + 32];
+#pragma unroll
+        for (int w = 1; w < SK_WAVES; ++w) u += red[w][e_nt][e_mb][e_lane + 32];
+    }
+
+    // ---- 4. epilogue ------------------------------------------------------------------------
+    const float bwf[4] = {bf16_bits_to_f32(bw2.x & 0xFFFFu), bf16_bits_to_f32(bw2.x >> 16),
+                          bf16_bits_to_f32(bw2.y & 0xFFFFu), bf16_bits_to_f32(bw2.y >> 16)};
+    const float buf[4] = {bf16_bits_to_f32(bu2.x & 0xFFFFu), bf16_bits_to_f32(bu2.x >> 16),
+                          bf16_bits_to_f32(bu2.y & 0xFFFFu), bf16_bits_to_f32(bu2.y >> 16)};
+    uint32_t o[4];
+#pragma unroll
+    for (int r = 0; r < 4; ++r) {
+        float v = g[r] * (sa * sw4[r]) + bwf[r];
+        if constexpr (GATED) {
+            const float up = u[r] * (sa * su4[r]) + buf[r];
+            v = apply_act<EPI>(round_bf16(v)) * round_bf16(up);
+        } else if constexpr (EPI != EPI_NONE) {
+            v = apply_act<EPI>(round_bf16(v));
+        }
+        o[r] = f32_to_bf16_bits(v);
+    }
+    if (e_live)
+        *reinterpret_cast<uint2*>(p.out + (int64_t)e_m * p.ldo + e_n) =
+            make_uint2(o[0] | (o[1] << 16), o[2] | (o[3] << 16));
+}
+
+// ---- host side -------------------------------------------------------------------------
+
+static int sk_ceil_div(int a, int b) { return (a + b - 1) / b; }
+
+// Widths are multiples of 8 so that four consecutive output columns are valid together.
+bool skinny_applicable(int M, int N, int K, int epilogue, int64_t ldo) {
+    if (M > 64 || K % 128 != 0 || ldo % 4 != 0) return false;
+    if (epi_is_gated(epilogue)) return (N / 2) % 8 == 0;
+    return N % 8 == 0;
+}
+
+SkinnyPlan skinny_plan(int M, int N, int K, int epilogue) {
+    const bool gated = epi_is_gated(epilogue);
+    const int cols = gated ? N / 2 : N;
+    const int per_tile = gated ? 8 : 16;
+    SkinnyPlan pl;
+    const int blocks = sk_ceil_div(M, 16);  // 16-row token blocks in all
+    // two weight tiles per workgroup once that still leaves a workgroup for every CU
+    pl.nt = sk_ceil_div(cols, 2 * per_tile) >= 256 ? 2 : 1;
+    pl.tiles = sk_ceil_div(cols, per_tile * pl.nt);
+    // split M while there are fewer workgroups than CUs
+    pl.msplit = 1;
+    if (blocks % 2 == 0 && pl.tiles * 2 <= 256) pl.msplit = 2;
+    if (blocks % 4 == 0 && pl.tiles * 4 <= 256) pl.msplit = 4;
+    if (blocks == 3 && pl.tiles * 3 <= 256) pl.msplit = 3;
+    pl.mb = blocks / pl.msplit;
+    const int steps = K / 128;
+    const int per_wave = sk_ceil_div(steps, SK_WAVES);
+    pl.kpw = per_wave >= 4 ? 4 : (per_wave >= 2 ? 2 : 1);
+    pl.rounds = sk_ceil_div(per_wave, pl.kpw);
+    if (const char* e = getenv("PHYAI_FP8_SKINNY_PLAN")) {  // "nt,msplit" tuning override
+        int nt = 0, ms = 0;
+        if (sscanf(e, "%d,%d", &nt, &ms) == 2 && (nt == 1 || nt == 2) && ms >= 1 && blocks % ms == 0) {
+            pl.nt = nt; pl.tiles = sk_ceil_div(cols, per_tile * nt); pl.msplit = ms; pl.mb = blocks / ms;
+        }
+    }
+    return pl;
+}
+
+template <int MB, int NT, int EPI>
+static int sk_launch_kpw(const SkinnyArgs& a, const SkinnyPlan& pl, hipStream_t st) {
+    const dim3 grid(pl.tiles, pl.msplit), block(SK_THREADS);
+    switch (pl.kpw) {
+    case 1: hipLaunchKernelGGL((gemm_fp8_skinny_kernel<MB, NT, 1, EPI>), grid, block, 0, st, a); return 0;
+    case 2: hipLaunchKernelGGL((gemm_fp8_skinny_kernel<MB, NT, 2, EPI>), grid, block, 0, st, a); return 0;
+    case 4: hipLaunchKernelGGL((gemm_fp8_skinny_kernel<MB, NT, 4, EPI>), grid, block, 0, st, a); return 0;
+    default: return -2;
+    }
+}
+
+template <int EPI>
+static int sk_launch_epi(const SkinnyArgs& a, const SkinnyPlan& pl, hipStream_t st) {
+    switch (pl.mb * 2 + (pl.nt - 1)) {
+    case 2: return sk_launch_kpw<1, 1, EPI>(a, pl, st);
+    case 3: return sk_launch_kpw<1, 2, EPI>(a, pl, st);
+    case 4: return sk_launch_kpw<2, 1, EPI>(a, pl, st);
+    case 5: return sk_launch_kpw<2, 2, EPI>(a, pl, st);
+    case 6: return sk_launch_kpw<3, 1, EPI>(a, pl, st);
+    case 7: return sk_launch_kpw<3, 2, EPI>(a, pl, st);
+    case 8: return sk_launch_kpw<4, 1, EPI>(a, pl, st);
+    case 9: return sk_launch_kpw<4, 2, EPI>(a, pl, st);
+    default: return -2;
+    }
+}
+
+int launch_gemm_skinny(const GemmProblem& g, const SkinnyPlan& pl, hipStream_t st) {
+    SkinnyArgs a;
+    a.xq = g.xq; a.w = g.w; a.x_scale = g.x_scale; a.w_scale = g.w_scale; a.bias = g.bias;
+    a.out = g.out; a.ldo = g.ldo; a.M = g.M; a.N = g.N; a.K = g.K;
+    a.x_scale_scalar = g.x_scale_is_scalar;
+    a.rounds = pl.rounds;
+    switch (g.epilogue) {
+    case EPI_NONE: return sk_launch_epi<EPI_NONE>(a, pl, st);
+    case EPI_GEGLU_TANH: return sk_launch_epi<EPI_GEGLU_TANH>(a, pl, st);
+    case EPI_GEGLU_ERF: return sk_launch_epi<EPI_GEGLU_ERF>(a, pl, st);
+    case EPI_SWIGLU: return sk_launch_epi<EPI_SWIGLU>(a, pl, st);
+    case EPI_GELU_TANH: return sk_launch_epi<EPI_GELU_TANH>(a, pl, st);
+    case EPI_GELU_ERF: return sk_launch_epi<EPI_GELU_ERF>(a, pl, st);
+    default: return -2;
+    }
+}
+
+}  // namespace phyai

@@ -25,6 +25,7 @@
 // counter, which keeps the workspace header zero between calls.
 #include "fp8_device.h"
 #include "launch.h"
+#include "splitk.h"
 
 namespace phyai {
 
@@ -176,59 +177,40 @@ __global__ __launch_bounds__(256) void gemm_fp8_tile_kernel(const TileArgs p) {
         const int S = gridDim.z;
         const int tile = blockIdx.y * gridDim.x + blockIdx.x;
         constexpr int FRAG = TM * TN * 16;  // floats per thread
-        float* mine = p.partials + ((size_t)tile * S + blockIdx.z) * (FRAG * 256);
+        float frag[FRAG];
 #pragma unroll
         for (int i = 0; i < TM; ++i)
 #pragma unroll
             for (int j = 0; j < TN; ++j)
 #pragma unroll
-                for (int r = 0; r < 16; ++r) mine[((i * TN + j) * 16 + r) * 256 + tid] = acc[i][j][r];
-        __threadfence();
-        __syncthreads();
-        if (tid == 0) {
-            const int old = __hip_atomic_fetch_add(p.counters + tile, 1, __ATOMIC_ACQ_REL,
-                                                   __HIP_MEMORY_SCOPE_AGENT);
-            s_last = (old == S - 1);
-        }
-        __syncthreads();
-        if (!s_last) return;
-        __threadfence();
-        const float* all = p.partials + (size_t)tile * S * (FRAG * 256);
+                for (int r = 0; r < 16; ++r) frag[(i * TN + j) * 16 + r] = acc[i][j][r];
+        splitk_publish<FRAG, 256>(p.partials, tile, S, blockIdx.z, frag);
+        if (!splitk_arrive(p.counters, tile, S, &s_last)) return;
+        splitk_gather<FRAG, 256>(p.partials, p.counters, tile, S, frag);
 #pragma unroll
         for (int i = 0; i < TM; ++i)
 #pragma unroll
             for (int j = 0; j < TN; ++j)
 #pragma unroll
-                for (int r = 0; r < 16; ++r) acc[i][j][r] = 0.f;
-        for (int z = 0; z < S; ++z) {
-            const float* pz = all + (size_t)z * (FRAG * 256);
-#pragma unroll
-            for (int i = 0; i < TM; ++i)
-#pragma unroll
-                for (int j = 0; j < TN; ++j)
-#pragma unroll
-                    for (int r = 0; r < 16; ++r)
-                        acc[i][j][r] += __builtin_nontemporal_load(pz + ((i * TN + j) * 16 + r) * 256 + tid);
-        }
-        if (tid == 0)
-            __hip_atomic_store(p.counters + tile, 0, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+                for (int r = 0; r < 16; ++r) acc[i][j][r] = frag[(i * TN + j) * 16 + r];
     }
 
     // ---- epilogue ------------------------------------------------------------
     constexpr int TNO = GATED ? TN / 2 : TN;  // output column blocks per wave
+    float sa[TM][16];
+#pragma unroll
+    for (int i = 0; i < TM; ++i)
+#pragma unroll
+        for (int r = 0; r < 16; ++r) {
+            const int m = m0 + wm * WM + i * 32 + 8 * (r / 4) + 4 * h + (r % 4);
+            sa[i][r] = p.a_scale[(p.a_scale_scalar || m >= p.M) ? 0 : m];
+        }
 #pragma unroll
     for (int j = 0; j < TNO; ++j) {
-        int n_gate, n_out;
-        if constexpr (GATED) {
-            n_out = n0 + wn * (WN / 2) + j * 32 + l32;  // column in [0, N/2)
-            n_gate = n_out;
-        } else {
-            n_out = n0 + wn * WN + j * 32 + l32;
-            n_gate = n_out;
-        }
+        const int n_out = n0 + (GATED ? wn * (WN / 2) : wn * WN) + j * 32 + l32;
         const int n_lim = GATED ? half_n : p.N;
         const bool n_ok = n_out < n_lim;
-        const int n_safe = n_ok ? n_gate : 0;
+        const int n_safe = n_ok ? n_out : 0;
         const float sg = p.b_scale[n_safe];
         const float bg = p.bias ? bf16_bits_to_f32(p.bias[n_safe]) : 0.f;
         float su = 0.f, bu = 0.f;
@@ -241,17 +223,14 @@ __global__ __launch_bounds__(256) void gemm_fp8_tile_kernel(const TileArgs p) {
 #pragma unroll
             for (int r = 0; r < 16; ++r) {
                 const int m = m0 + wm * WM + i * 32 + 8 * (r / 4) + 4 * h + (r % 4);
-                if (m < p.M && n_ok) {
-                    const float sa = p.a_scale[p.a_scale_scalar ? 0 : m];
-                    float v = acc[i][j][r] * (sa * sg) + bg;
-                    if constexpr (GATED) {
-                        const float u = acc[i][j + TN / 2][r] * (sa * su) + bu;
-                        v = apply_act<EPI>(round_bf16(v)) * round_bf16(u);
-                    } else if constexpr (EPI != EPI_NONE) {
-                        v = apply_act<EPI>(round_bf16(v));
-                    }
-                    p.out[(int64_t)m * p.ldo + n_out] = (uint16_t)f32_to_bf16_bits(v);
+                float v = acc[i][j][r] * (sa[i][r] * sg) + bg;
+                if constexpr (GATED) {
+                    const float u = acc[i][j + TN / 2][r] * (sa[i][r] * su) + bu;
+                    v = apply_act<EPI>(round_bf16(v)) * round_bf16(u);
+                } else if constexpr (EPI != EPI_NONE) {
+                    v = apply_act<EPI>(round_bf16(v));
                 }
+                if (m < p.M && n_ok) p.out[(int64_t)m * p.ldo + n_out] = (uint16_t)f32_to_bf16_bits(v);
             }
         }
     }
@@ -259,7 +238,7 @@ __global__ __launch_bounds__(256) void gemm_fp8_tile_kernel(const TileArgs p) {
 
 // ---- host side ---------------------------------------------------------------
 
-constexpr size_t kHeaderBytes = 16384;  // split-K tile counters (4096 ints)
+constexpr size_t kHeaderBytes = kGemmHeaderBytes;
 
 struct TileConfig {
     int bm, bn;
@@ -309,8 +288,9 @@ static size_t partial_bytes(const TileConfig& c, int M, int N, int epilogue) {
     return tiles * c.splits * (size_t)c.bm * c.bn * sizeof(float);
 }
 
-size_t gemm_workspace_bytes(int64_t M, int64_t N, int64_t K, int epilogue) {
+size_t gemm_workspace_bytes(int64_t M, int64_t N, int64_t K, int epilogue, int64_t ldo) {
     if (M <= 0 || N <= 0 || K <= 0) return kHeaderBytes;
+    if (skinny_applicable((int)M, (int)N, (int)K, epilogue, ldo)) return kHeaderBytes;
     const TileConfig c = pick_config((int)M, (int)N, (int)K, epilogue);
     return kHeaderBytes + partial_bytes(c, (int)M, (int)N, epilogue);
 }
@@ -338,6 +318,12 @@ static int launch_epi(const TileArgs& a, const TileConfig& c, dim3 grid, hipStre
 
 int launch_gemm(const GemmProblem& g, hipStream_t st) {
     if (g.M == 0 || g.N == 0) return 0;
+    // The skinny kernel reads scales / bias / output with 128- and 64-bit accesses.
+    const bool vec_ok = (reinterpret_cast<uintptr_t>(g.w_scale) % 16 == 0) &&
+                        (reinterpret_cast<uintptr_t>(g.bias) % 8 == 0) &&
+                        (reinterpret_cast<uintptr_t>(g.out) % 8 == 0);
+    if (vec_ok && skinny_applicable(g.M, g.N, g.K, g.epilogue, g.ldo))
+        return launch_gemm_skinny(g, skinny_plan(g.M, g.N, g.K, g.epilogue), st);
     const TileConfig c = pick_config(g.M, g.N, g.K, g.epilogue);
     const bool gated = epi_is_gated(g.epilogue);
     const int n_eff = gated ? g.N / 2 : g.N;

@@ -30,7 +30,22 @@ struct GemmProblem {
     size_t workspace_bytes;
 };
 
-size_t gemm_workspace_bytes(int64_t M, int64_t N, int64_t K, int epilogue);
+constexpr size_t kGemmHeaderBytes = 16384;  // split-K arrival counters (4096 ints) at the workspace start
+
+size_t gemm_workspace_bytes(int64_t M, int64_t N, int64_t K, int epilogue, int64_t ldo);
 int launch_gemm(const GemmProblem& p, hipStream_t st);
+
+// Weight-streaming kernel for M <= 64 (gemm_skinny.hip).  It needs no workspace.
+struct SkinnyPlan {
+    int tiles;   // workgroups (each owns 16*nt weight rows over the whole K)
+    int msplit;  // workgroups along M
+    int mb;      // 16-row token blocks per workgroup
+    int nt;      // weight tiles per workgroup
+    int kpw;     // K steps per wavefront per round
+    int rounds;
+};
+bool skinny_applicable(int M, int N, int K, int epilogue, int64_t ldo);
+SkinnyPlan skinny_plan(int M, int N, int K, int epilogue);
+int launch_gemm_skinny(const GemmProblem& p, const SkinnyPlan& pl, hipStream_t st);
 
 }  // namespace phyai

@@ -1,0 +1,77 @@
+// Cross-workgroup split-K reduction without cache-wide fences.
+//
+// An MI355X has eight XCDs, each with its own L2; a device-scope fence makes a
+// workgroup write back / invalidate that whole L2 and costs microseconds when a
+// few hundred workgroups do it.  Instead every access to data that crosses
+// workgroups (partial sums, arrival counters) is a relaxed device-scope atomic:
+// stores are written through to memory, loads never hit a stale L2 line, and no
+// fence wider than the workgroup is issued.  Ordering inside a workgroup:
+// each lane waits for its own stores to complete (vmcnt(0)), the workgroup
+// barrier collects all lanes, then one lane bumps the tile's counter.
+//
+// Partials are summed by the last workgroup to arrive, in split order, so the
+// result does not depend on arrival order.  That workgroup also resets the
+// counter, which is how the workspace header stays zero from call to call.
+#pragma once
+
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+namespace phyai {
+
+__device__ __forceinline__ void coherent_store2(float* p, float a, float b) {
+    uint64_t v = (uint64_t)__float_as_uint(a) | ((uint64_t)__float_as_uint(b) << 32);
+    __hip_atomic_store(reinterpret_cast<uint64_t*>(p), v, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+}
+
+__device__ __forceinline__ void coherent_load2(const float* p, float& a, float& b) {
+    uint64_t v = __hip_atomic_load(reinterpret_cast<const uint64_t*>(p), __ATOMIC_RELAXED,
+                                   __HIP_MEMORY_SCOPE_AGENT);
+    a = __uint_as_float((uint32_t)v);
+    b = __uint_as_float((uint32_t)(v >> 32));
+}
+
+__device__ __forceinline__ void wait_own_stores() { asm volatile("s_waitcnt vmcnt(0)" ::: "memory"); }
+
+// FRAG floats per thread (even), THREADS threads.  Layout of one partial:
+// [FRAG/2][THREADS][2] floats, so that a wavefront's 64-bit accesses are contiguous.
+template <int FRAG, int THREADS>
+__device__ __forceinline__ void splitk_publish(float* partials, int tile, int S, int z, const float* frag) {
+    float* mine = partials + ((size_t)tile * S + z) * (size_t)(FRAG * THREADS);
+#pragma unroll
+    for (int e = 0; e < FRAG; e += 2)
+        coherent_store2(mine + ((e / 2) * THREADS + threadIdx.x) * 2, frag[e], frag[e + 1]);
+    wait_own_stores();
+}
+
+// Returns true in every lane of the workgroup that arrived last.  Must be called by all
+// threads, after splitk_publish.
+__device__ __forceinline__ bool splitk_arrive(int* counters, int tile, int S, int* s_flag) {
+    __syncthreads();
+    if (threadIdx.x == 0) {
+        const int old = __hip_atomic_fetch_add(counters + tile, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        *s_flag = (old == S - 1);
+    }
+    __syncthreads();
+    return *s_flag != 0;
+}
+
+template <int FRAG, int THREADS>
+__device__ __forceinline__ void splitk_gather(const float* partials, int* counters, int tile, int S, float* frag) {
+    const float* all = partials + (size_t)tile * S * (size_t)(FRAG * THREADS);
+#pragma unroll
+    for (int e = 0; e < FRAG; ++e) frag[e] = 0.f;
+    for (int z = 0; z < S; ++z) {
+        const float* pz = all + (size_t)z * (FRAG * THREADS);
+        float t[FRAG];
+#pragma unroll
+        for (int e = 0; e < FRAG; e += 2)
+            coherent_load2(pz + ((e / 2) * THREADS + threadIdx.x) * 2, t[e], t[e + 1]);
+#pragma unroll
+        for (int e = 0; e < FRAG; ++e) frag[e] += t[e];
+    }
+    if (threadIdx.x == 0)
+        __hip_atomic_store(counters + tile, 0, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+}
+
+}  // namespace phyai

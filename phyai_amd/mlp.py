@@ -1,0 +1,116 @@
+"""DenseMLP - two-layer FFN, gated (SwiGLU / GeGLU) or plain.
+
+Constructor and semantics follow the reference's
+``phyai/layers/mlp/dense_mlp.py:127-289``.  The difference is where the
+activation runs: the reference launches a separate ``act_and_mul`` kernel on the
+``[M, 2I]`` bf16 output of ``gate_up_proj`` (``dense_mlp.py:256-261``); here,
+when the first linear is an fp8 layer served by the HIP kernel, the activation
+is the GEMM's epilogue and the ``[M, 2I]`` tensor never reaches memory.  The
+fused epilogue rounds gate and up to bf16 before the activation, exactly as the
+two-launch form does, so the two agree up to accumulation order.
+
+gate occupies columns ``[0, I)`` and up columns ``[I, 2I)`` of the fused
+projection (``dense_mlp.py:11-15``).
+"""
+
+from __future__ import annotations
+
+import functools
+from typing import Callable, Literal
+
+import torch
+import torch.nn as nn
+import torch.nn.functional as F
+
+from phyai_amd.linear import ColumnParallelLinear, MergedColumnParallelLinear, RowParallelLinear
+
+_GATED_ACTS = ("silu", "gelu", "gelu_tanh")
+_PLAIN_ACTS = ("gelu", "gelu_tanh")
+_TANH_ALIASES = ("gelu_tanh", "gelu_pytorch_tanh", "gelu_new")
+
+_GATED_EPILOGUE = {"silu": "swiglu", "gelu": "geglu_erf", "gelu_tanh": "geglu_tanh"}
+_PLAIN_EPILOGUE = {"gelu": "gelu_erf", "gelu_tanh": "gelu_tanh"}
+
+
+def _canonicalise_activation(name: str) -> str:
+    canon = name.lower().replace("-", "_")
+    return "gelu_tanh" if canon in _TANH_ALIASES else canon
+
+
+def _act_and_mul(name: str) -> Callable[[torch.Tensor], torch.Tensor]:
+    """Unfused ``act(x[..., :I]) * x[..., I:]`` for layers the HIP kernel does not serve
+    (bf16 weights): fp32 math, bf16 result, like the reference's activation kernel."""
+    canon = _canonicalise_activation(name)
+    if canon not in _GATED_ACTS:
+        raise ValueError(f"Unsupported gated activation {name!r}; expected one of {_GATED_ACTS!r}.")
+    act = {"silu": F.silu, "gelu": F.gelu, "gelu_tanh": functools.partial(F.gelu, approximate="tanh")}[canon]
+
+    def run(fused: torch.Tensor) -> torch.Tensor:
+        half = fused.shape[-1] // 2
+        return (act(fused[..., :half].float()) * fused[..., half:].float()).to(fused.dtype)
+
+    return run
+
+
+def _plain_act(name: str) -> Callable[[torch.Tensor], torch.Tensor]:
+    canon = _canonicalise_activation(name)
+    if canon == "gelu":
+        return F.gelu
+    if canon == "gelu_tanh":
+        return functools.partial(F.gelu, approximate="tanh")
+    if canon == "silu":
+        raise ValueError("non-gated SiLU is not supported (no real model uses it; did you mean gated=True?)")
+    raise ValueError(f"Unsupported plain activation {name!r}; expected one of {_PLAIN_ACTS!r}.")
+
+
+class DenseMLP(nn.Module):
+    def __init__(self, hidden_size: int, intermediate_size: int, *,
+                 activation: Literal["silu", "gelu", "gelu_tanh"] = "silu", gated: bool = True,
+                 bias: bool = False, axis: str = "tp", sp_axis: str | None = None,
+                 params_dtype: torch.dtype | None = None, spec_in: object | None = None,
+                 spec_out: object | None = None, gated_hf_legs: tuple[str, str] = ("gate_proj", "up_proj"),
+                 mesh: str = "model", prefix: str = "", fuse_activation: bool = True) -> None:
+        super().__init__()
+        self.hidden_size = hidden_size
+        self.intermediate_size = intermediate_size
+        self.activation = _canonicalise_activation(activation)
+        self.gated = gated
+        self.bias_enabled = bias
+        self.prefix = prefix
+        self.fuse_activation = fuse_activation
+        child = (lambda n: f"{prefix}.{n}" if prefix else n)
+        common = dict(axis=axis, sp_axis=sp_axis, bias=bias, params_dtype=params_dtype, mesh=mesh)
+        if gated:
+            self._unfused_act = _act_and_mul(activation)
+            self._epilogue = _GATED_EPILOGUE[self.activation]
+            self.gate_up_proj = MergedColumnParallelLinear(
+                hidden_size, [intermediate_size, intermediate_size], gather_output=False, spec=spec_in,
+                hf_legs=gated_hf_legs, prefix=child("gate_up_proj"), **common)
+            self.down_proj = RowParallelLinear(
+                intermediate_size, hidden_size, input_is_parallel=True, reduce_results=True, spec=spec_out,
+                prefix=child("down_proj"), **common)
+        else:
+            self._unfused_act = _plain_act(activation)
+            self._epilogue = _PLAIN_EPILOGUE[self.activation]
+            self.fc1 = ColumnParallelLinear(hidden_size, intermediate_size, gather_output=False, spec=spec_in,
+                                            prefix=child("fc1"), **common)
+            self.fc2 = RowParallelLinear(intermediate_size, hidden_size, input_is_parallel=True,
+                                         reduce_results=True, spec=spec_out, prefix=child("fc2"), **common)
+
+    def forward(self, x: torch.Tensor) -> torch.Tensor:
+        first = self.gate_up_proj if self.gated else self.fc1
+        second = self.down_proj if self.gated else self.fc2
+        if self.fuse_activation and first.supports_fused_epilogue(x):
+            h = first.forward_fused(x, self._epilogue)
+        else:
+            h, _ = first(x)
+            h = self._unfused_act(h)
+        out, _ = second(h)
+        return out
+
+    def extra_repr(self) -> str:
+        return (f"hidden_size={self.hidden_size}, intermediate_size={self.intermediate_size}, "
+                f"activation={self.activation!r}, gated={self.gated}, bias={self.bias_enabled}")
+
+
+__all__ = ["DenseMLP"]

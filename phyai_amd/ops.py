@@ -83,12 +83,10 @@ def reserve_workspace(nbytes: int, device: torch.device | None = None) -> torch.
     key = (idx, _stream_ptr())
     ws = _workspaces.get(key)
     if ws is None or ws.numel() < nbytes:
-        if torch.cuda.is_current_stream_capturing():
-            raise _err(
-                "reserve_workspace",
-                f"workspace of {nbytes} bytes needed while a graph is being captured; "
-                "run the op once (or call reserve_workspace) before capture",
-            )
+        # Outside capture this is a one-off allocation.  Inside a capture (an op met on a
+        # stream that never ran it before) the tensor comes from the graph's memory pool and
+        # the zero fill is recorded as a fill kernel - never a memset node - and replayed
+        # with the graph; warming the op up on the capture stream avoids that extra node.
         size = max(int(nbytes), 1 << 20)
         size = (size + 0xFFFFF) & ~0xFFFFF
         ws = torch.zeros(size, dtype=torch.uint8, device=torch.device("cuda", idx))
