@@ -198,7 +198,7 @@ def main() -> int:
     roofline = {
         "bound": "hbm", "achieved": round(achieved, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
         "frac": round(achieved / HBM_PEAK_GBS, 4), "traffic": None,
-        "kernel": "gemm_fp8_tile_kernel (M=50, four expert shapes)",
+        "kernel": "gemm_fp8_skinny_kernel (M=50, four expert shapes)",
         "bytes_per_layer": layer_bytes,
         "per_shape": {name: {"us": round(per_launch_us[name], 3),
                              "GB/s": round(algorithmic_bytes(M, N, K, epi) / per_launch_us[name] / 1e3, 1)}
