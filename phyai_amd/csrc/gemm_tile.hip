@@ -26,6 +26,8 @@
 #include "fp8_device.h"
 #include "launch.h"
 #include "splitk.h"
+#include <stdio.h>
+#include <stdlib.h>
 
 namespace phyai {
 
@@ -260,6 +262,15 @@ static TileConfig pick_config(int M, int N, int K, int epilogue) {
         c.bm = 128;
         c.bn = 128;
     }
+    int forced_splits = 0;
+    if (const char* e = getenv("PHYAI_FP8_TILE")) {  // "bm,bn,splits" tuning override
+        int bm = 0, bn = 0, sp = 0;
+        if (sscanf(e, "%d,%d,%d", &bm, &bn, &sp) == 3 && (bm == 64 || bm == 128 || bm == 256) &&
+            (bn == 64 || bn == 128 || bn == 256) && !(bm == 64 && bn == 256) && !(bm == 256 && bn == 64) &&
+            !(gated && bn == 64)) {
+            c.bm = bm; c.bn = bn; forced_splits = sp;
+        }
+    }
     const int n_eff = gated ? N / 2 : N;
     const int bn_eff = gated ? c.bn / 2 : c.bn;
     const int tiles = ceil_div(M, c.bm) * ceil_div(n_eff, bn_eff);
@@ -272,6 +283,7 @@ static TileConfig pick_config(int M, int N, int K, int epilogue) {
         if (s > 32) s = 32;
         if (tiles > 4096) s = 1;
     }
+    if (forced_splits > 0) s = forced_splits < slabs ? forced_splits : slabs;
     // every split must own at least one slab
     const int per = ceil_div(slabs, s);
     s = ceil_div(slabs, per);
@@ -307,13 +319,17 @@ template <int EPI>
 static int launch_epi(const TileArgs& a, const TileConfig& c, dim3 grid, hipStream_t st) {
     constexpr bool GATED = epi_is_gated(EPI);
     const bool split = c.splits > 1;
-    if (c.bm == 64) {
-        if constexpr (GATED) launch_one<64, 128, 2, 2, EPI>(a, grid, split, st);
-        else launch_one<64, 64, 2, 2, EPI>(a, grid, split, st);
-    } else {
-        launch_one<128, 128, 2, 2, EPI>(a, grid, split, st);
+    const int key = c.bm * 1000 + c.bn;
+    switch (key) {
+    case 64064: if constexpr (!GATED) { launch_one<64, 64, 2, 2, EPI>(a, grid, split, st); return 0; } return -2;
+    case 64128: launch_one<64, 128, 2, 2, EPI>(a, grid, split, st); return 0;
+    case 128064: if constexpr (!GATED) { launch_one<128, 64, 2, 2, EPI>(a, grid, split, st); return 0; } return -2;
+    case 128128: launch_one<128, 128, 2, 2, EPI>(a, grid, split, st); return 0;
+    case 128256: launch_one<128, 256, 2, 2, EPI>(a, grid, split, st); return 0;
+    case 256128: launch_one<256, 128, 2, 2, EPI>(a, grid, split, st); return 0;
+    case 256256: launch_one<256, 256, 2, 2, EPI>(a, grid, split, st); return 0;
+    default: return -2;
     }
-    return 0;
 }
 
 int launch_gemm(const GemmProblem& g, hipStream_t st) {
@@ -324,6 +340,10 @@ int launch_gemm(const GemmProblem& g, hipStream_t st) {
                         (reinterpret_cast<uintptr_t>(g.out) % 8 == 0);
     if (vec_ok && skinny_applicable(g.M, g.N, g.K, g.epilogue, g.ldo))
         return launch_gemm_skinny(g, skinny_plan(g.M, g.N, g.K, g.epilogue), st);
+    if (!getenv("PHYAI_FP8_TILE") && big_applicable(g.M, g.N, g.K, g.epilogue)) {
+        const int rc = launch_gemm_big(g, st);
+        if (rc != -2) return rc;  // -2: output not 16-byte addressable, take the generic tile kernel
+    }
     const TileConfig c = pick_config(g.M, g.N, g.K, g.epilogue);
     const bool gated = epi_is_gated(g.epilogue);
     const int n_eff = gated ? g.N / 2 : g.N;

@@ -48,4 +48,8 @@ bool skinny_applicable(int M, int N, int K, int epilogue, int64_t ldo);
 SkinnyPlan skinny_plan(int M, int N, int K, int epilogue);
 int launch_gemm_skinny(const GemmProblem& p, const SkinnyPlan& pl, hipStream_t st);
 
+// 256 x 256 tile kernel for large M (gemm_big.hip).  It needs no workspace.
+bool big_applicable(int M, int N, int K, int epilogue);
+int launch_gemm_big(const GemmProblem& p, hipStream_t st);
+
 }  // namespace phyai

@@ -323,3 +323,35 @@ def test_linear_repeatable_and_workspace_stays_clean(dev):
     torch.cuda.synchronize()
     for w in ops._workspaces.values():
         assert int(w[: ops.WORKSPACE_HEADER_BYTES].max().item()) == 0
+
+
+# ---------------------------------------------------------------------------
+# 256 x 256 tile kernel (large M), forced on shapes small enough for the oracle
+# ---------------------------------------------------------------------------
+
+@pytest.mark.parametrize("M,N,K,epi_name,epi", [
+    (256, 256, 256, None, 0), (300, 512, 384, None, 0), (816, 768, 1024, None, 0), (513, 400, 640, "gelu", 5),
+    (816, 1024, 512, "geglu_tanh", 1), (260, 288, 256, "swiglu", 3), (1000, 256, 2048, None, 0),
+])
+def test_big_tile_kernel_forced(dev, monkeypatch, M, N, K, epi_name, epi):
+    ops = _ops()
+    monkeypatch.setenv("PHYAI_FP8_BIG", "2")
+    x, wq, ws, b = _problem(M, N, K, seed=7 * M + N + K)
+    got = ops.fp8_linear(x.to(dev), wq.to(dev), ws.to(dev), b.to(dev), epilogue=epi_name)
+    torch.cuda.synchronize()
+    xq, xs = ref.quant_rowwise(x)
+    want = ref.epilogue(ref.gemm_f32(xq, xs, wq, ws, b), epi).float()
+    assert_close_to_ref(got, want, f"big kernel {M}x{N}x{K} epi={epi_name}")
+
+
+def test_big_tile_kernel_exact_integer(dev, monkeypatch):
+    ops = _ops()
+    monkeypatch.setenv("PHYAI_FP8_BIG", "2")
+    g = torch.Generator().manual_seed(11)
+    for (M, N, K) in [(256, 256, 256), (700, 528, 512), (257, 784, 1152)]:
+        xi = torch.randint(-4, 5, (M, K), generator=g).float()
+        wi = torch.randint(-4, 5, (N, K), generator=g).float()
+        got = ops.fp8_gemm(xi.to(torch.float8_e4m3fn).to(dev), torch.full((M, 1), 0.5, device=dev),
+                           wi.to(torch.float8_e4m3fn).to(dev), torch.full((N,), 0.25, device=dev))
+        want = ((xi @ wi.t()) * 0.125).bfloat16()
+        assert torch.equal(got.cpu(), want), f"{(M, N, K)}"
