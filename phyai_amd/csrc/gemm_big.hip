@@ -1,38 +1,46 @@
-// MFMA-bound fp8 GEMM for large M (prefix prefill, batched serving): 256 x 256 output tile
-// per workgroup, 128 x 128 per wavefront.
+// MFMA-bound fp8 GEMM for large M (prefix prefill, batched serving).
+// Workgroup = 4 wavefronts (2 x 2); a wavefront owns TM x TN blocks of 32 x 32, so the
+// workgroup tile is 64*TM x 64*TN: 256 x 256 (TM = TN = 4) when the grid still fills the chip,
+// 128 x 128 (TM = TN = 2, two workgroups per CU) for mid-sized problems.
 //
-// Why this shape.  One v_mfma_f32_32x32x64_f8f6f4 takes 64 cycles and consumes two 2 KB
-// operand blocks.  A wavefront that owns TM x TN blocks reads (TM + TN) blocks from LDS per
-// TM*TN MFMAs; LDS delivers 128 bytes per clock to the whole CU, so four wavefronts with
-// 4 x 4 blocks each ask for 64 bytes per clock (half of what LDS can give) while 2 x 2 blocks
-// would ask for 256.  4 x 4 blocks of 16 accumulators are 256 registers: the accumulators
-// live in AGPRs, one wavefront per SIMD, and latency is hidden inside the wavefront:
+// Why 4 x 4 blocks per wavefront.  One v_mfma_f32_32x32x64_f8f6f4 takes 64 cycles and consumes
+// two 2 KB operand blocks.  A wavefront with TM x TN blocks reads (TM + TN) blocks from LDS per
+// TM*TN MFMAs; LDS delivers 128 bytes per clock to the whole CU, so four wavefronts with 4 x 4
+// blocks ask for 64 bytes per clock, 2 x 2 blocks for 128.  The same ratio governs the bytes
+// that must come from L2: (BM + BN) * K per tile, and on this chip L2 -> CU delivery
+// (measured: about 10-13 TB/s over all CUs) is what finally bounds the kernel, not the MFMA
+// pipe.  4 x 4 blocks of 16 accumulators are 256 registers: they live in AGPRs, one
+// wavefront per SIMD, and latency is hidden inside the wavefront:
 //
 //  * global -> LDS copies bypass the register file (global_load_lds_dwordx4): lane i of a
 //    wavefront fetches one 16-byte chunk and the hardware deposits chunk i at LDS base + 16*i.
 //    The XOR swizzle that keeps the 128-bit operand reads conflict-free is therefore applied
 //    on the global side: lane i (row i/4 of a 16-row group, slot i%4 of the 64-byte row)
 //    fetches chunk (i%4) ^ ((row/2)%4) of its row.
-//  * K is consumed in 64-byte slabs through a ring of four 32 KB LDS stages: the copies of
-//    slab s+3 are issued while slab s is being multiplied, so a copy has three slab times
-//    (about 1.3 us of MFMA work) to arrive.  One barrier per slab: it tells every wavefront
-//    that slab s has landed everywhere and that the stage about to be refilled is no longer
-//    being read.
-//  * inside a slab the A block of the next row group is read from LDS before the current
-//    group's four MFMAs are issued, so ds_read latency overlaps MFMA time.
+//  * K is consumed in 64-byte slabs through a ring of four LDS stages: the copies of slab s+3
+//    are issued while slab s is being multiplied.  One barrier per slab, placed in the MIDDLE
+//    of slab s: it publishes slab s+1 and tells everyone that the stage about to be refilled
+//    is no longer read.  All wavefronts reach it at about the same time, with MFMAs queued.
+//  * the operand blocks that open slab s+1 are read from LDS during the last row group of
+//    slab s into a second register set, and inside a slab the A block of the next row group is
+//    read before the current group's MFMAs are issued, so ds_read latency overlaps MFMA time.
+//  * epilogue: the accumulator layout gives a lane one column and scattered rows; each
+//    wavefront stages its bf16 tile in its own slice of the (now idle) LDS - neighbouring lanes
+//    swap one value first (DPP) so every LDS write is a packed pair of columns - and writes it
+//    out row-wise, 16 bytes per lane, whole row segments per instruction.
 //
-// Gated epilogues use the same trick as the smaller tile kernel: within a wavefront's 128
-// columns the first 64 are gate columns and the last 64 the matching up columns.
+// Gated epilogues: within a wavefront's 32*TN columns the first half are gate columns and the
+// second half the matching up columns, so the pair sits in the same lane of two accumulators.
 // Requires K % 128 == 0 and K >= 256 (slabs are never partial and come in pairs).
 #include "fp8_device.h"
 #include "launch.h"
+#include "splitk.h"
 #include <stdlib.h>
 
 namespace phyai {
 
-constexpr int BIG_BM = 256, BIG_BN = 256, BIG_BK = 64;
+constexpr int BIG_BK = 64;
 constexpr int BIG_STAGES = 4;
-constexpr int BIG_TILE_BYTES = (BIG_BM + BIG_BN) * BIG_BK;  // 32 KB per K slab
 
 struct BigArgs {
     const uint8_t* __restrict__ a;   // xq [M, K]
@@ -44,6 +52,10 @@ struct BigArgs {
     int64_t ldo;
     int M, N, K;
     int a_scale_scalar;
+    // split-K (grid.z > 1): each split covers k_per_split bytes of K; see splitk.h
+    int k_per_split;
+    float* __restrict__ partials;
+    int* __restrict__ counters;
 };
 
 // One 16-byte chunk per lane from global memory straight into LDS: lane i's chunk lands at
@@ -52,6 +64,16 @@ struct BigArgs {
 __device__ __forceinline__ void copy16_to_lds(const uint8_t* base, uint32_t lane_offset, uint32_t lds_wave_base) {
     asm volatile("s_mov_b32 m0, %2\n\tglobal_load_lds_dwordx4 %0, %1"
                  :: "v"(lane_offset), "s"(base), "s"(lds_wave_base) : "memory", "m0");
+}
+
+// s_waitcnt vmcnt(N) with a compile-time N.
+template <int N>
+__device__ __forceinline__ void wait_copies() {
+    if constexpr (N == 0) asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+    else if constexpr (N == 4) asm volatile("s_waitcnt vmcnt(4)" ::: "memory");
+    else if constexpr (N == 8) asm volatile("s_waitcnt vmcnt(8)" ::: "memory");
+    else if constexpr (N == 16) asm volatile("s_waitcnt vmcnt(16)" ::: "memory");
+    else static_assert(N == 0, "unsupported copy count");
 }
 
 // Operand block of v_mfma_f32_32x32x64: lane (l32, h) reads bytes [32h, 32h+32) of its row,
@@ -67,102 +89,110 @@ __device__ __forceinline__ v8i big_frag(const uint8_t* buf, int row, int h) {
     return f;
 }
 
-template <int EPI>
-__global__ __launch_bounds__(256, 1) void gemm_fp8_big_kernel(const BigArgs p) {
+template <int TM, int TN, int EPI, bool SPLIT>
+__global__ __launch_bounds__(256) void gemm_fp8_big_kernel(const BigArgs p) {
     constexpr bool GATED = epi_is_gated(EPI);
-    __shared__ __attribute__((aligned(1024))) uint8_t lds[BIG_STAGES * BIG_TILE_BYTES];
+    constexpr int BM = 64 * TM, BN = 64 * TN;        // workgroup tile
+    constexpr int WM = 32 * TM, WN = 32 * TN;        // wavefront tile
+    constexpr int TILE_BYTES = (BM + BN) * BIG_BK;   // one K slab of A and B
+    constexpr int CA = BM / 64, CB = BN / 64;        // copy instructions per wavefront per slab
+    constexpr int COPIES = CA + CB;
+    static_assert(TM % 2 == 0 && TN % 2 == 0, "even block counts");
+
+    __shared__ __attribute__((aligned(1024))) uint8_t lds[BIG_STAGES * TILE_BYTES];
+    __shared__ int s_last;
 
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     const int wm = wave >> 1, wn = wave & 1;
     const int l32 = lane & 31, h = lane >> 5;
     const int half_n = p.N / 2;
-    const int m0 = blockIdx.y * BIG_BM;
-    const int n0 = GATED ? blockIdx.x * (BIG_BN / 2) : blockIdx.x * BIG_BN;
+    const int m0 = blockIdx.y * BM;
+    const int n0 = GATED ? blockIdx.x * (BN / 2) : blockIdx.x * BN;
 
-    // ---- copy geometry: wavefront w moves 16-row groups w*4 .. w*4+3 of A and of B ----------
+    // ---- copy geometry: wavefront w moves 16-row groups w*CA .. of A and w*CB .. of B --------
     const int crow = lane >> 2;                                   // row inside the 16-row group
     const int cchunk = ((lane & 3) ^ ((crow >> 1) & 3)) << 4;     // swizzled 16-byte chunk of that row
-    uint32_t aoff[4], boff[4];
+    uint32_t aoff[CA], boff[CB];
 #pragma unroll
-    for (int i = 0; i < 4; ++i) {
-        const int jj = (wave * 4 + i) * 16 + crow;    // row of the A tile / column of the output tile
-        int r = m0 + jj;
+    for (int i = 0; i < CA; ++i) {
+        int r = m0 + (wave * CA + i) * 16 + crow;
         r = r < p.M ? r : p.M - 1;
         aoff[i] = (uint32_t)r * (uint32_t)p.K + cchunk;
+    }
+#pragma unroll
+    for (int i = 0; i < CB; ++i) {
+        const int jj = (wave * CB + i) * 16 + crow;               // column of the output tile
         int rb;
         if constexpr (GATED) {
-            const int w_ = jj >> 7, j = jj & 127;
-            int g = n0 + w_ * 64 + (j & 63);
+            const int w_ = jj / WN, j = jj % WN;
+            int g = n0 + w_ * (WN / 2) + (j % (WN / 2));
             g = g < half_n ? g : half_n - 1;
-            rb = (j >> 6) * half_n + g;
+            rb = (j / (WN / 2)) * half_n + g;
         } else {
             rb = n0 + jj;
             rb = rb < p.N ? rb : p.N - 1;
         }
         boff[i] = (uint32_t)rb * (uint32_t)p.K + cchunk;
     }
+    const int k_begin = SPLIT ? blockIdx.z * p.k_per_split : 0;
     const uint32_t lds_base = (uint32_t)(uintptr_t)lds;
+    const uint32_t wave_a = __builtin_amdgcn_readfirstlane(lds_base + wave * (CA * 1024));
+    const uint32_t wave_b = __builtin_amdgcn_readfirstlane(lds_base + BM * BIG_BK + wave * (CB * 1024));
     auto issue = [&](int stage, int k) {
-        const uint32_t dst = __builtin_amdgcn_readfirstlane(lds_base + stage * BIG_TILE_BYTES + wave * 4096);
 #pragma unroll
-        for (int i = 0; i < 4; ++i) copy16_to_lds(p.a + k, aoff[i], dst + i * 1024);
+        for (int i = 0; i < CA; ++i) copy16_to_lds(p.a + k_begin + k, aoff[i], wave_a + stage * TILE_BYTES + i * 1024);
 #pragma unroll
-        for (int i = 0; i < 4; ++i) copy16_to_lds(p.b + k, boff[i], dst + BIG_BM * BIG_BK + i * 1024);
+        for (int i = 0; i < CB; ++i) copy16_to_lds(p.b + k_begin + k, boff[i], wave_b + stage * TILE_BYTES + i * 1024);
     };
 
-    v16f acc[4][4];
+    v16f acc[TM][TN];
 #pragma unroll
-    for (int i = 0; i < 4; ++i)
+    for (int i = 0; i < TM; ++i)
 #pragma unroll
-        for (int j = 0; j < 4; ++j)
+        for (int j = 0; j < TN; ++j)
 #pragma unroll
             for (int r = 0; r < 16; ++r) acc[i][j][r] = 0.f;
 
-    // One slab = four row groups of four MFMAs.  To keep the MFMA pipe fed across slabs:
-    //  * the barrier that publishes slab s+1 sits in the MIDDLE of slab s (after group 1), where
-    //    all wavefronts arrive at about the same time and still have MFMAs queued;
-    //  * the operand blocks that open slab s+1 (four B blocks, first A block) are read from LDS
-    //    during the last group of slab s, into a second register set.
-    const int n_slabs = p.K / BIG_BK;
-    const int arow = wm * 128 + l32, brow = wn * 128 + l32;
-    auto stage_ptr = [&](int s) -> const uint8_t* { return lds + (s % BIG_STAGES) * BIG_TILE_BYTES; };
-#define PHYAI_MFMA_GROUP(I, FA, FB0, FB1, FB2, FB3)                                                            \
-    acc[I][0] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(FA, FB0, acc[I][0], 0, 0, 0, 0, 0, 0);            \
-    acc[I][1] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(FA, FB1, acc[I][1], 0, 0, 0, 0, 0, 0);            \
-    acc[I][2] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(FA, FB2, acc[I][2], 0, 0, 0, 0, 0, 0);            \
-    acc[I][3] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(FA, FB3, acc[I][3], 0, 0, 0, 0, 0, 0);            \
+    const int n_slabs = (SPLIT ? p.k_per_split : p.K) / BIG_BK;
+    const int arow = wm * WM + l32, brow = wn * WN + l32;
+    auto stage_ptr = [&](int s) -> const uint8_t* { return lds + (s % BIG_STAGES) * TILE_BYTES; };
+
+    // Opening operand blocks of the current slab (cur) and of the next one (nxt); the two sets
+    // swap roles every slab.
+    v8i fa_cur, fa_nxt, fb_cur[TN], fb_nxt[TN];
+
+// Row group I of slab S: TN MFMAs with the A block FA against the B blocks FB[].
+#define PHYAI_MFMA_GROUP(I, FA, FB)                                                                            \
+    _Pragma("unroll") for (int j_ = 0; j_ < TN; ++j_)                                                          \
+        acc[I][j_] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(FA, FB[j_], acc[I][j_], 0, 0, 0, 0, 0, 0);  \
     __builtin_amdgcn_sched_barrier(0);
 
-// S: slab index; FA0/FB*: opening blocks of slab S (in registers); NFA0/NFB*: receive those of
+// S: slab index; FA0/FB: opening blocks of slab S (in registers); NFA0/NFB: receive those of
 // slab S+1.  NEXT: slab S+1 exists; NEXT2: slab S+2 exists (its copies may still be in flight);
 // ISSUE: slab S+3 exists and is requested here.  The flags are literals, so the steady-state
 // loop body is straight-line code.
-#define PHYAI_RUN_SLAB(S, NEXT, NEXT2, ISSUE, FA0, FB0, FB1, FB2, FB3, NFA0, NFB0, NFB1, NFB2, NFB3)               \
-    {                                                                                                             \
-        const int s_ = (S);                                                                                       \
-        const uint8_t* abuf_ = stage_ptr(s_);                                                                     \
-        const v8i fa1_ = big_frag(abuf_, arow + 32, h);                                                           \
-        PHYAI_MFMA_GROUP(0, FA0, FB0, FB1, FB2, FB3)                                                              \
-        const v8i fa2_ = big_frag(abuf_, arow + 64, h);                                                           \
-        PHYAI_MFMA_GROUP(1, fa1_, FB0, FB1, FB2, FB3)                                                             \
-        if (NEXT) {                                                                                               \
-            /* my copies of slab s+1 are done (slab s+2, if any, may still be in flight) ... */                   \
-            if (NEXT2) asm volatile("s_waitcnt vmcnt(8)" ::: "memory");                                           \
-            else asm volatile("s_waitcnt vmcnt(0)" ::: "memory");                                                 \
-            __syncthreads(); /* ... and so are everybody's; nobody reads slab s-1 any more */                      \
-            if (ISSUE) issue((s_ + BIG_STAGES - 1) % BIG_STAGES, (s_ + BIG_STAGES - 1) * BIG_BK);                 \
-        }                                                                                                         \
-        const v8i fa3_ = big_frag(abuf_, arow + 96, h);                                                           \
-        PHYAI_MFMA_GROUP(2, fa2_, FB0, FB1, FB2, FB3)                                                             \
-        if (NEXT) {                                                                                               \
-            const uint8_t* nbuf_ = stage_ptr(s_ + 1);                                                             \
-            NFB0 = big_frag(nbuf_ + BIG_BM * BIG_BK, brow, h);                                                    \
-            NFB1 = big_frag(nbuf_ + BIG_BM * BIG_BK, brow + 32, h);                                               \
-            NFB2 = big_frag(nbuf_ + BIG_BM * BIG_BK, brow + 64, h);                                               \
-            NFB3 = big_frag(nbuf_ + BIG_BM * BIG_BK, brow + 96, h);                                               \
-            NFA0 = big_frag(nbuf_, arow, h);                                                                      \
-        }                                                                                                         \
-        PHYAI_MFMA_GROUP(3, fa3_, FB0, FB1, FB2, FB3)                                                             \
+#define PHYAI_RUN_SLAB(S, NEXT, NEXT2, ISSUE, FA0, FB, NFA0, NFB)                                              \
+    {                                                                                                          \
+        const int s_ = (S);                                                                                    \
+        const uint8_t* abuf_ = stage_ptr(s_);                                                                  \
+        v8i fa_[TM];                                                                                           \
+        fa_[0] = FA0;                                                                                          \
+        _Pragma("unroll") for (int i_ = 0; i_ < TM; ++i_) {                                                    \
+            if (i_ + 1 < TM) fa_[i_ + 1] = big_frag(abuf_, arow + (i_ + 1) * 32, h);                           \
+            if (i_ == TM - 1 && NEXT) {                                                                        \
+                const uint8_t* nbuf_ = stage_ptr(s_ + 1);                                                      \
+                _Pragma("unroll") for (int j_ = 0; j_ < TN; ++j_)                                              \
+                    NFB[j_] = big_frag(nbuf_ + BM * BIG_BK, brow + j_ * 32, h);                                \
+                NFA0 = big_frag(nbuf_, arow, h);                                                               \
+            }                                                                                                  \
+            PHYAI_MFMA_GROUP(i_, fa_[i_], FB)                                                                  \
+            if (i_ == TM / 2 - 1 && NEXT) {                                                                    \
+                /* my copies of slab s+1 are done (slab s+2, if any, may still be in flight) ... */            \
+                if (NEXT2) wait_copies<COPIES>(); else wait_copies<0>();                                       \
+                __syncthreads(); /* ... and so are everybody's; nobody reads slab s-1 any more */              \
+                if (ISSUE) issue((s_ + BIG_STAGES - 1) % BIG_STAGES, (s_ + BIG_STAGES - 1) * BIG_BK);          \
+            }                                                                                                  \
+        }                                                                                                      \
     }
 
     // prologue: slabs 0..2 in flight, slab 0 published, its opening blocks in registers.
@@ -170,36 +200,53 @@ __global__ __launch_bounds__(256, 1) void gemm_fp8_big_kernel(const BigArgs p) {
     issue(0, 0);
     issue(1, BIG_BK);
     issue(2, 2 * BIG_BK);
-    asm volatile("s_waitcnt vmcnt(16)" ::: "memory");
+    wait_copies<2 * COPIES>();
     __syncthreads();
-    v8i a0, b0, b1, b2, b3, na0, nb0, nb1, nb2, nb3;
-    b0 = big_frag(lds + BIG_BM * BIG_BK, brow, h);
-    b1 = big_frag(lds + BIG_BM * BIG_BK, brow + 32, h);
-    b2 = big_frag(lds + BIG_BM * BIG_BK, brow + 64, h);
-    b3 = big_frag(lds + BIG_BM * BIG_BK, brow + 96, h);
-    a0 = big_frag(lds, arow, h);
+#pragma unroll
+    for (int j = 0; j < TN; ++j) fb_cur[j] = big_frag(lds + BM * BIG_BK, brow + j * 32, h);
+    fa_cur = big_frag(lds, arow, h);
     int s = 0;
     for (; s < n_slabs - 4; s += 2) {
-        PHYAI_RUN_SLAB(s, 1, 1, 1, a0, b0, b1, b2, b3, na0, nb0, nb1, nb2, nb3)
-        PHYAI_RUN_SLAB(s + 1, 1, 1, 1, na0, nb0, nb1, nb2, nb3, a0, b0, b1, b2, b3)
+        PHYAI_RUN_SLAB(s, 1, 1, 1, fa_cur, fb_cur, fa_nxt, fb_nxt)
+        PHYAI_RUN_SLAB(s + 1, 1, 1, 1, fa_nxt, fb_nxt, fa_cur, fb_cur)
     }
-    PHYAI_RUN_SLAB(s, 1, 1, 1, a0, b0, b1, b2, b3, na0, nb0, nb1, nb2, nb3)        // slab n-4 requests n-1
-    PHYAI_RUN_SLAB(s + 1, 1, 1, 0, na0, nb0, nb1, nb2, nb3, a0, b0, b1, b2, b3)    // slab n-3
-    PHYAI_RUN_SLAB(s + 2, 1, 0, 0, a0, b0, b1, b2, b3, na0, nb0, nb1, nb2, nb3)    // slab n-2
-    PHYAI_RUN_SLAB(s + 3, 0, 0, 0, na0, nb0, nb1, nb2, nb3, a0, b0, b1, b2, b3)    // slab n-1
+    PHYAI_RUN_SLAB(s, 1, 1, 1, fa_cur, fb_cur, fa_nxt, fb_nxt)        // slab n-4 requests slab n-1
+    PHYAI_RUN_SLAB(s + 1, 1, 1, 0, fa_nxt, fb_nxt, fa_cur, fb_cur)    // slab n-3
+    PHYAI_RUN_SLAB(s + 2, 1, 0, 0, fa_cur, fb_cur, fa_nxt, fb_nxt)    // slab n-2
+    PHYAI_RUN_SLAB(s + 3, 0, 0, 0, fa_nxt, fb_nxt, fa_cur, fb_cur)    // slab n-1
 #undef PHYAI_RUN_SLAB
 #undef PHYAI_MFMA_GROUP
 
+    // ---- split-K: publish partial sums; the last split to arrive adds them in split order --
+    if constexpr (SPLIT) {
+        constexpr int FRAG = TM * TN * 16;
+        const int S = gridDim.z;
+        const int tile = blockIdx.y * gridDim.x + blockIdx.x;
+        float frag[FRAG];
+#pragma unroll
+        for (int i = 0; i < TM; ++i)
+#pragma unroll
+            for (int j = 0; j < TN; ++j)
+#pragma unroll
+                for (int r = 0; r < 16; ++r) frag[(i * TN + j) * 16 + r] = acc[i][j][r];
+        splitk_publish<FRAG, 256>(p.partials, tile, S, blockIdx.z, frag);
+        if (!splitk_arrive(p.counters, tile, S, &s_last)) return;
+        splitk_gather<FRAG, 256>(p.partials, p.counters, tile, S, frag);
+#pragma unroll
+        for (int i = 0; i < TM; ++i)
+#pragma unroll
+            for (int j = 0; j < TN; ++j)
+#pragma unroll
+                for (int r = 0; r < 16; ++r) acc[i][j][r] = frag[(i * TN + j) * 16 + r];
+    }
+
     // ---- epilogue ------------------------------------------------------------------------
-    // The accumulator layout gives a lane one column and 16 scattered rows, which would mean
-    // 2-byte stores.  Instead each wavefront stages its bf16 output tile (128 rows x 128 or 64
-    // columns) in its own 32 KB slice of the now idle LDS and writes it out row-wise, 16 bytes
-    // per lane, whole 256- or 128-byte row segments per instruction.  Neighbouring lanes swap
-    // one value first (DPP) so that every LDS write is a packed pair of columns.
-    constexpr int TNO = GATED ? 2 : 4;
+    constexpr int TNO = GATED ? TN / 2 : TN;             // output column blocks per wavefront
     constexpr int ROWB = TNO * 64;                       // staged row length in bytes
+    constexpr int STG_BYTES = WM * ROWB;                 // per wavefront
+    static_assert(4 * STG_BYTES <= BIG_STAGES * TILE_BYTES, "staging fits in the operand LDS");
     const int n_lim = GATED ? half_n : p.N;
-    const int nbase = n0 + (GATED ? wn * 64 : wn * 128);
+    const int nbase = n0 + wn * (GATED ? WN / 2 : WN);
     float sg[TNO], bg[TNO], su[TNO], bu[TNO];
 #pragma unroll
     for (int j = 0; j < TNO; ++j) {
@@ -214,14 +261,14 @@ __global__ __launch_bounds__(256, 1) void gemm_fp8_big_kernel(const BigArgs p) {
         }
     }
     __syncthreads();  // every wavefront is done reading operands from LDS
-    uint8_t* stg = lds + wave * 32768;
+    uint8_t* stg = lds + wave * STG_BYTES;
     const int odd = lane & 1;
     // Row scales of this lane: rows mrow0 + i*32 + 8*g + (0..3), g = 0..3.
-    const int mrow0 = m0 + wm * 128 + 4 * h;
-    const bool vec_rows = !p.a_scale_scalar && m0 + BIG_BM <= p.M &&
+    const int mrow0 = m0 + wm * WM + 4 * h;
+    const bool vec_rows = !p.a_scale_scalar && m0 + BM <= p.M &&
                           (reinterpret_cast<uintptr_t>(p.a_scale) & 15) == 0;
 #pragma unroll
-    for (int i = 0; i < 4; ++i) {
+    for (int i = 0; i < TM; ++i) {
         v4f sa[4];
         if (vec_rows) {
 #pragma unroll
@@ -246,7 +293,7 @@ __global__ __launch_bounds__(256, 1) void gemm_fp8_big_kernel(const BigArgs p) {
                     const float s_a = sa[r / 4][r % 4];
                     float v = acc[i][j][r] * (s_a * sg[j]) + bg[j];
                     if constexpr (GATED) {
-                        const float u = acc[i][j + 2][r] * (s_a * su[j]) + bu[j];
+                        const float u = acc[i][j + TN / 2][r] * (s_a * su[j]) + bu[j];
                         v = apply_act<EPI>(round_bf16(v)) * round_bf16(u);
                     } else if constexpr (EPI != EPI_NONE) {
                         v = apply_act<EPI>(round_bf16(v));
@@ -264,13 +311,13 @@ __global__ __launch_bounds__(256, 1) void gemm_fp8_big_kernel(const BigArgs p) {
             }
         }
     }
-    // write the staged tile out: 1 KB (4 or 8 whole rows) per instruction
+    // write the staged tile out: 1 KB (whole rows) per instruction
 #pragma unroll 4
-    for (int qd = 0; qd < 128 * ROWB / 1024; ++qd) {
+    for (int qd = 0; qd < STG_BYTES / 1024; ++qd) {
         const int byte = qd * 1024 + lane * 16;
         const int row = byte / ROWB, colb = byte % ROWB;
         const uint4 v = *reinterpret_cast<const uint4*>(stg + byte);
-        const int m = m0 + wm * 128 + row;
+        const int m = m0 + wm * WM + row;
         const int n = nbase + (colb >> 1);
         if (m < p.M && n < n_lim) *reinterpret_cast<uint4*>(p.out + (int64_t)m * p.ldo + n) = v;
     }
@@ -280,43 +327,88 @@ __global__ __launch_bounds__(256, 1) void gemm_fp8_big_kernel(const BigArgs p) {
 
 static int big_ceil_div(int a, int b) { return (a + b - 1) / b; }
 
-// Worth it when the tile grid fills the chip at least once.
-bool big_applicable(int M, int N, int K, int epilogue) {
-    if (K % 128 != 0 || K < 256) return false;
-    if (const char* e = getenv("PHYAI_FP8_BIG")) {   // "0": never, "2": whenever the shape allows (tests)
-        if (e[0] == '0') return false;
-        if (e[0] == '2') return true;
+static int big_tiles(int M, int N, int epilogue, int bm, int bn) {
+    const bool gated = epi_is_gated(epilogue);
+    return big_ceil_div(M, bm) * big_ceil_div(gated ? N / 2 : N, gated ? bn / 2 : bn);
+}
+
+// Tile edge (256 or 128, 0 = this kernel does not apply) and K splits.  256 x 256 tiles once
+// they fill the chip; 128 x 128 tiles for problems that are still MFMA-sized but have fewer
+// tiles, and those are split along K when even the small tiles leave CUs idle: a CU can pull
+// only about 45 GB/s from L2, so a mid-sized GEMM finishes sooner on more CUs even though the
+// partial sums then make a round trip through memory.
+BigPlan big_plan(int M, int N, int K, int epilogue) {
+    BigPlan pl = {0, 1};
+    if (K % 128 != 0 || K < 256) return pl;
+    int forced = -1;
+    if (const char* e = getenv("PHYAI_FP8_BIG")) forced = atoi(e);   // "0": never; "256"/"128": force
+    if (forced == 0) return pl;
+    if (forced == 256 || forced == 128) pl.tile = forced;
+    else if (M < 128) return pl;
+    else if (big_tiles(M, N, epilogue, 256, 256) >= 200) pl.tile = 256;
+    else if (big_tiles(M, N, epilogue, 128, 128) >= 48) pl.tile = 128;
+    else return pl;
+    if (pl.tile == 128) {
+        const int tiles = big_tiles(M, N, epilogue, 128, 128);
+        // Measured at M = 816: splitting pays for K = 16384 (67 -> 49 us with two splits) and
+        // costs for K = 2048 (19 -> 25 us): the partial-sum round trip is worth about 6 us.
+        if (tiles < 200 && K >= 8192 && K % 256 == 0) pl.splits = 2;
+        if (const char* e = getenv("PHYAI_FP8_BIG_SPLITS")) {
+            const int s = atoi(e);
+            if (s >= 1 && K % (s * 128) == 0 && K / s >= 256 && tiles * s <= 4096) pl.splits = s;
+        }
     }
-    if (M < 192) return false;
-    const int n_eff = epi_is_gated(epilogue) ? N / 2 : N;
-    const int bn_eff = epi_is_gated(epilogue) ? BIG_BN / 2 : BIG_BN;
-    return big_ceil_div(M, BIG_BM) * big_ceil_div(n_eff, bn_eff) >= 200;
+    return pl;
 }
 
-template <int EPI>
-static void big_launch(const BigArgs& a, dim3 grid, hipStream_t st) {
-    hipLaunchKernelGGL((gemm_fp8_big_kernel<EPI>), grid, dim3(256), 0, st, a);
+size_t big_partial_bytes(int M, int N, int epilogue, const BigPlan& pl) {
+    if (pl.splits <= 1) return 0;
+    return (size_t)big_tiles(M, N, epilogue, 128, 128) * pl.splits * 128 * 128 * sizeof(float);
 }
 
-int launch_gemm_big(const GemmProblem& g, hipStream_t st) {
+template <int T, int EPI>
+static void big_launch(const BigArgs& a, const GemmProblem& g, int splits, hipStream_t st) {
+    const bool gated = epi_is_gated(EPI);
+    const int bn_eff = gated ? 32 * T : 64 * T;
+    const dim3 grid(big_ceil_div(gated ? g.N / 2 : g.N, bn_eff), big_ceil_div(g.M, 64 * T), splits);
+    if constexpr (T == 2) {
+        if (splits > 1) {
+            hipLaunchKernelGGL((gemm_fp8_big_kernel<T, T, EPI, true>), grid, dim3(256), 0, st, a);
+            return;
+        }
+    }
+    hipLaunchKernelGGL((gemm_fp8_big_kernel<T, T, EPI, false>), grid, dim3(256), 0, st, a);
+}
+
+template <int T>
+static int big_launch_epi(const BigArgs& a, const GemmProblem& g, int splits, hipStream_t st) {
+    switch (g.epilogue) {
+    case EPI_NONE: big_launch<T, EPI_NONE>(a, g, splits, st); return 0;
+    case EPI_GEGLU_TANH: big_launch<T, EPI_GEGLU_TANH>(a, g, splits, st); return 0;
+    case EPI_GEGLU_ERF: big_launch<T, EPI_GEGLU_ERF>(a, g, splits, st); return 0;
+    case EPI_SWIGLU: big_launch<T, EPI_SWIGLU>(a, g, splits, st); return 0;
+    case EPI_GELU_TANH: big_launch<T, EPI_GELU_TANH>(a, g, splits, st); return 0;
+    case EPI_GELU_ERF: big_launch<T, EPI_GELU_ERF>(a, g, splits, st); return 0;
+    default: return -2;
+    }
+}
+
+int launch_gemm_big(const GemmProblem& g, const BigPlan& pl, hipStream_t st) {
     // the epilogue writes 16 bytes per lane
     if (g.ldo % 8 != 0 || (reinterpret_cast<uintptr_t>(g.out) & 15) != 0) return -2;
     BigArgs a;
     a.a = g.xq; a.b = g.w; a.a_scale = g.x_scale; a.b_scale = g.w_scale; a.bias = g.bias;
     a.out = g.out; a.ldo = g.ldo; a.M = g.M; a.N = g.N; a.K = g.K;
     a.a_scale_scalar = g.x_scale_is_scalar;
-    const bool gated = epi_is_gated(g.epilogue);
-    const int n_eff = gated ? g.N / 2 : g.N;
-    const dim3 grid(big_ceil_div(n_eff, gated ? BIG_BN / 2 : BIG_BN), big_ceil_div(g.M, BIG_BM));
-    switch (g.epilogue) {
-    case EPI_NONE: big_launch<EPI_NONE>(a, grid, st); return 0;
-    case EPI_GEGLU_TANH: big_launch<EPI_GEGLU_TANH>(a, grid, st); return 0;
-    case EPI_GEGLU_ERF: big_launch<EPI_GEGLU_ERF>(a, grid, st); return 0;
-    case EPI_SWIGLU: big_launch<EPI_SWIGLU>(a, grid, st); return 0;
-    case EPI_GELU_TANH: big_launch<EPI_GELU_TANH>(a, grid, st); return 0;
-    case EPI_GELU_ERF: big_launch<EPI_GELU_ERF>(a, grid, st); return 0;
-    default: return -2;
-    }
+    a.k_per_split = g.K / pl.splits;
+    a.counters = static_cast<int*>(g.workspace);
+    a.partials = g.workspace ? reinterpret_cast<float*>(static_cast<uint8_t*>(g.workspace) + kGemmHeaderBytes) : nullptr;
+    if (pl.splits > 1 && (g.workspace == nullptr ||
+                          g.workspace_bytes < kGemmHeaderBytes + big_partial_bytes(g.M, g.N, g.epilogue, pl)))
+        return -3;
+    if (pl.tile == 256) return big_launch_epi<4>(a, g, 1, st);
+    if (pl.tile == 128) return big_launch_epi<2>(a, g, pl.splits, st);
+    return -2;
 }
 
 }  // namespace phyai

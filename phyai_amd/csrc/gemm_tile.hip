@@ -303,8 +303,14 @@ static size_t partial_bytes(const TileConfig& c, int M, int N, int epilogue) {
 size_t gemm_workspace_bytes(int64_t M, int64_t N, int64_t K, int epilogue, int64_t ldo) {
     if (M <= 0 || N <= 0 || K <= 0) return kHeaderBytes;
     if (skinny_applicable((int)M, (int)N, (int)K, epilogue, ldo)) return kHeaderBytes;
+    size_t big = 0;
+    {
+        const BigPlan bp = big_plan((int)M, (int)N, (int)K, epilogue);
+        if (bp.tile) big = big_partial_bytes((int)M, (int)N, epilogue, bp);
+    }
     const TileConfig c = pick_config((int)M, (int)N, (int)K, epilogue);
-    return kHeaderBytes + partial_bytes(c, (int)M, (int)N, epilogue);
+    const size_t own = partial_bytes(c, (int)M, (int)N, epilogue);
+    return kHeaderBytes + (own > big ? own : big);  // either kernel may end up serving the call
 }
 
 template <int BM, int BN, int WAVES_M, int WAVES_N, int EPI>
@@ -340,9 +346,12 @@ int launch_gemm(const GemmProblem& g, hipStream_t st) {
                         (reinterpret_cast<uintptr_t>(g.out) % 8 == 0);
     if (vec_ok && skinny_applicable(g.M, g.N, g.K, g.epilogue, g.ldo))
         return launch_gemm_skinny(g, skinny_plan(g.M, g.N, g.K, g.epilogue), st);
-    if (!getenv("PHYAI_FP8_TILE") && big_applicable(g.M, g.N, g.K, g.epilogue)) {
-        const int rc = launch_gemm_big(g, st);
-        if (rc != -2) return rc;  // -2: output not 16-byte addressable, take the generic tile kernel
+    if (!getenv("PHYAI_FP8_TILE")) {
+        const BigPlan bp = big_plan(g.M, g.N, g.K, g.epilogue);
+        if (bp.tile) {
+            const int rc = launch_gemm_big(g, bp, st);
+            if (rc != -2) return rc;  // -2: output not 16-byte addressable, take the generic tile kernel
+        }
     }
     const TileConfig c = pick_config(g.M, g.N, g.K, g.epilogue);
     const bool gated = epi_is_gated(g.epilogue);

@@ -48,8 +48,14 @@ bool skinny_applicable(int M, int N, int K, int epilogue, int64_t ldo);
 SkinnyPlan skinny_plan(int M, int N, int K, int epilogue);
 int launch_gemm_skinny(const GemmProblem& p, const SkinnyPlan& pl, hipStream_t st);
 
-// 256 x 256 tile kernel for large M (gemm_big.hip).  It needs no workspace.
-bool big_applicable(int M, int N, int K, int epilogue);
-int launch_gemm_big(const GemmProblem& p, hipStream_t st);
+// Pipelined tile kernel for large M (gemm_big.hip), 256 x 256 or 128 x 128 tiles; the small
+// tiles may be split along K (partials in the workspace, as for the generic tile kernel).
+struct BigPlan {
+    int tile;    // 256, 128, or 0 if the kernel does not apply
+    int splits;
+};
+BigPlan big_plan(int M, int N, int K, int epilogue);
+size_t big_partial_bytes(int M, int N, int epilogue, const BigPlan& pl);
+int launch_gemm_big(const GemmProblem& p, const BigPlan& pl, hipStream_t st);
 
 }  // namespace phyai

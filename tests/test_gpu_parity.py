@@ -333,9 +333,10 @@ def test_linear_repeatable_and_workspace_stays_clean(dev):
     (256, 256, 256, None, 0), (300, 512, 384, None, 0), (816, 768, 1024, None, 0), (513, 400, 640, "gelu", 5),
     (816, 1024, 512, "geglu_tanh", 1), (260, 288, 256, "swiglu", 3), (1000, 256, 2048, None, 0),
 ])
-def test_big_tile_kernel_forced(dev, monkeypatch, M, N, K, epi_name, epi):
+@pytest.mark.parametrize("tile", ["256", "128"])
+def test_big_tile_kernel_forced(dev, monkeypatch, tile, M, N, K, epi_name, epi):
     ops = _ops()
-    monkeypatch.setenv("PHYAI_FP8_BIG", "2")
+    monkeypatch.setenv("PHYAI_FP8_BIG", tile)
     x, wq, ws, b = _problem(M, N, K, seed=7 * M + N + K)
     got = ops.fp8_linear(x.to(dev), wq.to(dev), ws.to(dev), b.to(dev), epilogue=epi_name)
     torch.cuda.synchronize()
@@ -344,9 +345,10 @@ def test_big_tile_kernel_forced(dev, monkeypatch, M, N, K, epi_name, epi):
     assert_close_to_ref(got, want, f"big kernel {M}x{N}x{K} epi={epi_name}")
 
 
-def test_big_tile_kernel_exact_integer(dev, monkeypatch):
+@pytest.mark.parametrize("tile", ["256", "128"])
+def test_big_tile_kernel_exact_integer(dev, monkeypatch, tile):
     ops = _ops()
-    monkeypatch.setenv("PHYAI_FP8_BIG", "2")
+    monkeypatch.setenv("PHYAI_FP8_BIG", tile)
     g = torch.Generator().manual_seed(11)
     for (M, N, K) in [(256, 256, 256), (700, 528, 512), (257, 784, 1152)]:
         xi = torch.randint(-4, 5, (M, K), generator=g).float()
