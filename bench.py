@@ -48,6 +48,12 @@ PREFILL_SET = [("qkv", 2560, 2048, None), ("o", 2048, 2048, None),
                ("gate_up", 32768, 2048, "geglu_tanh"), ("down", 2048, 16384, None)]
 
 
+# HBM bytes moved by one layer's four GEMM launches at M = 50 (20.87 MB fetched + 0.87 MB written),
+# measured with rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE on `bench.py --probe` and calibrated against
+# a 64 MiB copy (profiles/expert_m50_hbm_traffic.md has the counter values).
+EXPERT_LAYER_HBM_TRAFFIC = 21_740_000
+
+
 def algorithmic_bytes(M: int, N: int, K: int, epilogue, bias: bool = False) -> int:
     """bf16 X in + fp8 W + fp32 weight scales (+ bf16 bias) + bf16 out (half width if gated)."""
     n_out = N // 2 if epilogue in ("geglu_tanh", "geglu_erf", "swiglu") else N
@@ -130,6 +136,27 @@ def gemm_only_times(dev, layers, shapes, M, reps=8, iters=30):
     return out
 
 
+def probe(dev, layers, M):
+    """Counter probe: per expert shape one GEMM launch per layer (18 distinct weight sets, so the
+    weights come from HBM), then a 64 MiB device-to-device copy whose traffic is known
+    (64 MiB read, 64 MiB written) to calibrate the counters."""
+    from phyai_amd import ops
+
+    for name, N, K, epi in EXPERT_SET:
+        pre = [(ops.fp8_quant_rowwise(layer[name]["x"]), layer[name]) for layer in layers]
+        torch.cuda.synchronize()
+        for (xq, xs), t in pre:
+            ops.fp8_gemm(xq, xs, t["w"], t["ws"], None, epilogue=t["epi"], out=t["out"])
+        torch.cuda.synchronize()
+    src = torch.empty(64 << 20, dtype=torch.uint8, device=dev).fill_(1)
+    dst = torch.empty_like(src)
+    torch.cuda.synchronize()
+    for _ in range(4):
+        dst.copy_(src)
+    torch.cuda.synchronize()
+    print("probe done")
+
+
 def cpu_baseline(layers, shapes, M, budget_s=12.0):
     """torch CPU dequantize + matmul (+ quantizer, + GeGLU) on layer 0's tensors."""
     from oracle import ref
@@ -161,6 +188,9 @@ def main() -> int:
     ap.add_argument("--warmup", type=int, default=20)
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--no-prefill", action="store_true")
+    ap.add_argument("--probe", action="store_true",
+                    help="launch each expert GEMM shape a few times plus a 64 MiB device copy and exit; "
+                         "meant to run under `rocprofv3 --pmc FETCH_SIZE` / `--pmc WRITE_SIZE`")
     args = ap.parse_args()
     if args.gpus != 1 or int(os.environ.get("WORLD_SIZE", "1")) != 1:
         print("bench.py: this path is built and measured on ONE GPU (TP=1, no collectives); "
@@ -177,6 +207,10 @@ def main() -> int:
     M, n_layers, denoise_steps = 50, 18, 10
 
     layers = make_layers(dev, EXPERT_SET, M, n_layers)
+
+    if args.probe:
+        probe(dev, layers, M)
+        return 0
 
     def chunk():
         for _ in range(denoise_steps):
@@ -197,7 +231,7 @@ def main() -> int:
     achieved = layer_bytes / (layer_us * 1e-6) / 1e9
     roofline = {
         "bound": "hbm", "achieved": round(achieved, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
-        "frac": round(achieved / HBM_PEAK_GBS, 4), "traffic": None,
+        "frac": round(achieved / HBM_PEAK_GBS, 4), "traffic": EXPERT_LAYER_HBM_TRAFFIC,
         "kernel": "gemm_fp8_skinny_kernel (M=50, four expert shapes)",
         "bytes_per_layer": layer_bytes,
         "per_shape": {name: {"us": round(per_launch_us[name], 3),
