@@ -1,4 +1,5 @@
-// Weight-streaming fp8 GEMM for at most 64 token rows (the M = 50 action-chunk regime).
+// Weight-streaming fp8 GEMM for small token counts (the M = 50 action-chunk regime, and the
+// batched M = 100 .. 400 cases where the weights still dominate the bytes).
 //
 // At these sizes a whole weight matrix (2-8 MB) is less than what the chip holds
 // in flight, so the kernel is built around latency, not throughput:
@@ -207,8 +208,16 @@ __global__ __launch_bounds__(SK_THREADS) void gemm_fp8_skinny_kernel(const Skinn
 static int sk_ceil_div(int a, int b) { return (a + b - 1) / b; }
 
 // Widths are multiples of 8 so that four consecutive output columns are valid together.
+// Largest M served here.  Every 64-row group of tokens re-reads the weight tiles from L2, so
+// beyond a few hundred rows the LDS-staged tile kernels win; the dispatcher prefers those as
+// soon as their grid is large enough (see launch_gemm) and falls back to this kernel up to here.
+static int skinny_max_m() {
+    if (const char* e = getenv("PHYAI_FP8_SKINNY_MAXM")) return atoi(e);
+    return 512;
+}
+
 bool skinny_applicable(int M, int N, int K, int epilogue, int64_t ldo) {
-    if (M > 64 || K % 128 != 0 || ldo % 4 != 0) return false;
+    if (M > skinny_max_m() || K % 128 != 0 || ldo % 4 != 0) return false;
     if (epi_is_gated(epilogue)) return (N / 2) % 8 == 0;
     return N % 8 == 0;
 }
@@ -222,20 +231,26 @@ SkinnyPlan skinny_plan(int M, int N, int K, int epilogue) {
     // two weight tiles per workgroup once that still leaves a workgroup for every CU
     pl.nt = sk_ceil_div(cols, 2 * per_tile) >= 256 ? 2 : 1;
     pl.tiles = sk_ceil_div(cols, per_tile * pl.nt);
-    // split M while there are fewer workgroups than CUs
-    pl.msplit = 1;
-    if (blocks % 2 == 0 && pl.tiles * 2 <= 256) pl.msplit = 2;
-    if (blocks % 4 == 0 && pl.tiles * 4 <= 256) pl.msplit = 4;
-    if (blocks == 3 && pl.tiles * 3 <= 256) pl.msplit = 3;
-    pl.mb = blocks / pl.msplit;
+    if (blocks <= 4) {
+        // split M while there are fewer workgroups than CUs
+        pl.msplit = 1;
+        if (blocks % 2 == 0 && pl.tiles * 2 <= 256) pl.msplit = 2;
+        if (blocks % 4 == 0 && pl.tiles * 4 <= 256) pl.msplit = 4;
+        if (blocks == 3 && pl.tiles * 3 <= 256) pl.msplit = 3;
+        pl.mb = blocks / pl.msplit;
+    } else {
+        // more than 64 rows: 64 rows per workgroup keeps the re-reads of a weight tile lowest
+        pl.mb = 4;
+        pl.msplit = sk_ceil_div(blocks, 4);
+    }
     const int steps = K / 128;
     const int per_wave = sk_ceil_div(steps, SK_WAVES);
     pl.kpw = per_wave >= 4 ? 4 : (per_wave >= 2 ? 2 : 1);
     pl.rounds = sk_ceil_div(per_wave, pl.kpw);
-    if (const char* e = getenv("PHYAI_FP8_SKINNY_PLAN")) {  // "nt,msplit" tuning override
-        int nt = 0, ms = 0;
-        if (sscanf(e, "%d,%d", &nt, &ms) == 2 && (nt == 1 || nt == 2) && ms >= 1 && blocks % ms == 0) {
-            pl.nt = nt; pl.tiles = sk_ceil_div(cols, per_tile * nt); pl.msplit = ms; pl.mb = blocks / ms;
+    if (const char* e = getenv("PHYAI_FP8_SKINNY_PLAN")) {  // "nt,mb" tuning override
+        int nt = 0, mb = 0;
+        if (sscanf(e, "%d,%d", &nt, &mb) == 2 && (nt == 1 || nt == 2) && mb >= 1 && mb <= 4) {
+            pl.nt = nt; pl.tiles = sk_ceil_div(cols, per_tile * nt); pl.mb = mb; pl.msplit = sk_ceil_div(blocks, mb);
         }
     }
     return pl;

@@ -302,7 +302,7 @@ static size_t partial_bytes(const TileConfig& c, int M, int N, int epilogue) {
 
 size_t gemm_workspace_bytes(int64_t M, int64_t N, int64_t K, int epilogue, int64_t ldo) {
     if (M <= 0 || N <= 0 || K <= 0) return kHeaderBytes;
-    if (skinny_applicable((int)M, (int)N, (int)K, epilogue, ldo)) return kHeaderBytes;
+    if (M <= 64 && skinny_applicable((int)M, (int)N, (int)K, epilogue, ldo)) return kHeaderBytes;
     size_t big = 0;
     {
         const BigPlan bp = big_plan((int)M, (int)N, (int)K, epilogue);
@@ -340,18 +340,24 @@ static int launch_epi(const TileArgs& a, const TileConfig& c, dim3 grid, hipStre
 
 int launch_gemm(const GemmProblem& g, hipStream_t st) {
     if (g.M == 0 || g.N == 0) return 0;
-    // The skinny kernel reads scales / bias / output with 128- and 64-bit accesses.
+    // Kernel choice (measured on the expert and prefill shapes):
+    //   M <= 64                      weight-streaming kernel, nothing else comes close;
+    //   pipelined tile kernel        as soon as its grid has enough tiles (big_plan);
+    //   64 < M <= 512 otherwise      weight-streaming kernel again (few output columns);
+    //   the rest                     generic LDS tile kernel (any K, any alignment).
+    // The weight-streaming kernel reads scales / bias / output with 128- and 64-bit accesses.
     const bool vec_ok = (reinterpret_cast<uintptr_t>(g.w_scale) % 16 == 0) &&
                         (reinterpret_cast<uintptr_t>(g.bias) % 8 == 0) &&
                         (reinterpret_cast<uintptr_t>(g.out) % 8 == 0);
-    if (vec_ok && skinny_applicable(g.M, g.N, g.K, g.epilogue, g.ldo))
-        return launch_gemm_skinny(g, skinny_plan(g.M, g.N, g.K, g.epilogue), st);
+    const bool skinny_ok = vec_ok && skinny_applicable(g.M, g.N, g.K, g.epilogue, g.ldo);
+    if (skinny_ok && g.M <= 64) return launch_gemm_skinny(g, skinny_plan(g.M, g.N, g.K, g.epilogue), st);
     if (!getenv("PHYAI_FP8_TILE")) {
         const BigPlan bp = big_plan(g.M, g.N, g.K, g.epilogue);
         if (bp.tile) {
             const int rc = launch_gemm_big(g, bp, st);
-            if (rc != -2) return rc;  // -2: output not 16-byte addressable, take the generic tile kernel
+            if (rc != -2) return rc;  // -2: output not 16-byte addressable, try the others
         }
+        if (skinny_ok) return launch_gemm_skinny(g, skinny_plan(g.M, g.N, g.K, g.epilogue), st);
     }
     const TileConfig c = pick_config(g.M, g.N, g.K, g.epilogue);
     const bool gated = epi_is_gated(g.epilogue);
