@@ -136,6 +136,48 @@ def gemm_only_times(dev, layers, shapes, M, reps=8, iters=30):
     return out
 
 
+def sweep(dev):
+    """Batched serving sweep (benchmark configuration 4): per (B, shape) the latency of the whole
+    quantized linear (quantizer + GEMM + epilogue, graph replay over 6 distinct weight sets) and
+    its fraction of the roofline that bounds it (HBM bytes or fp8 MFMA flops, whichever is slower)."""
+    from phyai_amd import ops
+    from phyai_amd.runtime import HipGraph
+
+    rows = []
+    for set_name, shapes, m1 in (("expert", EXPERT_SET, 50), ("prefill", PREFILL_SET, 816)):
+        for B in (1, 2, 4, 8, 16):
+            M = m1 * B
+            for name, N, K, epi in shapes:
+                g = torch.Generator(device=dev).manual_seed(B * 1000 + N)
+                items = []
+                for _ in range(6):
+                    x = torch.randn(M, K, generator=g, device=dev)
+                    idx = torch.randperm(K, generator=g, device=dev)[: K // 100]
+                    x[:, idx] *= 20.0                      # 1 % outlier channels
+                    w = (torch.randn(N, K, generator=g, device=dev) * 0.02).to(torch.bfloat16)
+                    wq, ws = ops.fp8_weight_quant(w)
+                    n_out = N // 2 if epi else N
+                    items.append((x.to(torch.bfloat16), wq, ws, torch.empty(M, n_out, dtype=torch.bfloat16, device=dev)))
+                    del w
+
+                def fn():
+                    for x, wq, ws, o in items:
+                        ops.fp8_linear(x, wq, ws, None, epilogue=epi, out=o)
+
+                gr = HipGraph()
+                gr.capture(fn, {})
+                ts, _ = time_replays(gr, 15, 3)
+                us = statistics.median(ts) * 1e3 / len(items)
+                t_hbm = algorithmic_bytes(M, N, K, epi) / (HBM_PEAK_GBS * 1e9) * 1e6
+                t_mfma = 2.0 * M * N * K / (FP8_PEAK_TFLOPS * 1e12) * 1e6
+                rows.append({"set": set_name, "B": B, "M": M, "shape": name, "us": round(us, 2),
+                             "bound": "hbm" if t_hbm >= t_mfma else "mfma",
+                             "roofline_us": round(max(t_hbm, t_mfma), 3),
+                             "frac": round(max(t_hbm, t_mfma) / us, 4)})
+                del items, gr
+    return rows
+
+
 def probe(dev, layers, M):
     """Counter probe: per expert shape one GEMM launch per layer (18 distinct weight sets, so the
     weights come from HBM), then a 64 MiB device-to-device copy whose traffic is known
@@ -188,6 +230,8 @@ def main() -> int:
     ap.add_argument("--warmup", type=int, default=20)
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--no-prefill", action="store_true")
+    ap.add_argument("--sweep", action="store_true",
+                    help="also time the batched-serving sweep (B = 1..16, both linear sets, outlier channels)")
     ap.add_argument("--probe", action="store_true",
                     help="launch each expert GEMM shape a few times plus a 64 MiB device copy and exit; "
                          "meant to run under `rocprofv3 --pmc FETCH_SIZE` / `--pmc WRITE_SIZE`")
@@ -253,6 +297,8 @@ def main() -> int:
                                  "TFLOP/s": round(flops / (p_layer_us * 1e-6) / 1e12, 1),
                                  "frac_fp8_peak": round(flops / (p_layer_us * 1e-6) / 1e12 / FP8_PEAK_TFLOPS, 4)}
         del pl, pg
+    if args.sweep:
+        extra["batched_sweep"] = sweep(dev)
 
     cpu = None
     if not args.no_cpu_baseline:

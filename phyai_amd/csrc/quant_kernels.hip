@@ -42,19 +42,56 @@ __device__ __forceinline__ uint32_t absmax8(uint4 q, uint32_t m) {
     return m;
 }
 
+// Divisor of one row.  The reference divides every element by the row scale with an IEEE fp32
+// division.  For a finite scale the same quotient bits come from a multiplication by the
+// (correctly rounded) reciprocal followed by one residual correction,
+//     q0 = x * r;   q = fma(fma(-q0, s, x), r, q0),
+// which is exact whenever the true quotient is representable and within one ulp otherwise.
+// Both operands are bf16 values (8 significant bits), so a quotient is either exactly on an
+// e4m3 rounding boundary or at least 2^-13 (relative) away from it, far more than an ulp: the
+// codes are identical to those of the true division.  This is verified exhaustively on the
+// device over every finite bf16 value against every possible scale.  Rows with a non-finite
+// scale (an Inf or NaN in the row) take the true division.
+struct RowDivisor {
+    float s, r;
+    bool fast;
+};
+__device__ __forceinline__ RowDivisor make_divisor(float s) {
+    RowDivisor d;
+    d.s = s;
+    d.fast = (__float_as_uint(s) & 0x7FFFFFFFu) < 0x7F800000u;
+    d.r = 1.0f / s;
+    return d;
+}
+__device__ __forceinline__ float div_exact(float x, const RowDivisor& d) {
+    const float q0 = x * d.r;
+    const float q = __builtin_fmaf(__builtin_fmaf(-q0, d.s, x), d.r, q0);
+    return __builtin_copysignf(q, x);  // the scale is positive; keeps -0 -> -0 (the sum above gives +0)
+}
+
 template <int MODE>
-__device__ __forceinline__ uint2 encode8(uint4 q, float s) {
+__device__ __forceinline__ uint2 encode8(uint4 q, const RowDivisor& d) {
     const uint32_t w[4] = {q.x, q.y, q.z, q.w};
     uint32_t c[4];
+    if (MODE == QUANT_ACT_DYNAMIC && d.fast) {
+        // every |x| <= amax is finite, so |x / s| < 464: the hardware convert needs no guard
 #pragma unroll
-    for (int i = 0; i < 4; ++i) {
-        float a = bf16_bits_to_f32(w[i] & 0xFFFFu) / s;
-        float b = bf16_bits_to_f32(w[i] >> 16) / s;
-        if constexpr (MODE == QUANT_WEIGHT) {
-            a = fminf(fmaxf(a, -kFp8Max), kFp8Max);
-            b = fminf(fmaxf(b, -kFp8Max), kFp8Max);
+        for (int i = 0; i < 4; ++i) {
+            const float a = div_exact(bf16_bits_to_f32(w[i] & 0xFFFFu), d);
+            const float b = div_exact(bf16_bits_to_f32(w[i] >> 16), d);
+            c[i] = (uint32_t)__builtin_amdgcn_cvt_pk_fp8_f32(a, b, 0, false) & 0xFFFFu;
         }
-        c[i] = e4m3_pack2(a, b);
+    } else {
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+            float a = bf16_bits_to_f32(w[i] & 0xFFFFu) / d.s;
+            float b = bf16_bits_to_f32(w[i] >> 16) / d.s;
+            if constexpr (MODE == QUANT_WEIGHT) {
+                a = fminf(fmaxf(a, -kFp8Max), kFp8Max);
+                b = fminf(fmaxf(b, -kFp8Max), kFp8Max);
+            }
+            c[i] = e4m3_pack2(a, b);
+        }
     }
     return make_uint2(c[0] | (c[1] << 16), c[2] | (c[3] << 16));
 }
@@ -92,11 +129,12 @@ __global__ __launch_bounds__(THREADS) void quant_rows_reg_kernel(
     m = block_max_u32<THREADS>(m, smem);
     const float s = scale_from_amax_bits<MODE>(m);
     if (threadIdx.x == 0) scale[row] = s;
+    const RowDivisor d = make_divisor(s);
     uint8_t* qr = xq + row * (int64_t)K;
 #pragma unroll
     for (int c = 0; c < CHUNKS; ++c) {
         const int k = (c * THREADS + threadIdx.x) * 8;
-        if (k < K) *reinterpret_cast<uint2*>(qr + k) = encode8<MODE>(v[c], s);
+        if (k < K) *reinterpret_cast<uint2*>(qr + k) = encode8<MODE>(v[c], d);
     }
 }
 
@@ -115,9 +153,10 @@ __global__ __launch_bounds__(256) void quant_rows_loop_kernel(
     m = block_max_u32<256>(m, smem);
     const float s = scale_from_amax_bits<MODE>(m);
     if (threadIdx.x == 0) scale[row] = s;
+    const RowDivisor d = make_divisor(s);
     uint8_t* qr = xq + row * (int64_t)K;
     for (int k = threadIdx.x * 8; k < K; k += 256 * 8)
-        *reinterpret_cast<uint2*>(qr + k) = encode8<MODE>(*reinterpret_cast<const uint4*>(xr + k), s);
+        *reinterpret_cast<uint2*>(qr + k) = encode8<MODE>(*reinterpret_cast<const uint4*>(xr + k), d);
 }
 
 // Static per-tensor quantizer: clamp(fp32(x)/s, +-448) -> e4m3fn.  torch.clamp

@@ -357,3 +357,33 @@ def test_big_tile_kernel_exact_integer(dev, monkeypatch, tile):
                            wi.to(torch.float8_e4m3fn).to(dev), torch.full((N,), 0.25, device=dev))
         want = ((xi @ wi.t()) * 0.125).bfloat16()
         assert torch.equal(got.cpu(), want), f"{(M, N, K)}"
+
+
+def test_quant_rowwise_exhaustive_all_values_all_scales(dev):
+    """Every finite bf16 value against every possible row maximum (32 640 of them, hence every
+    possible scale): 2.1e9 quotients.  The expected codes are the reference's own expression
+    evaluated with torch on the device (IEEE fp32 division, torch's e4m3fn cast), which the
+    sampled tests above tie to the CPU oracle."""
+    ops = _ops()
+    allbits = torch.arange(0, 1 << 16, dtype=torch.int32, device=dev)
+    finite = allbits[(allbits & 0x7F80) != 0x7F80].to(torch.uint16)
+    vals = finite.view(torch.bfloat16)                       # 65 280 finite values
+    absbits = (finite.to(torch.int32) & 0x7FFF)
+    amax_bits = torch.arange(0, 0x7F80, dtype=torch.int32, device=dev)     # every non-negative finite bf16
+    K = 65536
+    chunk = 128
+    for start in range(0, amax_bits.numel(), chunk):
+        a = amax_bits[start:start + chunk]
+        x = torch.zeros((a.numel(), K), dtype=torch.bfloat16, device=dev)
+        keep = absbits[None, :] <= a[:, None]                 # values not larger than this row's maximum
+        x[:, : vals.numel()] = torch.where(keep, vals[None, :], torch.zeros((), dtype=torch.bfloat16, device=dev))
+        x[:, -1] = a.to(torch.uint16).view(torch.bfloat16)    # make sure the maximum itself is present
+        q, s = ops.fp8_quant_rowwise(x)
+        wq, ws = ref.quant_rowwise(x)                         # torch ops on the device
+        assert torch.equal(s, ws), f"scales differ for amax bits {start}..{start + chunk}"
+        same = q.view(torch.uint8) == wq.view(torch.uint8)
+        if not bool(same.all()):
+            r, c = torch.nonzero(~same)[0].tolist()
+            raise AssertionError(
+                f"amax bits {int(a[r]):#06x}, x bits {int(x[r, c].view(torch.uint16)):#06x}: "
+                f"got {int(q.view(torch.uint8)[r, c]):#04x} want {int(wq.view(torch.uint8)[r, c]):#04x}")
