@@ -16,11 +16,13 @@
 //    wavefront fetches one 16-byte chunk and the hardware deposits chunk i at LDS base + 16*i.
 //    The XOR swizzle that keeps the 128-bit operand reads conflict-free is therefore applied
 //    on the global side: lane i (row i/4 of a 16-row group, slot i%4 of the 64-byte row)
-//    fetches chunk (i%4) ^ ((row/2)%4) of its row.
+//    fetches chunk (i%4) ^ swizzle(row) of its row.
 //  * K is consumed in 64-byte slabs through a ring of four LDS stages: the copies of slab s+3
-//    are issued while slab s is being multiplied.  One barrier per slab, placed in the MIDDLE
-//    of slab s: it publishes slab s+1 and tells everyone that the stage about to be refilled
-//    is no longer read.  All wavefronts reach it at about the same time, with MFMAs queued.
+//    are requested while slabs s and s+1 are being multiplied, one copy instruction after every
+//    second MFMA, so the wavefront never waits on the memory pipeline's issue queue with its
+//    MFMA pipe empty.  One barrier per slab, placed in the MIDDLE of slab s: it publishes slab
+//    s+1 and tells everyone that the stage about to be refilled is no longer read.  All
+//    wavefronts reach it at about the same time, with MFMAs queued.
 //  * the operand blocks that open slab s+1 are read from LDS during the last row group of
 //    slab s into a second register set, and inside a slab the A block of the next row group is
 //    read before the current group's MFMAs are issued, so ds_read latency overlaps MFMA time.
@@ -31,7 +33,8 @@
 //
 // Gated epilogues: within a wavefront's 32*TN columns the first half are gate columns and the
 // second half the matching up columns, so the pair sits in the same lane of two accumulators.
-// Requires K % 128 == 0 and K >= 256 (slabs are never partial and come in pairs).
+// Requires K % 128 == 0 and K >= 512 per split (slabs are never partial, come in pairs, and
+// must fill the ring).
 #include "fp8_device.h"
 #include "launch.h"
 #include "splitk.h"
@@ -40,7 +43,6 @@
 namespace phyai {
 
 constexpr int BIG_BK = 64;
-constexpr int BIG_STAGES = 4;
 
 struct BigArgs {
     const uint8_t* __restrict__ a;   // xq [M, K]
@@ -66,23 +68,27 @@ __device__ __forceinline__ void copy16_to_lds(const uint8_t* base, uint32_t lane
                  :: "v"(lane_offset), "s"(base), "s"(lds_wave_base) : "memory", "m0");
 }
 
-// s_waitcnt vmcnt(N) with a compile-time N.
+// s_waitcnt vmcnt(N) with a compile-time N: at most N of this wavefront's copies still in flight.
 template <int N>
 __device__ __forceinline__ void wait_copies() {
-    if constexpr (N == 0) asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
-    else if constexpr (N == 4) asm volatile("s_waitcnt vmcnt(4)" ::: "memory");
-    else if constexpr (N == 8) asm volatile("s_waitcnt vmcnt(8)" ::: "memory");
-    else if constexpr (N == 16) asm volatile("s_waitcnt vmcnt(16)" ::: "memory");
-    else static_assert(N == 0, "unsupported copy count");
+    static_assert(N >= 0 && N < 64, "vmcnt is a 6-bit counter");
+    asm volatile("s_waitcnt vmcnt(%0)" ::"n"(N) : "memory");
 }
 
-// Operand block of v_mfma_f32_32x32x64: lane (l32, h) reads bytes [32h, 32h+32) of its row,
-// i.e. chunks 2h and 2h+1, from their swizzled places.
+// Swizzle of the 16-byte chunks of a 64-byte row.  LDS has 64 banks of 4 bytes, so one pass over
+// the banks spans four rows and a 128-bit read is served 16 lanes at a time: rows r, r+4, r+8,
+// r+12 must land in different chunk columns (bit 3 of the row folded in), and so must rows
+// r, r+2, r+4, r+6 (narrower grouping).
+__device__ __forceinline__ int big_swizzle(int row) { return ((row >> 1) & 3) ^ ((row >> 3) & 1); }
+
+// Operand block of v_mfma_f32_32x32x64: lane (l32, h) supplies 32 of the 64 K-bytes of its row.
+// Which 32 is free as long as A and B agree; chunks h and 2+h are taken so that the two halves of
+// a wavefront never meet in a chunk column either.
 __device__ __forceinline__ v8i big_frag(const uint8_t* buf, int row, int h) {
-    const int sw = (row >> 1) & 3;
+    const int sw = big_swizzle(row);
     const uint8_t* r = buf + row * BIG_BK;
-    const v4i lo = *reinterpret_cast<const v4i*>(r + (((2 * h) ^ sw) << 4));
-    const v4i hi = *reinterpret_cast<const v4i*>(r + (((2 * h + 1) ^ sw) << 4));
+    const v4i lo = *reinterpret_cast<const v4i*>(r + ((h ^ sw) << 4));
+    const v4i hi = *reinterpret_cast<const v4i*>(r + (((2 + h) ^ sw) << 4));
     v8i f;
     f[0] = lo[0]; f[1] = lo[1]; f[2] = lo[2]; f[3] = lo[3];
     f[4] = hi[0]; f[5] = hi[1]; f[6] = hi[2]; f[7] = hi[3];
@@ -97,9 +103,9 @@ __global__ __launch_bounds__(256) void gemm_fp8_big_kernel(const BigArgs p) {
     constexpr int TILE_BYTES = (BM + BN) * BIG_BK;   // one K slab of A and B
     constexpr int CA = BM / 64, CB = BN / 64;        // copy instructions per wavefront per slab
     constexpr int COPIES = CA + CB;
-    static_assert(TM % 2 == 0 && TN % 2 == 0, "even block counts");
-
-    __shared__ __attribute__((aligned(1024))) uint8_t lds[BIG_STAGES * TILE_BYTES];
+    constexpr int STAGES = 4;                        // depth of the LDS ring
+    static_assert(TM == TN && TM % 2 == 0, "square wavefront tile, even block count");
+    __shared__ __attribute__((aligned(1024))) uint8_t lds[STAGES * TILE_BYTES];
     __shared__ int s_last;
 
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
@@ -111,7 +117,7 @@ __global__ __launch_bounds__(256) void gemm_fp8_big_kernel(const BigArgs p) {
 
     // ---- copy geometry: wavefront w moves 16-row groups w*CA .. of A and w*CB .. of B --------
     const int crow = lane >> 2;                                   // row inside the 16-row group
-    const int cchunk = ((lane & 3) ^ ((crow >> 1) & 3)) << 4;     // swizzled 16-byte chunk of that row
+    const int cchunk = ((lane & 3) ^ big_swizzle(crow)) << 4;      // swizzled 16-byte chunk of that row
     uint32_t aoff[CA], boff[CB];
 #pragma unroll
     for (int i = 0; i < CA; ++i) {
@@ -138,11 +144,12 @@ __global__ __launch_bounds__(256) void gemm_fp8_big_kernel(const BigArgs p) {
     const uint32_t lds_base = (uint32_t)(uintptr_t)lds;
     const uint32_t wave_a = __builtin_amdgcn_readfirstlane(lds_base + wave * (CA * 1024));
     const uint32_t wave_b = __builtin_amdgcn_readfirstlane(lds_base + BM * BIG_BK + wave * (CB * 1024));
-    auto issue = [&](int stage, int k) {
-#pragma unroll
-        for (int i = 0; i < CA; ++i) copy16_to_lds(p.a + k_begin + k, aoff[i], wave_a + stage * TILE_BYTES + i * 1024);
-#pragma unroll
-        for (int i = 0; i < CB; ++i) copy16_to_lds(p.b + k_begin + k, boff[i], wave_b + stage * TILE_BYTES + i * 1024);
+    // copy c (0 .. COPIES-1) of this wavefront's share of slab `slab`
+    auto issue = [&](int slab, int c) {
+        const int k = k_begin + slab * BIG_BK;
+        const uint32_t stage_off = (slab % STAGES) * TILE_BYTES;
+        if (c < CA) copy16_to_lds(p.a + k, aoff[c], wave_a + stage_off + c * 1024);
+        else copy16_to_lds(p.b + k, boff[c - CA], wave_b + stage_off + (c - CA) * 1024);
     };
 
     v16f acc[TM][TN];
@@ -155,23 +162,20 @@ __global__ __launch_bounds__(256) void gemm_fp8_big_kernel(const BigArgs p) {
 
     const int n_slabs = (SPLIT ? p.k_per_split : p.K) / BIG_BK;
     const int arow = wm * WM + l32, brow = wn * WN + l32;
-    auto stage_ptr = [&](int s) -> const uint8_t* { return lds + (s % BIG_STAGES) * TILE_BYTES; };
+    auto stage_ptr = [&](int s) -> const uint8_t* { return lds + (s % STAGES) * TILE_BYTES; };
 
     // Opening operand blocks of the current slab (cur) and of the next one (nxt); the two sets
     // swap roles every slab.
     v8i fa_cur, fa_nxt, fb_cur[TN], fb_nxt[TN];
 
-// Row group I of slab S: TN MFMAs with the A block FA against the B blocks FB[].
-#define PHYAI_MFMA_GROUP(I, FA, FB)                                                                            \
-    _Pragma("unroll") for (int j_ = 0; j_ < TN; ++j_)                                                          \
-        acc[I][j_] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(FA, FB[j_], acc[I][j_], 0, 0, 0, 0, 0, 0);  \
-    __builtin_amdgcn_sched_barrier(0);
-
 // S: slab index; FA0/FB: opening blocks of slab S (in registers); NFA0/NFB: receive those of
-// slab S+1.  NEXT: slab S+1 exists; NEXT2: slab S+2 exists (its copies may still be in flight);
-// ISSUE: slab S+3 exists and is requested here.  The flags are literals, so the steady-state
-// loop body is straight-line code.
-#define PHYAI_RUN_SLAB(S, NEXT, NEXT2, ISSUE, FA0, FB, NFA0, NFB)                                              \
+// slab S+1.  NEXT: slab S+1 exists; AHEAD: how many slabs beyond S+1 may still be in flight when
+// S+1 is needed.  Copies are issued one at a time between MFMAs - a wavefront that queues all of
+// a slab's copies at once sits in the memory pipeline's issue queue while its MFMA pipe runs dry:
+// the row groups after the barrier request the first half of slab S+STAGES-1 (ISSUE), the row
+// groups before it the second half of slab S+STAGES-2 (ISSUE_P), whose stage the previous
+// barrier released.  All flags are literals, so the steady-state loop body is straight-line code.
+#define PHYAI_RUN_SLAB(S, NEXT, AHEAD, ISSUE_P, ISSUE, FA0, FB, NFA0, NFB)                                     \
     {                                                                                                          \
         const int s_ = (S);                                                                                    \
         const uint8_t* abuf_ = stage_ptr(s_);                                                                  \
@@ -185,37 +189,54 @@ __global__ __launch_bounds__(256) void gemm_fp8_big_kernel(const BigArgs p) {
                     NFB[j_] = big_frag(nbuf_ + BM * BIG_BK, brow + j_ * 32, h);                                \
                 NFA0 = big_frag(nbuf_, arow, h);                                                               \
             }                                                                                                  \
-            PHYAI_MFMA_GROUP(i_, fa_[i_], FB)                                                                  \
+            const bool before_ = i_ < TM / 2;                                                                  \
+            const bool req_ = before_ ? (ISSUE_P) : (ISSUE);                                                   \
+            const int slab_ = before_ ? s_ + STAGES - 2 : s_ + STAGES - 1;                                     \
+            const int c0_ = before_ ? COPIES / 2 + i_ * 2 : (i_ - TM / 2) * 2;                                 \
+            _Pragma("unroll") for (int j_ = 0; j_ < TN; ++j_) {                                                \
+                acc[i_][j_] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(fa_[i_], FB[j_], acc[i_][j_],    \
+                                                                               0, 0, 0, 0, 0, 0);              \
+                if (req_ && j_ % (TN / 2) == TN / 2 - 1) issue(slab_, c0_ + j_ / (TN / 2));                    \
+                __builtin_amdgcn_sched_barrier(0);                                                             \
+            }                                                                                                  \
             if (i_ == TM / 2 - 1 && NEXT) {                                                                    \
-                /* my copies of slab s+1 are done (slab s+2, if any, may still be in flight) ... */            \
-                if (NEXT2) wait_copies<COPIES>(); else wait_copies<0>();                                       \
+                wait_copies<COPIES * (AHEAD)>(); /* my copies of slab s+1 are done ... */                      \
                 __syncthreads(); /* ... and so are everybody's; nobody reads slab s-1 any more */              \
-                if (ISSUE) issue((s_ + BIG_STAGES - 1) % BIG_STAGES, (s_ + BIG_STAGES - 1) * BIG_BK);          \
             }                                                                                                  \
         }                                                                                                      \
     }
+#define PHYAI_SLAB_A(S, NEXT, AHEAD, ISSUE_P, ISSUE) \
+    PHYAI_RUN_SLAB(S, NEXT, AHEAD, ISSUE_P, ISSUE, fa_cur, fb_cur, fa_nxt, fb_nxt)
+#define PHYAI_SLAB_B(S, NEXT, AHEAD, ISSUE_P, ISSUE) \
+    PHYAI_RUN_SLAB(S, NEXT, AHEAD, ISSUE_P, ISSUE, fa_nxt, fb_nxt, fa_cur, fb_cur)
 
-    // prologue: slabs 0..2 in flight, slab 0 published, its opening blocks in registers.
-    // n_slabs is even and at least 4 (K is a multiple of 128 and at least 256).
-    issue(0, 0);
-    issue(1, BIG_BK);
-    issue(2, 2 * BIG_BK);
-    wait_copies<2 * COPIES>();
+    // prologue: slabs 0 .. STAGES-3 and the first half of slab STAGES-2 in flight, slab 0
+    // published, its opening blocks in registers.  n_slabs is even and at least 2*STAGES (checked
+    // on the host).
+#pragma unroll
+    for (int i = 0; i < STAGES - 2; ++i)
+#pragma unroll
+        for (int c = 0; c < COPIES; ++c) issue(i, c);
+#pragma unroll
+    for (int c = 0; c < COPIES / 2; ++c) issue(STAGES - 2, c);
+    wait_copies<COPIES * (STAGES - 3) + COPIES / 2>();
     __syncthreads();
 #pragma unroll
     for (int j = 0; j < TN; ++j) fb_cur[j] = big_frag(lds + BM * BIG_BK, brow + j * 32, h);
     fa_cur = big_frag(lds, arow, h);
     int s = 0;
-    for (; s < n_slabs - 4; s += 2) {
-        PHYAI_RUN_SLAB(s, 1, 1, 1, fa_cur, fb_cur, fa_nxt, fb_nxt)
-        PHYAI_RUN_SLAB(s + 1, 1, 1, 1, fa_nxt, fb_nxt, fa_cur, fb_cur)
+    for (; s < n_slabs - STAGES; s += 2) {          // both slabs of the pair still request new slabs
+        PHYAI_SLAB_A(s, 1, STAGES - 3, 1, 1)
+        PHYAI_SLAB_B(s + 1, 1, STAGES - 3, 1, 1)
     }
-    PHYAI_RUN_SLAB(s, 1, 1, 1, fa_cur, fb_cur, fa_nxt, fb_nxt)        // slab n-4 requests slab n-1
-    PHYAI_RUN_SLAB(s + 1, 1, 1, 0, fa_nxt, fb_nxt, fa_cur, fb_cur)    // slab n-3
-    PHYAI_RUN_SLAB(s + 2, 1, 0, 0, fa_cur, fb_cur, fa_nxt, fb_nxt)    // slab n-2
-    PHYAI_RUN_SLAB(s + 3, 0, 0, 0, fa_nxt, fb_nxt, fa_cur, fb_cur)    // slab n-1
+    // s == n_slabs - STAGES: the last requests, then the ring drains
+    PHYAI_SLAB_A(s, 1, 1, 1, 1)
+    PHYAI_SLAB_B(s + 1, 1, 1, 1, 0)
+    PHYAI_SLAB_A(s + 2, 1, 0, 0, 0)
+    PHYAI_SLAB_B(s + 3, 0, 0, 0, 0)
+#undef PHYAI_SLAB_A
+#undef PHYAI_SLAB_B
 #undef PHYAI_RUN_SLAB
-#undef PHYAI_MFMA_GROUP
 
     // ---- split-K: publish partial sums; the last split to arrive adds them in split order --
     if constexpr (SPLIT) {
@@ -244,7 +265,7 @@ __global__ __launch_bounds__(256) void gemm_fp8_big_kernel(const BigArgs p) {
     constexpr int TNO = GATED ? TN / 2 : TN;             // output column blocks per wavefront
     constexpr int ROWB = TNO * 64;                       // staged row length in bytes
     constexpr int STG_BYTES = WM * ROWB;                 // per wavefront
-    static_assert(4 * STG_BYTES <= BIG_STAGES * TILE_BYTES, "staging fits in the operand LDS");
+    static_assert(4 * STG_BYTES <= STAGES * TILE_BYTES, "staging fits in the operand LDS");
     const int n_lim = GATED ? half_n : p.N;
     const int nbase = n0 + wn * (GATED ? WN / 2 : WN);
     float sg[TNO], bg[TNO], su[TNO], bu[TNO];
@@ -339,7 +360,7 @@ static int big_tiles(int M, int N, int epilogue, int bm, int bn) {
 // partial sums then make a round trip through memory.
 BigPlan big_plan(int M, int N, int K, int epilogue) {
     BigPlan pl = {0, 1};
-    if (K % 128 != 0 || K < 256) return pl;
+    if (K % 128 != 0 || K < 512) return pl;   // slabs come in pairs and must fill the ring
     int forced = -1;
     if (const char* e = getenv("PHYAI_FP8_BIG")) forced = atoi(e);   // "0": never; "256"/"128": force
     if (forced == 0) return pl;
@@ -355,7 +376,7 @@ BigPlan big_plan(int M, int N, int K, int epilogue) {
         if (tiles < 200 && K >= 8192 && K % 256 == 0) pl.splits = 2;
         if (const char* e = getenv("PHYAI_FP8_BIG_SPLITS")) {
             const int s = atoi(e);
-            if (s >= 1 && K % (s * 128) == 0 && K / s >= 256 && tiles * s <= 4096) pl.splits = s;
+            if (s >= 1 && K % (s * 128) == 0 && K / s >= 512 && tiles * s <= 4096) pl.splits = s;
         }
     }
     return pl;
@@ -372,12 +393,11 @@ static void big_launch(const BigArgs& a, const GemmProblem& g, int splits, hipSt
     const int bn_eff = gated ? 32 * T : 64 * T;
     const dim3 grid(big_ceil_div(gated ? g.N / 2 : g.N, bn_eff), big_ceil_div(g.M, 64 * T), splits);
     if constexpr (T == 2) {
-        if (splits > 1) {
-            hipLaunchKernelGGL((gemm_fp8_big_kernel<T, T, EPI, true>), grid, dim3(256), 0, st, a);
-            return;
-        }
+        if (splits > 1) hipLaunchKernelGGL((gemm_fp8_big_kernel<2, 2, EPI, true>), grid, dim3(256), 0, st, a);
+        else hipLaunchKernelGGL((gemm_fp8_big_kernel<2, 2, EPI, false>), grid, dim3(256), 0, st, a);
+    } else {
+        hipLaunchKernelGGL((gemm_fp8_big_kernel<4, 4, EPI, false>), grid, dim3(256), 0, st, a);
     }
-    hipLaunchKernelGGL((gemm_fp8_big_kernel<T, T, EPI, false>), grid, dim3(256), 0, st, a);
 }
 
 template <int T>

@@ -330,8 +330,8 @@ def test_linear_repeatable_and_workspace_stays_clean(dev):
 # ---------------------------------------------------------------------------
 
 @pytest.mark.parametrize("M,N,K,epi_name,epi", [
-    (256, 256, 256, None, 0), (300, 512, 384, None, 0), (816, 768, 1024, None, 0), (513, 400, 640, "gelu", 5),
-    (816, 1024, 512, "geglu_tanh", 1), (260, 288, 256, "swiglu", 3), (1000, 256, 2048, None, 0),
+    (256, 256, 1024, None, 0), (300, 512, 1280, None, 0), (816, 768, 1024, None, 0), (513, 400, 1536, "gelu", 5),
+    (816, 1024, 1152, "geglu_tanh", 1), (260, 288, 1024, "swiglu", 3), (1000, 256, 2048, None, 0),
 ])
 @pytest.mark.parametrize("tile", ["256", "128"])
 def test_big_tile_kernel_forced(dev, monkeypatch, tile, M, N, K, epi_name, epi):
@@ -350,13 +350,33 @@ def test_big_tile_kernel_exact_integer(dev, monkeypatch, tile):
     ops = _ops()
     monkeypatch.setenv("PHYAI_FP8_BIG", tile)
     g = torch.Generator().manual_seed(11)
-    for (M, N, K) in [(256, 256, 256), (700, 528, 512), (257, 784, 1152)]:
+    for (M, N, K) in [(256, 256, 1024), (700, 528, 1280), (257, 784, 1152)]:
         xi = torch.randint(-4, 5, (M, K), generator=g).float()
         wi = torch.randint(-4, 5, (N, K), generator=g).float()
         got = ops.fp8_gemm(xi.to(torch.float8_e4m3fn).to(dev), torch.full((M, 1), 0.5, device=dev),
                            wi.to(torch.float8_e4m3fn).to(dev), torch.full((N,), 0.25, device=dev))
         want = ((xi @ wi.t()) * 0.125).bfloat16()
         assert torch.equal(got.cpu(), want), f"{(M, N, K)}"
+
+
+def test_big_tile_kernel_split_k(dev, monkeypatch):
+    """128 x 128 tiles with the K range split over two and four workgroups (partials in the workspace)."""
+    ops = _ops()
+    monkeypatch.setenv("PHYAI_FP8_BIG", "128")
+    x, wq, ws, b = _problem(300, 384, 4096, seed=77)
+    xq, xs = ref.quant_rowwise(x)
+    want = ref.gemm_f32(xq, xs, wq, ws, b)
+    outs = []
+    for splits in ("1", "2", "4"):
+        monkeypatch.setenv("PHYAI_FP8_BIG_SPLITS", splits)
+        got = ops.fp8_linear(x.to(dev), wq.to(dev), ws.to(dev), b.to(dev))
+        torch.cuda.synchronize()
+        assert_close_to_ref(got, want, f"split-K {splits}")
+        again = ops.fp8_linear(x.to(dev), wq.to(dev), ws.to(dev), b.to(dev))
+        assert torch.equal(got, again), "split-K result must not depend on arrival order"
+        outs.append(got)
+    for w in ops._workspaces.values():
+        assert int(w[: ops.WORKSPACE_HEADER_BYTES].max().item()) == 0
 
 
 def test_quant_rowwise_exhaustive_all_values_all_scales(dev):
