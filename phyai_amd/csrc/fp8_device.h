@@ -25,6 +25,14 @@ __device__ __forceinline__ uint32_t f32_to_bf16_bits(float f) {
     return (f != f) ? 0x7FC0u : r;
 }
 
+// Two fp32 -> two bf16 (round to nearest even) packed as lo | hi << 16, one v_cvt_pk_bf16_f32.
+typedef __bf16 bf16x2_t __attribute__((ext_vector_type(2)));
+typedef float f32x2_t __attribute__((ext_vector_type(2)));
+__device__ __forceinline__ uint32_t pack_bf16x2(float lo, float hi) {
+    const f32x2_t v = {lo, hi};
+    return __builtin_bit_cast(uint32_t, __builtin_convertvector(v, bf16x2_t));
+}
+
 // Two fp32 -> two e4m3fn codes (OCP, round to nearest even) in the low 16 bits.
 // The hardware convert is used for the in-range part; values at or beyond 480
 // and NaN take the NaN code with the input's sign, which is what a software
@@ -47,12 +55,14 @@ __device__ __forceinline__ uint32_t wave_max_u32(uint32_t v) {
 }
 
 // ---- epilogue activations (fp32 math) ------------------------------------
+// gelu_tanh(v) = 0.5 v (1 + tanh u), u = k0 (v + k1 v^3).  With tanh u = 1 - 2 / (exp(2u) + 1) this
+// is v - v / (exp(2u) + 1): exact limits (v and 0) when the exponential overflows or underflows,
+// no cancellation, and seven instructions: 2u log2(e) = v (a + b v^2) feeds v_exp_f32 directly.
 __device__ __forceinline__ float gelu_tanh_f(float v) {
-    const float k0 = 0.7978845608028654f, k1 = 0.044715f;
-    float u = k0 * (v + k1 * v * v * v);
-    // tanh(u) = 1 - 2 / (exp(2u) + 1); exact limits at +-inf, no cancellation blow-up
-    float t = 1.0f - 2.0f * __builtin_amdgcn_rcpf(__expf(2.0f * u) + 1.0f);
-    return 0.5f * v * (1.0f + t);
+    constexpr float a = 2.0f * 0.7978845608028654f * 1.4426950408889634f;
+    constexpr float b = a * 0.044715f;
+    const float e = __builtin_amdgcn_exp2f(v * __builtin_fmaf(b, v * v, a));
+    return __builtin_fmaf(-v, __builtin_amdgcn_rcpf(e + 1.0f), v);
 }
 __device__ __forceinline__ float gelu_erf_f(float v) { return 0.5f * v * (1.0f + erff(v * 0.70710678118654752f)); }
 __device__ __forceinline__ float silu_f(float v) { return v * __builtin_amdgcn_rcpf(1.0f + __expf(-v)); }

@@ -26,10 +26,10 @@
 //  * the operand blocks that open slab s+1 are read from LDS during the last row group of
 //    slab s into a second register set, and inside a slab the A block of the next row group is
 //    read before the current group's MFMAs are issued, so ds_read latency overlaps MFMA time.
-//  * epilogue: the accumulator layout gives a lane one column and scattered rows; each
-//    wavefront stages its bf16 tile in its own slice of the (now idle) LDS - neighbouring lanes
-//    swap one value first (DPP) so every LDS write is a packed pair of columns - and writes it
-//    out row-wise, 16 bytes per lane, whole row segments per instruction.
+//  * epilogue: the weight block is the MFMA's first operand, which gives a lane runs of four
+//    consecutive output columns of one token row; each wavefront stages its bf16 tile in its own
+//    slice of the (now idle) LDS and writes it out row-wise, 16 bytes per lane, whole row
+//    segments per instruction.
 //
 // Gated epilogues: within a wavefront's 32*TN columns the first half are gate columns and the
 // second half the matching up columns, so the pair sits in the same lane of two accumulators.
@@ -194,7 +194,7 @@ __global__ __launch_bounds__(256) void gemm_fp8_big_kernel(const BigArgs p) {
             const int slab_ = before_ ? s_ + STAGES - 2 : s_ + STAGES - 1;                                     \
             const int c0_ = before_ ? COPIES / 2 + i_ * 2 : (i_ - TM / 2) * 2;                                 \
             _Pragma("unroll") for (int j_ = 0; j_ < TN; ++j_) {                                                \
-                acc[i_][j_] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(fa_[i_], FB[j_], acc[i_][j_],    \
+                acc[i_][j_] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(FB[j_], fa_[i_], acc[i_][j_],    \
                                                                                0, 0, 0, 0, 0, 0);              \
                 if (req_ && j_ % (TN / 2) == TN / 2 - 1) issue(slab_, c0_ + j_ / (TN / 2));                    \
                 __builtin_amdgcn_sched_barrier(0);                                                             \
@@ -262,73 +262,93 @@ __global__ __launch_bounds__(256) void gemm_fp8_big_kernel(const BigArgs p) {
     }
 
     // ---- epilogue ------------------------------------------------------------------------
+    // The weight block is the MFMA's first operand, so accumulator r of lane (l32, h) of block
+    // (i, j) is the output at token row i*32 + l32, column j*32 + 8*(r/4) + 4*h + r%4: a lane
+    // owns runs of four consecutive columns of one row.  A run becomes four bf16 with two packed
+    // converts and goes to the wavefront's slice of the (now idle) LDS as one 8-byte write; the
+    // staged tile leaves row-wise, 16 bytes per lane, whole row segments per instruction.  The
+    // 16-byte slots of a staged row are XOR-swizzled with the row so that the 32 rows written by
+    // one instruction spread over the banks.
     constexpr int TNO = GATED ? TN / 2 : TN;             // output column blocks per wavefront
     constexpr int ROWB = TNO * 64;                       // staged row length in bytes
+    constexpr int SLOTS = ROWB / 16;
+    constexpr int ROWS_PER_PASS = 16 / SLOTS > 0 ? 16 / SLOTS : 1;   // rows per 256 bytes of banks
     constexpr int STG_BYTES = WM * ROWB;                 // per wavefront
     static_assert(4 * STG_BYTES <= STAGES * TILE_BYTES, "staging fits in the operand LDS");
     const int n_lim = GATED ? half_n : p.N;
     const int nbase = n0 + wn * (GATED ? WN / 2 : WN);
-    float sg[TNO], bg[TNO], su[TNO], bu[TNO];
+    // column constants are read 4 at a time when the arrays allow it (N is a multiple of 16, so
+    // a run of four columns is valid or invalid as a whole)
+    const bool vec_cols = (reinterpret_cast<uintptr_t>(p.b_scale) & 15) == 0 &&
+                          (reinterpret_cast<uintptr_t>(p.bias) & 7) == 0;
+    auto load_cols = [&](int n, v4f& sc, v4f& bi) {
+        if (vec_cols) {
+            sc = *reinterpret_cast<const v4f*>(p.b_scale + n);
+            if (p.bias) {
+                const uint2 b = *reinterpret_cast<const uint2*>(p.bias + n);
+                bi[0] = bf16_bits_to_f32(b.x & 0xFFFFu); bi[1] = __uint_as_float(b.x & 0xFFFF0000u);
+                bi[2] = bf16_bits_to_f32(b.y & 0xFFFFu); bi[3] = __uint_as_float(b.y & 0xFFFF0000u);
+            } else {
+                bi[0] = bi[1] = bi[2] = bi[3] = 0.f;
+            }
+        } else {
 #pragma unroll
-    for (int j = 0; j < TNO; ++j) {
-        const int n = nbase + j * 32 + l32;
-        const int n_safe = n < n_lim ? n : 0;
-        sg[j] = p.b_scale[n_safe];
-        bg[j] = p.bias ? bf16_bits_to_f32(p.bias[n_safe]) : 0.f;
-        su[j] = 0.f; bu[j] = 0.f;
-        if constexpr (GATED) {
-            su[j] = p.b_scale[half_n + n_safe];
-            bu[j] = p.bias ? bf16_bits_to_f32(p.bias[half_n + n_safe]) : 0.f;
+            for (int e = 0; e < 4; ++e) {
+                sc[e] = p.b_scale[n + e];
+                bi[e] = p.bias ? bf16_bits_to_f32(p.bias[n + e]) : 0.f;
+            }
         }
+    };
+    float sa[TM];
+#pragma unroll
+    for (int i = 0; i < TM; ++i) {
+        const int m = m0 + wm * WM + i * 32 + l32;
+        sa[i] = p.a_scale[p.a_scale_scalar ? 0 : (m < p.M ? m : p.M - 1)];
     }
     __syncthreads();  // every wavefront is done reading operands from LDS
     uint8_t* stg = lds + wave * STG_BYTES;
-    const int odd = lane & 1;
-    // Row scales of this lane: rows mrow0 + i*32 + 8*g + (0..3), g = 0..3.
-    const int mrow0 = m0 + wm * WM + 4 * h;
-    const bool vec_rows = !p.a_scale_scalar && m0 + BM <= p.M &&
-                          (reinterpret_cast<uintptr_t>(p.a_scale) & 15) == 0;
 #pragma unroll
-    for (int i = 0; i < TM; ++i) {
-        v4f sa[4];
-        if (vec_rows) {
+    for (int j = 0; j < TNO; ++j) {
+        v4f sg[4], bg[4], su[4], bu[4];
 #pragma unroll
-            for (int g = 0; g < 4; ++g) sa[g] = *reinterpret_cast<const v4f*>(p.a_scale + mrow0 + i * 32 + 8 * g);
-        } else {
-#pragma unroll
-            for (int g = 0; g < 4; ++g)
-#pragma unroll
-                for (int e = 0; e < 4; ++e) {
-                    const int m = mrow0 + i * 32 + 8 * g + e;
-                    sa[g][e] = p.a_scale[p.a_scale_scalar ? 0 : (m < p.M ? m : p.M - 1)];
-                }
+        for (int g = 0; g < 4; ++g) {
+            const int n = nbase + j * 32 + 8 * g + 4 * h;
+            const int n_safe = n < n_lim ? n : 0;
+            load_cols(n_safe, sg[g], bg[g]);
+            if constexpr (GATED) load_cols(half_n + n_safe, su[g], bu[g]);
         }
 #pragma unroll
-        for (int j = 0; j < TNO; ++j) {
+        for (int i = 0; i < TM; ++i) {
+            const int row = i * 32 + l32;
+            const int sw = (row / ROWS_PER_PASS) & (SLOTS - 1);
 #pragma unroll
-            for (int t = 0; t < 8; ++t) {
-                uint32_t b[2];
+            for (int g = 0; g < 4; ++g) {
+                float o[4];
 #pragma unroll
-                for (int e = 0; e < 2; ++e) {
-                    const int r = 2 * t + e;
-                    const float s_a = sa[r / 4][r % 4];
-                    float v = acc[i][j][r] * (s_a * sg[j]) + bg[j];
-                    if constexpr (GATED) {
-                        const float u = acc[i][j + TN / 2][r] * (s_a * su[j]) + bu[j];
-                        v = apply_act<EPI>(round_bf16(v)) * round_bf16(u);
-                    } else if constexpr (EPI != EPI_NONE) {
-                        v = apply_act<EPI>(round_bf16(v));
-                    }
-                    b[e] = f32_to_bf16_bits(v);
+                for (int e = 0; e < 4; ++e) o[e] = acc[i][j][4 * g + e] * (sa[i] * sg[g][e]) + bg[g][e];
+                if constexpr (GATED) {
+                    float u[4];
+#pragma unroll
+                    for (int e = 0; e < 4; ++e) u[e] = acc[i][j + TN / 2][4 * g + e] * (sa[i] * su[g][e]) + bu[g][e];
+                    // gate and up pass through bf16 first, as the two-launch form materialises them
+                    const uint32_t g01 = pack_bf16x2(o[0], o[1]), g23 = pack_bf16x2(o[2], o[3]);
+                    const uint32_t u01 = pack_bf16x2(u[0], u[1]), u23 = pack_bf16x2(u[2], u[3]);
+                    o[0] = apply_act<EPI>(__uint_as_float(g01 << 16)) * __uint_as_float(u01 << 16);
+                    o[1] = apply_act<EPI>(__uint_as_float(g01 & 0xFFFF0000u)) * __uint_as_float(u01 & 0xFFFF0000u);
+                    o[2] = apply_act<EPI>(__uint_as_float(g23 << 16)) * __uint_as_float(u23 << 16);
+                    o[3] = apply_act<EPI>(__uint_as_float(g23 & 0xFFFF0000u)) * __uint_as_float(u23 & 0xFFFF0000u);
+                } else if constexpr (EPI != EPI_NONE) {
+                    const uint32_t g01 = pack_bf16x2(o[0], o[1]), g23 = pack_bf16x2(o[2], o[3]);
+                    o[0] = apply_act<EPI>(__uint_as_float(g01 << 16));
+                    o[1] = apply_act<EPI>(__uint_as_float(g01 & 0xFFFF0000u));
+                    o[2] = apply_act<EPI>(__uint_as_float(g23 << 16));
+                    o[3] = apply_act<EPI>(__uint_as_float(g23 & 0xFFFF0000u));
                 }
-                // even lane keeps row r0 and receives the neighbour's r0 value (column n+1);
-                // odd lane keeps row r1 and receives the neighbour's r1 value (column n-1).
-                const uint32_t send = odd ? b[0] : b[1];
-                const uint32_t recv = (uint32_t)__builtin_amdgcn_mov_dpp((int)send, 0xB1, 0xF, 0xF, true);
-                const uint32_t word = odd ? (recv | (b[1] << 16)) : (b[0] | (recv << 16));
-                const int row = i * 32 + 8 * (t / 2) + 4 * h + 2 * (t % 2) + odd;
-                const int col = j * 32 + (l32 & ~1);
-                *reinterpret_cast<uint32_t*>(stg + row * ROWB + col * 2) = word;
+                uint2 w;
+                w.x = pack_bf16x2(o[0], o[1]);
+                w.y = pack_bf16x2(o[2], o[3]);
+                const int slot = (j * 4 + g) ^ sw;
+                *reinterpret_cast<uint2*>(stg + row * ROWB + slot * 16 + h * 8) = w;
             }
         }
     }
@@ -336,10 +356,11 @@ __global__ __launch_bounds__(256) void gemm_fp8_big_kernel(const BigArgs p) {
 #pragma unroll 4
     for (int qd = 0; qd < STG_BYTES / 1024; ++qd) {
         const int byte = qd * 1024 + lane * 16;
-        const int row = byte / ROWB, colb = byte % ROWB;
-        const uint4 v = *reinterpret_cast<const uint4*>(stg + byte);
+        const int row = byte / ROWB, slot = (byte % ROWB) / 16;
+        const int sw = (row / ROWS_PER_PASS) & (SLOTS - 1);
+        const uint4 v = *reinterpret_cast<const uint4*>(stg + row * ROWB + ((slot ^ sw) << 4));
         const int m = m0 + wm * WM + row;
-        const int n = nbase + (colb >> 1);
+        const int n = nbase + slot * 8;
         if (m < p.M && n < n_lim) *reinterpret_cast<uint4*>(p.out + (int64_t)m * p.ldo + n) = v;
     }
 }
