@@ -42,7 +42,7 @@
 
 namespace phyai {
 
-constexpr int BIG_BK = 64;
+constexpr int BIG_BK = 128;   // bytes of K per LDS row: one L2 cache line
 
 struct BigArgs {
     const uint8_t* __restrict__ a;   // xq [M, K]
@@ -75,38 +75,40 @@ __device__ __forceinline__ void wait_copies() {
     asm volatile("s_waitcnt vmcnt(%0)" ::"n"(N) : "memory");
 }
 
-// Swizzle of the 16-byte chunks of a 64-byte row.  LDS has 64 banks of 4 bytes, so one pass over
-// the banks spans four rows and a 128-bit read is served 16 lanes at a time: rows r, r+4, r+8,
-// r+12 must land in different chunk columns (bit 3 of the row folded in), and so must rows
-// r, r+2, r+4, r+6 (narrower grouping).
-__device__ __forceinline__ int big_swizzle(int row) { return ((row >> 1) & 3) ^ ((row >> 3) & 1); }
+// Swizzle of the eight 16-byte chunks of a 128-byte row.  LDS has 64 banks of 4 bytes, so one
+// pass over the banks spans two rows and a 128-bit read is served 16 lanes at a time: the eight
+// rows of equal parity among 16 consecutive ones must land in different chunk columns.
+__device__ __forceinline__ int big_swizzle(int row) { return (row >> 1) & 7; }
 
-// Operand block of v_mfma_f32_32x32x64: lane (l32, h) supplies 32 of the 64 K-bytes of its row.
-// Which 32 is free as long as A and B agree; chunks h and 2+h are taken so that the two halves of
-// a wavefront never meet in a chunk column either.
-__device__ __forceinline__ v8i big_frag(const uint8_t* buf, int row, int h) {
+// Operand block of v_mfma_f32_32x32x64 for K half kh (bytes [64 kh, 64 kh + 64) of the row): lane
+// (l32, h) supplies 32 of the 64 K-bytes.  Which 32 is free as long as A and B agree; chunks h
+// and 2+h of the half are taken so that the two halves of a wavefront never meet in a chunk
+// column either.
+__device__ __forceinline__ v8i big_frag(const uint8_t* buf, int row, int h, int kh) {
     const int sw = big_swizzle(row);
     const uint8_t* r = buf + row * BIG_BK;
-    const v4i lo = *reinterpret_cast<const v4i*>(r + ((h ^ sw) << 4));
-    const v4i hi = *reinterpret_cast<const v4i*>(r + (((2 + h) ^ sw) << 4));
+    const v4i lo = *reinterpret_cast<const v4i*>(r + (((4 * kh + h) ^ sw) << 4));
+    const v4i hi = *reinterpret_cast<const v4i*>(r + (((4 * kh + 2 + h) ^ sw) << 4));
     v8i f;
     f[0] = lo[0]; f[1] = lo[1]; f[2] = lo[2]; f[3] = lo[3];
     f[4] = hi[0]; f[5] = hi[1]; f[6] = hi[2]; f[7] = hi[3];
     return f;
 }
 
-template <int TM, int TN, int EPI, bool SPLIT>
+// DEPTH: stages of the LDS ring, each holding BIG_BK bytes of K for the whole tile.
+template <int TM, int TN, int DEPTH, int EPI, bool SPLIT>
 __global__ __launch_bounds__(256) void gemm_fp8_big_kernel(const BigArgs p) {
     constexpr bool GATED = epi_is_gated(EPI);
     constexpr int BM = 64 * TM, BN = 64 * TN;        // workgroup tile
     constexpr int WM = 32 * TM, WN = 32 * TN;        // wavefront tile
-    constexpr int TILE_BYTES = (BM + BN) * BIG_BK;   // one K slab of A and B
-    constexpr int CA = BM / 64, CB = BN / 64;        // copy instructions per wavefront per slab
+    constexpr int STAGE_BYTES = (BM + BN) * BIG_BK;  // one stage: A rows, then B rows
+    constexpr int CA = BM / 32, CB = BN / 32;        // copy instructions (8 rows each) per wavefront per stage
     constexpr int COPIES = CA + CB;
-    constexpr int STAGES = 4;                        // depth of the LDS ring
+    constexpr int SLOTS_PER_STAGE = 2 * TM * TN;     // MFMAs of a wavefront per stage
+    constexpr int CPS = (COPIES * 2 + SLOTS_PER_STAGE - 1) / SLOTS_PER_STAGE;   // copies per MFMA: done by mid-stage
     static_assert(TM == TN && TM % 2 == 0, "square wavefront tile, even block count");
-    __shared__ __attribute__((aligned(1024))) uint8_t lds[STAGES * TILE_BYTES];
-    __shared__ int s_last;
+    static_assert(DEPTH == 2 || DEPTH == 4, "ring depth");
+    __shared__ __attribute__((aligned(1024))) uint8_t lds[DEPTH * STAGE_BYTES];
 
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     const int wm = wave >> 1, wn = wave & 1;
@@ -115,19 +117,19 @@ __global__ __launch_bounds__(256) void gemm_fp8_big_kernel(const BigArgs p) {
     const int m0 = blockIdx.y * BM;
     const int n0 = GATED ? blockIdx.x * (BN / 2) : blockIdx.x * BN;
 
-    // ---- copy geometry: wavefront w moves 16-row groups w*CA .. of A and w*CB .. of B --------
-    const int crow = lane >> 2;                                   // row inside the 16-row group
-    const int cchunk = ((lane & 3) ^ big_swizzle(crow)) << 4;      // swizzled 16-byte chunk of that row
+    // ---- copy geometry: wavefront w moves 8-row groups w*CA .. of A and w*CB .. of B; lane i
+    // fills slot i%8 of row i/8 of its group with the chunk that the swizzle assigns to it ------
     uint32_t aoff[CA], boff[CB];
 #pragma unroll
     for (int i = 0; i < CA; ++i) {
-        int r = m0 + (wave * CA + i) * 16 + crow;
+        const int rt = (wave * CA + i) * 8 + (lane >> 3);         // row of the tile
+        int r = m0 + rt;
         r = r < p.M ? r : p.M - 1;
-        aoff[i] = (uint32_t)r * (uint32_t)p.K + cchunk;
+        aoff[i] = (uint32_t)r * (uint32_t)p.K + (((lane & 7) ^ big_swizzle(rt)) << 4);
     }
 #pragma unroll
     for (int i = 0; i < CB; ++i) {
-        const int jj = (wave * CB + i) * 16 + crow;               // column of the output tile
+        const int jj = (wave * CB + i) * 8 + (lane >> 3);         // column of the output tile
         int rb;
         if constexpr (GATED) {
             const int w_ = jj / WN, j = jj % WN;
@@ -138,16 +140,16 @@ __global__ __launch_bounds__(256) void gemm_fp8_big_kernel(const BigArgs p) {
             rb = n0 + jj;
             rb = rb < p.N ? rb : p.N - 1;
         }
-        boff[i] = (uint32_t)rb * (uint32_t)p.K + cchunk;
+        boff[i] = (uint32_t)rb * (uint32_t)p.K + (((lane & 7) ^ big_swizzle(jj)) << 4);
     }
     const int k_begin = SPLIT ? blockIdx.z * p.k_per_split : 0;
     const uint32_t lds_base = (uint32_t)(uintptr_t)lds;
     const uint32_t wave_a = __builtin_amdgcn_readfirstlane(lds_base + wave * (CA * 1024));
     const uint32_t wave_b = __builtin_amdgcn_readfirstlane(lds_base + BM * BIG_BK + wave * (CB * 1024));
-    // copy c (0 .. COPIES-1) of this wavefront's share of slab `slab`
-    auto issue = [&](int slab, int c) {
-        const int k = k_begin + slab * BIG_BK;
-        const uint32_t stage_off = (slab % STAGES) * TILE_BYTES;
+    // copy c (0 .. COPIES-1) of this wavefront's share of stage-load `d` (K bytes [128 d, 128 d + 128))
+    auto issue = [&](int d, int c) {
+        const int k = k_begin + d * BIG_BK;
+        const uint32_t stage_off = (d % DEPTH) * STAGE_BYTES;
         if (c < CA) copy16_to_lds(p.a + k, aoff[c], wave_a + stage_off + c * 1024);
         else copy16_to_lds(p.b + k, boff[c - CA], wave_b + stage_off + (c - CA) * 1024);
     };
@@ -160,83 +162,110 @@ __global__ __launch_bounds__(256) void gemm_fp8_big_kernel(const BigArgs p) {
 #pragma unroll
             for (int r = 0; r < 16; ++r) acc[i][j][r] = 0.f;
 
-    const int n_slabs = (SPLIT ? p.k_per_split : p.K) / BIG_BK;
+    const int n_loads = (SPLIT ? p.k_per_split : p.K) / BIG_BK;   // stage-loads in all, >= DEPTH
     const int arow = wm * WM + l32, brow = wn * WN + l32;
-    auto stage_ptr = [&](int s) -> const uint8_t* { return lds + (s % STAGES) * TILE_BYTES; };
+    auto stage_ptr = [&](int d) -> const uint8_t* { return lds + (d % DEPTH) * STAGE_BYTES; };
 
-    // Opening operand blocks of the current slab (cur) and of the next one (nxt); the two sets
-    // swap roles every slab.
-    v8i fa_cur, fa_nxt, fb_cur[TN], fb_nxt[TN];
+    // Operand blocks read one K half ahead: those of the current half (cur) and of the next one
+    // (nxt); the two sets swap roles every half.  All B blocks and the first A block - or all A
+    // blocks when there are only two row groups, which are too short to hide an LDS read.
+    constexpr bool A_AHEAD = TM == 2;
+    constexpr int NA = A_AHEAD ? TM : 1;             // A blocks read a half ahead
+    v8i fa_cur[TM], fa_nxt[TM], fb_cur[TN], fb_nxt[TN];
 
-// S: slab index; FA0/FB: opening blocks of slab S (in registers); NFA0/NFB: receive those of
-// slab S+1.  NEXT: slab S+1 exists; AHEAD: how many slabs beyond S+1 may still be in flight when
-// S+1 is needed.  Copies are issued one at a time between MFMAs - a wavefront that queues all of
-// a slab's copies at once sits in the memory pipeline's issue queue while its MFMA pipe runs dry:
-// the row groups after the barrier request the first half of slab S+STAGES-1 (ISSUE), the row
-// groups before it the second half of slab S+STAGES-2 (ISSUE_P), whose stage the previous
-// barrier released.  All flags are literals, so the steady-state loop body is straight-line code.
-#define PHYAI_RUN_SLAB(S, NEXT, AHEAD, ISSUE_P, ISSUE, FA0, FB, NFA0, NFB)                                     \
+// One K half (64 bytes, TM*TN MFMAs per wavefront) of stage-load D.  KH: which half.  FA0/FB: its
+// opening blocks (in registers); NFA0/NFB receive those of the half that follows (the other half
+// of the same stage, or half 0 of stage-load D+1).  NEXT: that half exists.
+//
+// LDS reads are issued long before their MFMAs: a batch of 128-bit reads takes several hundred
+// cycles to land, a row group of four MFMAs 256.  Row group 0 requests the remaining A blocks of
+// this half, row groups 1.. the opening blocks of the next half (B0 and A0 first).
+//
+// One barrier per stage-load, in half 1 after row group 0: by then a wavefront has issued every
+// LDS read of stage-load D, so the barrier both publishes stage-load D+1 (own copies awaited
+// first: AHEAD later stage-loads may stay in flight) and releases D's stage, which load D+DEPTH
+// then refills.  Its copies are requested one or two at a time between the MFMAs that follow - a
+// wavefront that queues them all at once sits in the memory pipeline's issue queue while its
+// MFMA pipe runs dry.  ISSUE: load D+DEPTH exists (requests after the barrier); ISSUE_P: load
+// D-1+DEPTH exists (requests still being spread before the barrier).  All flags are literals, so
+// the steady-state loop body is straight-line code.
+#define PHYAI_RUN_HALF(D, KH, NEXT, AHEAD, ISSUE_P, ISSUE, FA0, FB, NFA0, NFB)                                 \
     {                                                                                                          \
-        const int s_ = (S);                                                                                    \
-        const uint8_t* abuf_ = stage_ptr(s_);                                                                  \
+        const int d_ = (D);                                                                                    \
+        const uint8_t* abuf_ = stage_ptr(d_);                                                                  \
+        const uint8_t* nbuf_ = (KH) == 0 ? abuf_ : stage_ptr(d_ + 1);                                          \
         v8i fa_[TM];                                                                                           \
-        fa_[0] = FA0;                                                                                          \
+        _Pragma("unroll") for (int i_ = 0; i_ < TM; ++i_) fa_[i_] = FA0[A_AHEAD ? i_ : 0];                     \
         _Pragma("unroll") for (int i_ = 0; i_ < TM; ++i_) {                                                    \
-            if (i_ + 1 < TM) fa_[i_ + 1] = big_frag(abuf_, arow + (i_ + 1) * 32, h);                           \
-            if (i_ == TM - 1 && NEXT) {                                                                        \
-                const uint8_t* nbuf_ = stage_ptr(s_ + 1);                                                      \
-                _Pragma("unroll") for (int j_ = 0; j_ < TN; ++j_)                                              \
-                    NFB[j_] = big_frag(nbuf_ + BM * BIG_BK, brow + j_ * 32, h);                                \
-                NFA0 = big_frag(nbuf_, arow, h);                                                               \
+            if (!A_AHEAD && i_ == 0) {                                                                         \
+                _Pragma("unroll") for (int a_ = 1; a_ < TM; ++a_)                                              \
+                    fa_[a_] = big_frag(abuf_, arow + a_ * 32, h, KH);                                          \
             }                                                                                                  \
-            const bool before_ = i_ < TM / 2;                                                                  \
-            const bool req_ = before_ ? (ISSUE_P) : (ISSUE);                                                   \
-            const int slab_ = before_ ? s_ + STAGES - 2 : s_ + STAGES - 1;                                     \
-            const int c0_ = before_ ? COPIES / 2 + i_ * 2 : (i_ - TM / 2) * 2;                                 \
+            if (i_ >= 1 && (NEXT)) {                                                                           \
+                /* item 0: B0; items 1..NA: the A blocks; then B1..: spread over row groups 1..TM-1 */         \
+                _Pragma("unroll") for (int q_ = 0; q_ < TN + NA; ++q_) {                                       \
+                    if (q_ * (TM - 1) / (TN + NA) != i_ - 1) continue;                                         \
+                    if (q_ >= 1 && q_ <= NA) NFA0[q_ - 1] = big_frag(nbuf_, arow + (q_ - 1) * 32, h, 1 - (KH)); \
+                    else {                                                                                     \
+                        const int j_ = q_ == 0 ? 0 : q_ - NA;                                                  \
+                        NFB[j_] = big_frag(nbuf_ + BM * BIG_BK, brow + j_ * 32, h, 1 - (KH));                  \
+                    }                                                                                          \
+                }                                                                                              \
+            }                                                                                                  \
+            const bool after_ = (KH) == 1 && i_ >= 1;   /* past this stage-load's barrier */                   \
+            const bool req_ = after_ ? (ISSUE) : (ISSUE_P);                                                    \
+            const int load_ = after_ ? d_ + DEPTH : d_ - 1 + DEPTH;                                            \
+            /* MFMAs since the last barrier */                                                                 \
+            const int slot0_ = after_ ? (i_ - 1) * TN : (TM - 1) * TN + ((KH) * TM + i_) * TN;                 \
             _Pragma("unroll") for (int j_ = 0; j_ < TN; ++j_) {                                                \
                 acc[i_][j_] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(FB[j_], fa_[i_], acc[i_][j_],    \
                                                                                0, 0, 0, 0, 0, 0);              \
-                if (req_ && j_ % (TN / 2) == TN / 2 - 1) issue(slab_, c0_ + j_ / (TN / 2));                    \
+                _Pragma("unroll") for (int c_ = 0; c_ < CPS; ++c_)                                             \
+                    if (req_ && (slot0_ + j_) * CPS + c_ < COPIES) issue(load_, (slot0_ + j_) * CPS + c_);     \
                 __builtin_amdgcn_sched_barrier(0);                                                             \
             }                                                                                                  \
-            if (i_ == TM / 2 - 1 && NEXT) {                                                                    \
-                wait_copies<COPIES * (AHEAD)>(); /* my copies of slab s+1 are done ... */                      \
-                __syncthreads(); /* ... and so are everybody's; nobody reads slab s-1 any more */              \
+            if ((KH) == 1 && i_ == 0 && (NEXT)) {                                                              \
+                asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory"); /* my reads of stage-load D have landed */  \
+                wait_copies<COPIES * (AHEAD)>();                   /* ... my copies of D+1 too ... */          \
+                __syncthreads();                                   /* ... and so have everybody's */           \
             }                                                                                                  \
         }                                                                                                      \
     }
-#define PHYAI_SLAB_A(S, NEXT, AHEAD, ISSUE_P, ISSUE) \
-    PHYAI_RUN_SLAB(S, NEXT, AHEAD, ISSUE_P, ISSUE, fa_cur, fb_cur, fa_nxt, fb_nxt)
-#define PHYAI_SLAB_B(S, NEXT, AHEAD, ISSUE_P, ISSUE) \
-    PHYAI_RUN_SLAB(S, NEXT, AHEAD, ISSUE_P, ISSUE, fa_nxt, fb_nxt, fa_cur, fb_cur)
+// a whole stage-load: half 0 with the cur register set, half 1 with the nxt set
+#define PHYAI_RUN_STAGE(D, NEXT, AHEAD, ISSUE_P, ISSUE)                                                        \
+    PHYAI_RUN_HALF(D, 0, 1, 0, ISSUE_P, 0, fa_cur, fb_cur, fa_nxt, fb_nxt)                                     \
+    PHYAI_RUN_HALF(D, 1, NEXT, AHEAD, ISSUE_P, ISSUE, fa_nxt, fb_nxt, fa_cur, fb_cur)
 
-    // prologue: slabs 0 .. STAGES-3 and the first half of slab STAGES-2 in flight, slab 0
-    // published, its opening blocks in registers.  n_slabs is even and at least 2*STAGES (checked
-    // on the host).
+    // prologue: stage-loads 0 .. DEPTH-2 and the copies of load DEPTH-1 that the row groups after
+    // a barrier would have requested in flight (the rest of it is spread over stage-load 0 like
+    // every later one), load 0 published, its opening blocks in registers.
+    constexpr int HEAD = (TM - 1) * TN * CPS < COPIES ? (TM - 1) * TN * CPS : COPIES;
 #pragma unroll
-    for (int i = 0; i < STAGES - 2; ++i)
+    for (int d = 0; d < DEPTH - 1; ++d)
 #pragma unroll
-        for (int c = 0; c < COPIES; ++c) issue(i, c);
+        for (int c = 0; c < COPIES; ++c) issue(d, c);
 #pragma unroll
-    for (int c = 0; c < COPIES / 2; ++c) issue(STAGES - 2, c);
-    wait_copies<COPIES * (STAGES - 3) + COPIES / 2>();
+    for (int c = 0; c < HEAD; ++c) issue(DEPTH - 1, c);
+    wait_copies<COPIES * (DEPTH - 2) + HEAD>();
     __syncthreads();
 #pragma unroll
-    for (int j = 0; j < TN; ++j) fb_cur[j] = big_frag(lds + BM * BIG_BK, brow + j * 32, h);
-    fa_cur = big_frag(lds, arow, h);
-    int s = 0;
-    for (; s < n_slabs - STAGES; s += 2) {          // both slabs of the pair still request new slabs
-        PHYAI_SLAB_A(s, 1, STAGES - 3, 1, 1)
-        PHYAI_SLAB_B(s + 1, 1, STAGES - 3, 1, 1)
+    for (int j = 0; j < TN; ++j) fb_cur[j] = big_frag(lds + BM * BIG_BK, brow + j * 32, h, 0);
+#pragma unroll
+    for (int i = 0; i < (A_AHEAD ? TM : 1); ++i) fa_cur[i] = big_frag(lds, arow + i * 32, h, 0);
+    int d = 0;
+    for (; d < n_loads - DEPTH; ++d) { PHYAI_RUN_STAGE(d, 1, DEPTH - 2, 1, 1) }
+    // d == n_loads - DEPTH: the last requests are still being spread, then the ring drains
+    if constexpr (DEPTH == 2) {
+        PHYAI_RUN_STAGE(d, 1, 0, 1, 0)
+        PHYAI_RUN_STAGE(d + 1, 0, 0, 0, 0)
+    } else {
+        PHYAI_RUN_STAGE(d, 1, 2, 1, 0)
+        PHYAI_RUN_STAGE(d + 1, 1, 1, 0, 0)
+        PHYAI_RUN_STAGE(d + 2, 1, 0, 0, 0)
+        PHYAI_RUN_STAGE(d + 3, 0, 0, 0, 0)
     }
-    // s == n_slabs - STAGES: the last requests, then the ring drains
-    PHYAI_SLAB_A(s, 1, 1, 1, 1)
-    PHYAI_SLAB_B(s + 1, 1, 1, 1, 0)
-    PHYAI_SLAB_A(s + 2, 1, 0, 0, 0)
-    PHYAI_SLAB_B(s + 3, 0, 0, 0, 0)
-#undef PHYAI_SLAB_A
-#undef PHYAI_SLAB_B
-#undef PHYAI_RUN_SLAB
+#undef PHYAI_RUN_STAGE
+#undef PHYAI_RUN_HALF
 
     // ---- split-K: publish partial sums; the last split to arrive adds them in split order --
     if constexpr (SPLIT) {
@@ -251,7 +280,9 @@ __global__ __launch_bounds__(256) void gemm_fp8_big_kernel(const BigArgs p) {
 #pragma unroll
                 for (int r = 0; r < 16; ++r) frag[(i * TN + j) * 16 + r] = acc[i][j][r];
         splitk_publish<FRAG, 256>(p.partials, tile, S, blockIdx.z, frag);
-        if (!splitk_arrive(p.counters, tile, S, &s_last)) return;
+        // splitk_arrive opens with a barrier, after which nobody reads operands any more: a word
+        // of the ring serves as its flag
+        if (!splitk_arrive(p.counters, tile, S, reinterpret_cast<int*>(lds))) return;
         splitk_gather<FRAG, 256>(p.partials, p.counters, tile, S, frag);
 #pragma unroll
         for (int i = 0; i < TM; ++i)
@@ -274,7 +305,7 @@ __global__ __launch_bounds__(256) void gemm_fp8_big_kernel(const BigArgs p) {
     constexpr int SLOTS = ROWB / 16;
     constexpr int ROWS_PER_PASS = 16 / SLOTS > 0 ? 16 / SLOTS : 1;   // rows per 256 bytes of banks
     constexpr int STG_BYTES = WM * ROWB;                 // per wavefront
-    static_assert(4 * STG_BYTES <= STAGES * TILE_BYTES, "staging fits in the operand LDS");
+    static_assert(4 * STG_BYTES <= DEPTH * STAGE_BYTES, "staging fits in the operand LDS");
     const int n_lim = GATED ? half_n : p.N;
     const int nbase = n0 + wn * (GATED ? WN / 2 : WN);
     // column constants are read 4 at a time when the arrays allow it (N is a multiple of 16, so
@@ -408,16 +439,19 @@ size_t big_partial_bytes(int M, int N, int epilogue, const BigPlan& pl) {
     return (size_t)big_tiles(M, N, epilogue, 128, 128) * pl.splits * 128 * 128 * sizeof(float);
 }
 
+#ifndef BIG_DEPTH_SMALL
+#define BIG_DEPTH_SMALL 4
+#endif
 template <int T, int EPI>
 static void big_launch(const BigArgs& a, const GemmProblem& g, int splits, hipStream_t st) {
     const bool gated = epi_is_gated(EPI);
     const int bn_eff = gated ? 32 * T : 64 * T;
     const dim3 grid(big_ceil_div(gated ? g.N / 2 : g.N, bn_eff), big_ceil_div(g.M, 64 * T), splits);
     if constexpr (T == 2) {
-        if (splits > 1) hipLaunchKernelGGL((gemm_fp8_big_kernel<2, 2, EPI, true>), grid, dim3(256), 0, st, a);
-        else hipLaunchKernelGGL((gemm_fp8_big_kernel<2, 2, EPI, false>), grid, dim3(256), 0, st, a);
+        if (splits > 1) hipLaunchKernelGGL((gemm_fp8_big_kernel<2, 2, BIG_DEPTH_SMALL, EPI, true>), grid, dim3(256), 0, st, a);
+        else hipLaunchKernelGGL((gemm_fp8_big_kernel<2, 2, BIG_DEPTH_SMALL, EPI, false>), grid, dim3(256), 0, st, a);
     } else {
-        hipLaunchKernelGGL((gemm_fp8_big_kernel<4, 4, EPI, false>), grid, dim3(256), 0, st, a);
+        hipLaunchKernelGGL((gemm_fp8_big_kernel<4, 4, 2, EPI, false>), grid, dim3(256), 0, st, a);
     }
 }
 
