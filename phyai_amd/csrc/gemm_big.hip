@@ -64,7 +64,7 @@ struct BigArgs {
 // lds_wave_base + 16*i.  Issued as inline assembly so that the compiler does not order its own
 // LDS reads behind copies that are still in flight; the waits are placed by hand below.
 __device__ __forceinline__ void copy16_to_lds(const uint8_t* base, uint32_t lane_offset, uint32_t lds_wave_base) {
-    asm volatile("s_mov_b32 m0, %2\n\tglobal_load_lds_dwordx4 %0, %1"
+    asm volatile("s_mov_b32 m0, %2\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, %1"
                  :: "v"(lane_offset), "s"(base), "s"(lds_wave_base) : "memory", "m0");
 }
 
@@ -356,11 +356,11 @@ __global__ __launch_bounds__(256) void gemm_fp8_big_kernel(const BigArgs p) {
             for (int g = 0; g < 4; ++g) {
                 float o[4];
 #pragma unroll
-                for (int e = 0; e < 4; ++e) o[e] = acc[i][j][4 * g + e] * (sa[i] * sg[g][e]) + bg[g][e];
+                for (int e = 0; e < 4; ++e) o[e] = __builtin_fmaf(acc[i][j][4 * g + e], sa[i] * sg[g][e], bg[g][e]);
                 if constexpr (GATED) {
                     float u[4];
 #pragma unroll
-                    for (int e = 0; e < 4; ++e) u[e] = acc[i][j + TN / 2][4 * g + e] * (sa[i] * su[g][e]) + bu[g][e];
+                    for (int e = 0; e < 4; ++e) u[e] = __builtin_fmaf(acc[i][j + TN / 2][4 * g + e], sa[i] * su[g][e], bu[g][e]);
                     // gate and up pass through bf16 first, as the two-launch form materialises them
                     const uint32_t g01 = pack_bf16x2(o[0], o[1]), g23 = pack_bf16x2(o[2], o[3]);
                     const uint32_t u01 = pack_bf16x2(u[0], u[1]), u23 = pack_bf16x2(u[2], u[3]);
