@@ -46,6 +46,11 @@ EXPERT_SET = [("qkv", 2560, 1024, None), ("o", 1024, 2048, None),
               ("gate_up", 8192, 1024, "geglu_tanh"), ("down", 1024, 4096, None)]
 PREFILL_SET = [("qkv", 2560, 2048, None), ("o", 2048, 2048, None),
                ("gate_up", 32768, 2048, "geglu_tanh"), ("down", 2048, 16384, None)]
+# DiT block (benchmark configuration 5): M = 4800 video-latent tokens, every linear with bias; the
+# adaLN modulation linear runs at M = batch = 1.  (name, N, K, epilogue, M)
+DIT_SET = [("qkv", 6144, 2048, None, 4800), ("out", 2048, 2048, None, 4800),
+           ("fc1", 8192, 2048, "gelu", 4800), ("fc2", 2048, 8192, None, 4800),
+           ("adaLN", 12288, 2048, None, 1)]
 
 
 # HBM bytes moved by one layer's four GEMM launches at M = 50 (20.87 MB fetched + 0.87 MB written),
@@ -144,37 +149,41 @@ def sweep(dev):
     from phyai_amd.runtime import HipGraph
 
     rows = []
-    for set_name, shapes, m1 in (("expert", EXPERT_SET, 50), ("prefill", PREFILL_SET, 816)):
-        for B in (1, 2, 4, 8, 16):
-            M = m1 * B
-            for name, N, K, epi in shapes:
-                g = torch.Generator(device=dev).manual_seed(B * 1000 + N)
-                items = []
-                for _ in range(6):
-                    x = torch.randn(M, K, generator=g, device=dev)
-                    idx = torch.randperm(K, generator=g, device=dev)[: K // 100]
-                    x[:, idx] *= 20.0                      # 1 % outlier channels
-                    w = (torch.randn(N, K, generator=g, device=dev) * 0.02).to(torch.bfloat16)
-                    wq, ws = ops.fp8_weight_quant(w)
-                    n_out = N // 2 if epi else N
-                    items.append((x.to(torch.bfloat16), wq, ws, torch.empty(M, n_out, dtype=torch.bfloat16, device=dev)))
-                    del w
+    cases = [(set_name, B, m1 * B, name, N, K, epi, False)
+             for set_name, shapes, m1 in (("expert", EXPERT_SET, 50), ("prefill", PREFILL_SET, 816))
+             for B in (1, 2, 4, 8, 16) for name, N, K, epi in shapes]
+    cases += [("dit_block", 1, M, name, N, K, epi, True) for name, N, K, epi, M in DIT_SET]
+    for set_name, B, M, name, N, K, epi, with_bias in cases:
+        g = torch.Generator(device=dev).manual_seed(B * 1000 + N)
+        gated = epi in ("geglu_tanh", "geglu_erf", "swiglu")
+        items = []
+        for _ in range(6):
+            x = torch.randn(M, K, generator=g, device=dev)
+            if set_name != "dit_block":
+                idx = torch.randperm(K, generator=g, device=dev)[: K // 100]
+                x[:, idx] *= 20.0                  # 1 % outlier channels
+            w = (torch.randn(N, K, generator=g, device=dev) * 0.02).to(torch.bfloat16)
+            wq, ws = ops.fp8_weight_quant(w)
+            b = (torch.randn(N, generator=g, device=dev) * 0.01).to(torch.bfloat16) if with_bias else None
+            n_out = N // 2 if gated else N
+            items.append((x.to(torch.bfloat16), wq, ws, b, torch.empty(M, n_out, dtype=torch.bfloat16, device=dev)))
+            del w
 
-                def fn():
-                    for x, wq, ws, o in items:
-                        ops.fp8_linear(x, wq, ws, None, epilogue=epi, out=o)
+        def fn():
+            for x, wq, ws, b, o in items:
+                ops.fp8_linear(x, wq, ws, b, epilogue=epi, out=o)
 
-                gr = HipGraph()
-                gr.capture(fn, {})
-                ts, _ = time_replays(gr, 15, 3)
-                us = statistics.median(ts) * 1e3 / len(items)
-                t_hbm = algorithmic_bytes(M, N, K, epi) / (HBM_PEAK_GBS * 1e9) * 1e6
-                t_mfma = 2.0 * M * N * K / (FP8_PEAK_TFLOPS * 1e12) * 1e6
-                rows.append({"set": set_name, "B": B, "M": M, "shape": name, "us": round(us, 2),
-                             "bound": "hbm" if t_hbm >= t_mfma else "mfma",
-                             "roofline_us": round(max(t_hbm, t_mfma), 3),
-                             "frac": round(max(t_hbm, t_mfma) / us, 4)})
-                del items, gr
+        gr = HipGraph()
+        gr.capture(fn, {})
+        ts, _ = time_replays(gr, 15, 3)
+        us = statistics.median(ts) * 1e3 / len(items)
+        t_hbm = algorithmic_bytes(M, N, K, epi, with_bias) / (HBM_PEAK_GBS * 1e9) * 1e6
+        t_mfma = 2.0 * M * N * K / (FP8_PEAK_TFLOPS * 1e12) * 1e6
+        rows.append({"set": set_name, "B": B, "M": M, "shape": name, "us": round(us, 2),
+                     "bound": "hbm" if t_hbm >= t_mfma else "mfma",
+                     "roofline_us": round(max(t_hbm, t_mfma), 3),
+                     "frac": round(max(t_hbm, t_mfma) / us, 4)})
+        del items, gr
     return rows
 
 

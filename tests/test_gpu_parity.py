@@ -278,6 +278,45 @@ def test_linear_epilogues(dev, epi_name, epi, M, N, K):
     assert_close_to_ref(got, want, f"{epi_name} {M}x{N}x{K}")
 
 
+@pytest.mark.parametrize("epi_name,epi", [("gelu_tanh", 4), ("gelu", 5), ("geglu_tanh", 1), ("geglu_erf", 2), ("swiglu", 3)])
+@pytest.mark.parametrize("M,force_big", [(64, ""), (256, "256"), (256, "128")])
+def test_epilogue_activation_values(dev, monkeypatch, epi_name, epi, M, force_big):
+    """One-hot weights hand chosen values to the epilogue: every e4m3 value times a per-row power of
+    two reaches the activation exactly, so the device activation is compared with torch's value by
+    value (within one bf16 step of the rounded result; most must agree exactly)."""
+    ops = _ops()
+    if force_big:
+        monkeypatch.setenv("PHYAI_FP8_BIG", force_big)
+    K = 1024                                                       # also the number of pass-through columns
+    codes = torch.arange(K, dtype=torch.int32) % 256
+    codes[(codes & 0x7F) == 0x7F] = 0                              # no NaN codes
+    xq = codes.to(torch.uint8).repeat(M, 1).view(torch.float8_e4m3fn)
+    xs = torch.tensor([2.0 ** ((m % 13) - 9) for m in range(M)], dtype=torch.float32).reshape(M, 1)
+    gated = epi in ref.GATED
+    N = 2 * K if gated else K
+    w = torch.zeros(N, K)
+    w[torch.arange(K), torch.arange(K)] = 1.0                      # gate / plain rows: column n passes code n
+    if gated:
+        w[K + torch.arange(K), 0x38] = 1.0                         # up rows: the column that holds 1.0
+    wq = w.to(torch.float8_e4m3fn)
+    ws = torch.ones(N)
+    got = ops.fp8_gemm(xq.to(dev), xs.to(dev), wq.to(dev), ws.to(dev), None, epilogue=epi_name).float().cpu()
+    y = ref.gemm_f32(xq, xs, wq, ws)
+    want = ref.epilogue(y, epi).float()
+    assert got.shape == want.shape == (M, K)
+    step = torch.maximum(want.abs(), torch.full_like(want, 2.0 ** -126)) * 2.0 ** -7    # one bf16 step
+    # negative tail: 1 + tanh / 1 + erf cancel in the textbook form, leaving an error of about one
+    # fp32 epsilon of the argument; the device form does not cancel
+    slack = 3e-7 * y[:, :K].abs() * (y[:, K:].abs() if gated else 1.0)
+    bad = (got - want).abs() > step + slack
+    assert not bool(bad.any()), (f"{epi_name}: off by more than one bf16 step at pre-activation values "
+                                 f"{y[:, :K][bad][:8].tolist()}: got {got[bad][:8].tolist()} want {want[bad][:8].tolist()}")
+    # exact agreement is asked only where the textbook form is itself accurate (no cancellation)
+    clean = y[:, :K] > -2.0
+    agree = float((got == want)[clean].float().mean())
+    assert agree > 0.995, f"{epi_name}: only {agree:.4f} of the rounded results agree"
+
+
 def test_linear_no_bias_and_batched(dev):
     ops = _ops()
     x = seeded((2, 25, 1024), seed=9)
