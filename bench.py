@@ -187,13 +187,13 @@ def sweep(dev):
     return rows
 
 
-def probe(dev, layers, M):
-    """Counter probe: per expert shape one GEMM launch per layer (18 distinct weight sets, so the
-    weights come from HBM), then a 64 MiB device-to-device copy whose traffic is known
-    (64 MiB read, 64 MiB written) to calibrate the counters."""
+def probe(dev, layers, M, shapes=EXPERT_SET):
+    """Counter probe: per shape one GEMM launch per layer (distinct weight sets, so the weights
+    come from HBM), then a 64 MiB device-to-device copy whose traffic is known (64 MiB read,
+    64 MiB written) to calibrate the counters."""
     from phyai_amd import ops
 
-    for name, N, K, epi in EXPERT_SET:
+    for name, N, K, epi in shapes:
         pre = [(ops.fp8_quant_rowwise(layer[name]["x"]), layer[name]) for layer in layers]
         torch.cuda.synchronize()
         for (xq, xs), t in pre:
@@ -244,6 +244,8 @@ def main() -> int:
     ap.add_argument("--probe", action="store_true",
                     help="launch each expert GEMM shape a few times plus a 64 MiB device copy and exit; "
                          "meant to run under `rocprofv3 --pmc FETCH_SIZE` / `--pmc WRITE_SIZE`")
+    ap.add_argument("--probe-prefill", action="store_true",
+                    help="the same for the prefill GEMM shapes (M = 816, 4 weight sets), for the MFMA / LDS counters")
     args = ap.parse_args()
     if args.gpus != 1 or int(os.environ.get("WORLD_SIZE", "1")) != 1:
         print("bench.py: this path is built and measured on ONE GPU (TP=1, no collectives); "
@@ -258,6 +260,10 @@ def main() -> int:
     dev = torch.device("cuda", 0)
     torch.cuda.set_device(dev)
     M, n_layers, denoise_steps = 50, 18, 10
+
+    if args.probe_prefill:
+        probe(dev, make_layers(dev, PREFILL_SET, 816, 4, seed0=10_000), 816, PREFILL_SET)
+        return 0
 
     layers = make_layers(dev, EXPERT_SET, M, n_layers)
 

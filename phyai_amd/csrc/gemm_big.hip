@@ -58,7 +58,27 @@ struct BigArgs {
     int k_per_split;
     float* __restrict__ partials;
     int* __restrict__ counters;
+    int m_tiles, n_tiles;            // tile grid; the launch is 1-D over it (see big_tile_of)
 };
+
+// Workgroup id -> tile.  Workgroups go to the 8 XCDs round-robin (id % 8) and each XCD has its own
+// L2, so ids are laid out for the tiles that share an XCD at a time to share operands: the tile
+// grid is cut into bands of 4 tile rows; inside a band, 8 consecutive ids are 8 neighbouring
+// tile columns (one per XCD), and the next 8 ids the same columns one tile row further down.  An
+// XCD thus works on all (up to 4) tile rows of one tile column together - the weight rows come
+// from HBM once per band - while the activation rows of the band stay in its L2.  Tile columns
+// are padded to a multiple of 8; ids that fall into the padding have no tile.
+struct BigTile { int m, n; };
+__device__ __forceinline__ BigTile big_tile_of(int id, int m_tiles, int n_tiles) {
+    const int nt8 = (n_tiles + 7) & ~7;
+    const int band = id / (4 * nt8);
+    const int local = id - band * 4 * nt8;
+    const int bm = m_tiles - 4 * band < 4 ? m_tiles - 4 * band : 4;
+    BigTile t;
+    t.n = (local / (8 * bm)) * 8 + (local & 7);
+    t.m = 4 * band + (local >> 3) % bm;
+    return t;
+}
 
 // One 16-byte chunk per lane from global memory straight into LDS: lane i's chunk lands at
 // lds_wave_base + 16*i.  Issued as inline assembly so that the compiler does not order its own
@@ -114,8 +134,10 @@ __global__ __launch_bounds__(256) void gemm_fp8_big_kernel(const BigArgs p) {
     const int wm = wave >> 1, wn = wave & 1;
     const int l32 = lane & 31, h = lane >> 5;
     const int half_n = p.N / 2;
-    const int m0 = blockIdx.y * BM;
-    const int n0 = GATED ? blockIdx.x * (BN / 2) : blockIdx.x * BN;
+    const BigTile tile_id = big_tile_of(blockIdx.x, p.m_tiles, p.n_tiles);
+    if (tile_id.n >= p.n_tiles) return;              // padding of the tile order
+    const int m0 = tile_id.m * BM;
+    const int n0 = GATED ? tile_id.n * (BN / 2) : tile_id.n * BN;
 
     // ---- copy geometry: wavefront w moves 8-row groups w*CA .. of A and w*CB .. of B; lane i
     // fills slot i%8 of row i/8 of its group with the chunk that the swizzle assigns to it ------
@@ -271,7 +293,7 @@ __global__ __launch_bounds__(256) void gemm_fp8_big_kernel(const BigArgs p) {
     if constexpr (SPLIT) {
         constexpr int FRAG = TM * TN * 16;
         const int S = gridDim.z;
-        const int tile = blockIdx.y * gridDim.x + blockIdx.x;
+        const int tile = tile_id.m * p.n_tiles + tile_id.n;
         float frag[FRAG];
 #pragma unroll
         for (int i = 0; i < TM; ++i)
@@ -443,10 +465,12 @@ size_t big_partial_bytes(int M, int N, int epilogue, const BigPlan& pl) {
 #define BIG_DEPTH_SMALL 4
 #endif
 template <int T, int EPI>
-static void big_launch(const BigArgs& a, const GemmProblem& g, int splits, hipStream_t st) {
+static void big_launch(BigArgs a, const GemmProblem& g, int splits, hipStream_t st) {
     const bool gated = epi_is_gated(EPI);
     const int bn_eff = gated ? 32 * T : 64 * T;
-    const dim3 grid(big_ceil_div(gated ? g.N / 2 : g.N, bn_eff), big_ceil_div(g.M, 64 * T), splits);
+    a.n_tiles = big_ceil_div(gated ? g.N / 2 : g.N, bn_eff);
+    a.m_tiles = big_ceil_div(g.M, 64 * T);
+    const dim3 grid(a.m_tiles * ((a.n_tiles + 7) & ~7), 1, splits);
     if constexpr (T == 2) {
         if (splits > 1) hipLaunchKernelGGL((gemm_fp8_big_kernel<2, 2, BIG_DEPTH_SMALL, EPI, true>), grid, dim3(256), 0, st, a);
         else hipLaunchKernelGGL((gemm_fp8_big_kernel<2, 2, BIG_DEPTH_SMALL, EPI, false>), grid, dim3(256), 0, st, a);
