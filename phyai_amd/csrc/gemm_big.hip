@@ -290,28 +290,31 @@ __global__ __launch_bounds__(256) void gemm_fp8_big_kernel(const BigArgs p) {
 #undef PHYAI_RUN_HALF
 
     // ---- split-K: publish partial sums; the last split to arrive adds them in split order --
+    // Two blocks (32 floats per lane) at a time, so that the 4 x 4 variant never holds more than
+    // that outside its accumulators.
     if constexpr (SPLIT) {
-        constexpr int FRAG = TM * TN * 16;
+        constexpr int FRAG = TM * TN * 16, CHUNK = 32;
         const int S = gridDim.z;
         const int tile = tile_id.m * p.n_tiles + tile_id.n;
-        float frag[FRAG];
 #pragma unroll
-        for (int i = 0; i < TM; ++i)
+        for (int c = 0; c < TM * TN / 2; ++c) {
+            float frag[CHUNK];
 #pragma unroll
-            for (int j = 0; j < TN; ++j)
-#pragma unroll
-                for (int r = 0; r < 16; ++r) frag[(i * TN + j) * 16 + r] = acc[i][j][r];
-        splitk_publish<FRAG, 256>(p.partials, tile, S, blockIdx.z, frag);
+            for (int r = 0; r < 32; ++r) frag[r] = acc[(2 * c) / TN][(2 * c) % TN + r / 16][r % 16];
+            splitk_publish_part<FRAG, 256, CHUNK>(p.partials, tile, S, blockIdx.z, c * CHUNK, frag);
+        }
+        wait_own_stores();
         // splitk_arrive opens with a barrier, after which nobody reads operands any more: a word
         // of the ring serves as its flag
         if (!splitk_arrive(p.counters, tile, S, reinterpret_cast<int*>(lds))) return;
-        splitk_gather<FRAG, 256>(p.partials, p.counters, tile, S, frag);
 #pragma unroll
-        for (int i = 0; i < TM; ++i)
+        for (int c = 0; c < TM * TN / 2; ++c) {
+            float frag[CHUNK];
+            splitk_gather_part<FRAG, 256, CHUNK>(p.partials, tile, S, c * CHUNK, frag);
 #pragma unroll
-            for (int j = 0; j < TN; ++j)
-#pragma unroll
-                for (int r = 0; r < 16; ++r) acc[i][j][r] = frag[(i * TN + j) * 16 + r];
+            for (int r = 0; r < 32; ++r) acc[(2 * c) / TN][(2 * c) % TN + r / 16][r % 16] = frag[r];
+        }
+        splitk_reset(p.counters, tile);
     }
 
     // ---- epilogue ------------------------------------------------------------------------
@@ -443,22 +446,22 @@ BigPlan big_plan(int M, int N, int K, int epilogue) {
     else if (big_tiles(M, N, epilogue, 256, 256) >= 200) pl.tile = 256;
     else if (big_tiles(M, N, epilogue, 128, 128) >= 48) pl.tile = 128;
     else return pl;
+    const int tiles = big_tiles(M, N, epilogue, pl.tile, pl.tile);
     if (pl.tile == 128) {
-        const int tiles = big_tiles(M, N, epilogue, 128, 128);
         // Measured at M = 816: splitting pays for K = 16384 (67 -> 49 us with two splits) and
         // costs for K = 2048 (19 -> 25 us): the partial-sum round trip is worth about 6 us.
         if (tiles < 200 && K >= 8192 && K % 256 == 0) pl.splits = 2;
-        if (const char* e = getenv("PHYAI_FP8_BIG_SPLITS")) {
-            const int s = atoi(e);
-            if (s >= 1 && K % (s * 128) == 0 && K / s >= 512 && tiles * s <= 4096) pl.splits = s;
-        }
+    }
+    if (const char* e = getenv("PHYAI_FP8_BIG_SPLITS")) {
+        const int s = atoi(e);
+        if (s >= 1 && K % (s * 128) == 0 && K / s >= 512 && tiles * s <= 4096) pl.splits = s;
     }
     return pl;
 }
 
 size_t big_partial_bytes(int M, int N, int epilogue, const BigPlan& pl) {
     if (pl.splits <= 1) return 0;
-    return (size_t)big_tiles(M, N, epilogue, 128, 128) * pl.splits * 128 * 128 * sizeof(float);
+    return (size_t)big_tiles(M, N, epilogue, pl.tile, pl.tile) * pl.splits * pl.tile * pl.tile * sizeof(float);
 }
 
 #ifndef BIG_DEPTH_SMALL
@@ -475,7 +478,8 @@ static void big_launch(BigArgs a, const GemmProblem& g, int splits, hipStream_t 
         if (splits > 1) hipLaunchKernelGGL((gemm_fp8_big_kernel<2, 2, BIG_DEPTH_SMALL, EPI, true>), grid, dim3(256), 0, st, a);
         else hipLaunchKernelGGL((gemm_fp8_big_kernel<2, 2, BIG_DEPTH_SMALL, EPI, false>), grid, dim3(256), 0, st, a);
     } else {
-        hipLaunchKernelGGL((gemm_fp8_big_kernel<4, 4, 2, EPI, false>), grid, dim3(256), 0, st, a);
+        if (splits > 1) hipLaunchKernelGGL((gemm_fp8_big_kernel<4, 4, 2, EPI, true>), grid, dim3(256), 0, st, a);
+        else hipLaunchKernelGGL((gemm_fp8_big_kernel<4, 4, 2, EPI, false>), grid, dim3(256), 0, st, a);
     }
 }
 
@@ -505,7 +509,7 @@ int launch_gemm_big(const GemmProblem& g, const BigPlan& pl, hipStream_t st) {
     if (pl.splits > 1 && (g.workspace == nullptr ||
                           g.workspace_bytes < kGemmHeaderBytes + big_partial_bytes(g.M, g.N, g.epilogue, pl)))
         return -3;
-    if (pl.tile == 256) return big_launch_epi<4>(a, g, 1, st);
+    if (pl.tile == 256) return big_launch_epi<4>(a, g, pl.splits, st);
     if (pl.tile == 128) return big_launch_epi<2>(a, g, pl.splits, st);
     return -2;
 }

@@ -35,17 +35,24 @@ __device__ __forceinline__ void wait_own_stores() { asm volatile("s_waitcnt vmcn
 
 // FRAG floats per thread (even), THREADS threads.  Layout of one partial:
 // [FRAG/2][THREADS][2] floats, so that a wavefront's 64-bit accesses are contiguous.
-template <int FRAG, int THREADS>
-__device__ __forceinline__ void splitk_publish(float* partials, int tile, int S, int z, const float* frag) {
+// The *_part forms move CHUNK of the FRAG floats, elements e0 .. e0+CHUNK-1, so that a thread with
+// a large fragment never holds more than a chunk of it outside its accumulators.
+template <int FRAG, int THREADS, int CHUNK>
+__device__ __forceinline__ void splitk_publish_part(float* partials, int tile, int S, int z, int e0, const float* frag) {
     float* mine = partials + ((size_t)tile * S + z) * (size_t)(FRAG * THREADS);
 #pragma unroll
-    for (int e = 0; e < FRAG; e += 2)
-        coherent_store2(mine + ((e / 2) * THREADS + threadIdx.x) * 2, frag[e], frag[e + 1]);
+    for (int e = 0; e < CHUNK; e += 2)
+        coherent_store2(mine + (((e0 + e) / 2) * THREADS + threadIdx.x) * 2, frag[e], frag[e + 1]);
+}
+
+template <int FRAG, int THREADS>
+__device__ __forceinline__ void splitk_publish(float* partials, int tile, int S, int z, const float* frag) {
+    splitk_publish_part<FRAG, THREADS, FRAG>(partials, tile, S, z, 0, frag);
     wait_own_stores();
 }
 
 // Returns true in every lane of the workgroup that arrived last.  Must be called by all
-// threads, after splitk_publish.
+// threads, after splitk_publish (or the last splitk_publish_part and wait_own_stores).
 __device__ __forceinline__ bool splitk_arrive(int* counters, int tile, int S, int* s_flag) {
     __syncthreads();
     if (threadIdx.x == 0) {
@@ -56,22 +63,33 @@ __device__ __forceinline__ bool splitk_arrive(int* counters, int tile, int S, in
     return *s_flag != 0;
 }
 
-template <int FRAG, int THREADS>
-__device__ __forceinline__ void splitk_gather(const float* partials, int* counters, int tile, int S, float* frag) {
+// Sum of elements e0 .. e0+CHUNK-1 over the S partials of a tile, in split order.
+template <int FRAG, int THREADS, int CHUNK>
+__device__ __forceinline__ void splitk_gather_part(const float* partials, int tile, int S, int e0, float* frag) {
     const float* all = partials + (size_t)tile * S * (size_t)(FRAG * THREADS);
 #pragma unroll
-    for (int e = 0; e < FRAG; ++e) frag[e] = 0.f;
+    for (int e = 0; e < CHUNK; ++e) frag[e] = 0.f;
     for (int z = 0; z < S; ++z) {
         const float* pz = all + (size_t)z * (FRAG * THREADS);
-        float t[FRAG];
+        float t[CHUNK];
 #pragma unroll
-        for (int e = 0; e < FRAG; e += 2)
-            coherent_load2(pz + ((e / 2) * THREADS + threadIdx.x) * 2, t[e], t[e + 1]);
+        for (int e = 0; e < CHUNK; e += 2)
+            coherent_load2(pz + (((e0 + e) / 2) * THREADS + threadIdx.x) * 2, t[e], t[e + 1]);
 #pragma unroll
-        for (int e = 0; e < FRAG; ++e) frag[e] += t[e];
+        for (int e = 0; e < CHUNK; ++e) frag[e] += t[e];
     }
+}
+
+// The gathering workgroup puts the tile's counter back to zero for the next call.
+__device__ __forceinline__ void splitk_reset(int* counters, int tile) {
     if (threadIdx.x == 0)
         __hip_atomic_store(counters + tile, 0, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+}
+
+template <int FRAG, int THREADS>
+__device__ __forceinline__ void splitk_gather(const float* partials, int* counters, int tile, int S, float* frag) {
+    splitk_gather_part<FRAG, THREADS, FRAG>(partials, tile, S, 0, frag);
+    splitk_reset(counters, tile);
 }
 
 }  // namespace phyai

@@ -398,10 +398,11 @@ def test_big_tile_kernel_exact_integer(dev, monkeypatch, tile):
         assert torch.equal(got.cpu(), want), f"{(M, N, K)}"
 
 
-def test_big_tile_kernel_split_k(dev, monkeypatch):
-    """128 x 128 tiles with the K range split over two and four workgroups (partials in the workspace)."""
+@pytest.mark.parametrize("tile", ["128", "256"])
+def test_big_tile_kernel_split_k(dev, monkeypatch, tile):
+    """Both tile sizes with the K range split over two and four workgroups (partials in the workspace)."""
     ops = _ops()
-    monkeypatch.setenv("PHYAI_FP8_BIG", "128")
+    monkeypatch.setenv("PHYAI_FP8_BIG", tile)
     x, wq, ws, b = _problem(300, 384, 4096, seed=77)
     xq, xs = ref.quant_rowwise(x)
     want = ref.gemm_f32(xq, xs, wq, ws, b)
