@@ -31,7 +31,7 @@
 extern "C" {
 #endif
 
-#define PHYAI_FP8_ABI_VERSION 1
+#define PHYAI_FP8_ABI_VERSION 2
 
 enum {
     PHYAI_FP8_OK = 0,
@@ -117,6 +117,35 @@ int phyai_fp8_linear(const void *x, int64_t ldx, const void *w, const float *w_s
                      const void *bias, void *out, int64_t ldo, int64_t M, int64_t N,
                      int64_t K, int epilogue, void *workspace, size_t workspace_bytes,
                      void *stream);
+
+/*
+ * RMSNorm whose output feeds the quantizer without a round trip through memory.
+ * Replaces phyai_kernel.triton.rmsnorm / gemma_rmsnorm
+ * (phyai-kernel/phyai_kernel/triton/rms_norm.py:42-75: fp32 reduction,
+ * out = bf16(x * rsqrt(mean(x^2) + eps) * w), w + 1 for the Gemma form) followed
+ * by Fp8Spec.quantize_activation (layers/quant/fp8.py:150-155) on that bf16
+ * output.  x: [M, D] bf16, row stride ldx; weight: [D] bf16.  out ([M, D] bf16,
+ * row stride ldo) may be NULL when only the codes are wanted; xq / x_scale may
+ * both be NULL when only the normalised bf16 tensor is wanted.  D % 8 == 0,
+ * D <= 8192 (the reference's single-block limit).
+ */
+int phyai_fp8_rmsnorm_quant(const void *x, int64_t ldx, const void *weight, int gemma,
+                            int64_t M, int64_t D, float eps, void *out, int64_t ldo,
+                            void *xq, float *x_scale, void *stream);
+
+/*
+ * Adaptive RMSNorm (scale, shift, gate from a projected conditioning row) with the
+ * same fused quantizer.  Replaces phyai_kernel.triton.adarmsnorm
+ * (phyai-kernel/phyai_kernel/triton/ada_rms_norm.py:63-117:
+ * out = bf16(x * rsqrt(mean(x^2) + eps) * (1 + scale) + shift), gate copied once per
+ * modulation row) + the quantizer.  modulation: [mod_rows, 3 * D] bf16 = scale |
+ * shift | gate, row stride ld_mod; M must be a multiple of mod_rows and row m uses
+ * modulation row m / (M / mod_rows).  gate_out: [mod_rows, D] bf16 or NULL.
+ */
+int phyai_fp8_adarmsnorm_quant(const void *x, int64_t ldx, const void *modulation,
+                               int64_t ld_mod, int64_t mod_rows, int64_t M, int64_t D,
+                               float eps, void *out, int64_t ldo, void *gate_out,
+                               int64_t ld_gate, void *xq, float *x_scale, void *stream);
 
 /*
  * Test hook: run the device fp32 -> e4m3fn cast used by the quantizers over n

@@ -99,3 +99,33 @@ def linear(x, wq, w_scale, bias=None, epi: int = EPI_NONE) -> torch.Tensor:
     y = gemm_f32(xq, xs, wq, w_scale, bias)
     out = epilogue(y, epi, x.dtype)
     return out.reshape(*x.shape[:-1], out.shape[-1])
+
+
+# ---- norms (phyai-kernel/phyai_kernel/triton/rms_norm.py:58-75, ada_rms_norm.py:83-117) --------
+
+def rmsnorm(x: torch.Tensor, weight: torch.Tensor, eps: float = 1e-6, gemma: bool = False) -> torch.Tensor:
+    """fp32 reduction, ``x_hat = x * rsqrt(var + eps)``, ``out = (x_hat * w).to(x.dtype)`` with
+    ``w + 1`` for the Gemma form (rms_norm.py:58-73, the non-HF branch)."""
+    xf = x.float()
+    var = (xf * xf).sum(-1, keepdim=True) / x.shape[-1]
+    x_hat = xf * torch.rsqrt(var + eps)
+    w = weight.float()
+    if gemma:
+        w = w + 1.0
+    return (x_hat * w).to(x.dtype)
+
+
+def adarmsnorm(x: torch.Tensor, modulation: torch.Tensor, eps: float = 1e-6) -> tuple[torch.Tensor, torch.Tensor]:
+    """``out = (x_hat * (1 + scale) + shift).to(x.dtype)``, ``gate = gate.to(x.dtype)``; modulation row
+    ``r`` serves x rows ``[r * g, (r + 1) * g)`` (ada_rms_norm.py:77-117)."""
+    D = x.shape[-1]
+    x2 = x.reshape(-1, D).float()
+    m2 = modulation.reshape(-1, 3 * D).float()
+    g = x2.shape[0] // m2.shape[0]
+    m_rows = m2.repeat_interleave(g, dim=0)
+    scale, shift = m_rows[:, :D], m_rows[:, D:2 * D]
+    var = (x2 * x2).sum(-1, keepdim=True) / D
+    x_hat = x2 * torch.rsqrt(var + eps)
+    out = (x_hat * (1.0 + scale) + shift).to(x.dtype).reshape(x.shape)
+    gate = modulation[..., 2 * D:].to(x.dtype).contiguous()
+    return out, gate

@@ -167,6 +167,65 @@ int phyai_fp8_linear(const void* x, int64_t ldx, const void* w, const float* w_s
                           c.gemm_bytes, stream);
 }
 
+namespace {
+int check_norm_args(const char* fn, const void* x, int64_t ldx, int64_t M, int64_t D, const void* out,
+                    int64_t ldo, const void* xq, const float* x_scale) {
+    if (M < 0 || D <= 0) return fail(PHYAI_FP8_EINVAL, "%s: bad shape M=%lld D=%lld", fn, (long long)M, (long long)D);
+    if (M == 0) return 0;
+    if (!x) return fail(PHYAI_FP8_EINVAL, "%s: null x", fn);
+    if (!out && !xq) return fail(PHYAI_FP8_EINVAL, "%s: neither out nor xq given", fn);
+    if ((xq == nullptr) != (x_scale == nullptr)) return fail(PHYAI_FP8_EINVAL, "%s: xq and x_scale go together", fn);
+    if (D % 8 != 0) return fail(PHYAI_FP8_EUNSUPPORTED, "%s: D=%lld must be a multiple of 8", fn, (long long)D);
+    if (D > 8192) return fail(PHYAI_FP8_EUNSUPPORTED, "%s: D=%lld exceeds 8192", fn, (long long)D);
+    if (ldx < D || ldx % 8 != 0 || (out && (ldo < D || ldo % 8 != 0)))
+        return fail(PHYAI_FP8_EINVAL, "%s: row strides must be >= D and multiples of 8", fn);
+    if (!aligned(x, 16) || (out && !aligned(out, 16)) || (xq && !aligned(xq, 8)))
+        return fail(PHYAI_FP8_EINVAL, "%s: x and out must be 16-byte, xq 8-byte aligned", fn);
+    if (M * ldx >= kMaxElems * 4 || M >= kMaxElems) return fail(PHYAI_FP8_EUNSUPPORTED, "%s: tensor too large", fn);
+    return 0;
+}
+}  // namespace
+
+int phyai_fp8_rmsnorm_quant(const void* x, int64_t ldx, const void* weight, int gemma, int64_t M,
+                            int64_t D, float eps, void* out, int64_t ldo, void* xq, float* x_scale,
+                            void* stream) {
+    if (int rc = check_norm_args("phyai_fp8_rmsnorm_quant", x, ldx, M, D, out, ldo, xq, x_scale)) return rc;
+    if (M == 0) return PHYAI_FP8_OK;
+    if (!weight || !aligned(weight, 16)) return fail(PHYAI_FP8_EINVAL, "phyai_fp8_rmsnorm_quant: weight must be a 16-byte aligned pointer");
+    phyai::NormQuantArgs a = {};
+    a.x = static_cast<const uint16_t*>(x); a.ldx = ldx; a.D = (int)D; a.eps = eps;
+    a.weight = static_cast<const uint16_t*>(weight); a.gemma = gemma ? 1 : 0;
+    a.group = 1;
+    a.out = static_cast<uint16_t*>(out); a.ldo = ldo;
+    a.xq = static_cast<uint8_t*>(xq); a.scale = x_scale;
+    if (phyai::launch_norm_quant(a, M, false, static_cast<hipStream_t>(stream)) != 0)
+        return fail(PHYAI_FP8_EUNSUPPORTED, "phyai_fp8_rmsnorm_quant: no kernel for D=%lld", (long long)D);
+    return check_launch("phyai_fp8_rmsnorm_quant");
+}
+
+int phyai_fp8_adarmsnorm_quant(const void* x, int64_t ldx, const void* modulation, int64_t ld_mod,
+                               int64_t mod_rows, int64_t M, int64_t D, float eps, void* out,
+                               int64_t ldo, void* gate_out, int64_t ld_gate, void* xq, float* x_scale,
+                               void* stream) {
+    if (int rc = check_norm_args("phyai_fp8_adarmsnorm_quant", x, ldx, M, D, out, ldo, xq, x_scale)) return rc;
+    if (M == 0) return PHYAI_FP8_OK;
+    if (!modulation || !aligned(modulation, 16) || ld_mod < 3 * D || ld_mod % 8 != 0)
+        return fail(PHYAI_FP8_EINVAL, "phyai_fp8_adarmsnorm_quant: modulation must be 16-byte aligned with row stride >= 3*D, a multiple of 8");
+    if (mod_rows <= 0 || M % mod_rows != 0)
+        return fail(PHYAI_FP8_EINVAL, "phyai_fp8_adarmsnorm_quant: M=%lld must be a non-zero multiple of the modulation rows (%lld)", (long long)M, (long long)mod_rows);
+    if (gate_out && (!aligned(gate_out, 16) || ld_gate < D || ld_gate % 8 != 0))
+        return fail(PHYAI_FP8_EINVAL, "phyai_fp8_adarmsnorm_quant: gate_out must be 16-byte aligned with row stride >= D, a multiple of 8");
+    phyai::NormQuantArgs a = {};
+    a.x = static_cast<const uint16_t*>(x); a.ldx = ldx; a.D = (int)D; a.eps = eps;
+    a.mod = static_cast<const uint16_t*>(modulation); a.ld_mod = ld_mod; a.group = (int)(M / mod_rows);
+    a.out = static_cast<uint16_t*>(out); a.ldo = ldo;
+    a.gate = static_cast<uint16_t*>(gate_out); a.ld_gate = ld_gate;
+    a.xq = static_cast<uint8_t*>(xq); a.scale = x_scale;
+    if (phyai::launch_norm_quant(a, M, true, static_cast<hipStream_t>(stream)) != 0)
+        return fail(PHYAI_FP8_EUNSUPPORTED, "phyai_fp8_adarmsnorm_quant: no kernel for D=%lld", (long long)D);
+    return check_launch("phyai_fp8_adarmsnorm_quant");
+}
+
 int phyai_fp8_debug_cast_e4m3(const float* v, int64_t n, void* codes, void* stream) {
     if (n < 0 || (n > 0 && (!v || !codes))) return fail(PHYAI_FP8_EINVAL, "phyai_fp8_debug_cast_e4m3: bad arguments");
     phyai::launch_debug_cast(v, n, codes, static_cast<hipStream_t>(stream));

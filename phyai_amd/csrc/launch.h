@@ -15,6 +15,26 @@ int launch_quant_static(const void* x, int64_t M, int64_t K, int64_t ldx, const 
                         void* xq, hipStream_t st);
 int launch_debug_cast(const float* v, int64_t n, void* codes, hipStream_t st);
 
+// RMSNorm / adaptive RMSNorm with the activation quantizer fused behind it (quant_kernels.hip).
+struct NormQuantArgs {
+    const uint16_t* x;        // [M, D] bf16
+    int64_t ldx;
+    int D;
+    float eps;
+    const uint16_t* weight;   // RMSNorm: [D] bf16
+    int gemma;                //          weight + 1
+    const uint16_t* mod;      // adaptive: [M / group, 3 D] bf16 = scale | shift | gate
+    int64_t ld_mod;
+    int group;                //          rows of x per modulation row
+    uint16_t* out;            // [M, D] bf16 or null
+    int64_t ldo;
+    uint16_t* gate;           // adaptive: [M / group, D] bf16 or null
+    int64_t ld_gate;
+    uint8_t* xq;              // [M, D] codes or null
+    float* scale;             // [M]
+};
+int launch_norm_quant(const NormQuantArgs& a, int64_t M, bool adaptive, hipStream_t st);  // -2: D too large
+
 struct GemmProblem {
     const uint8_t* xq;      // [M, K]
     const float* x_scale;   // [M] or [1]

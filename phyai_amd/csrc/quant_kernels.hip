@@ -223,6 +223,121 @@ int launch_weight_quant(const void* w, int64_t N, int64_t K, int64_t ldw, void* 
                         hipStream_t st) {
     return launch_quant_rows<QUANT_WEIGHT>(w, N, K, ldw, wq, ws, st);
 }
+// ---- RMSNorm / adaptive RMSNorm + quantizer ----------------------------------------------
+template <int THREADS>
+__device__ __forceinline__ float block_sum_f32(float v, float* smem) {
+#pragma unroll
+    for (int off = 32; off >= 1; off >>= 1) v += __shfl_xor(v, off, kWave);
+    if constexpr (THREADS > kWave) {
+        constexpr int NW = THREADS / kWave;
+        const int wave = threadIdx.x / kWave, lane = threadIdx.x % kWave;
+        if (lane == 0) smem[wave] = v;
+        __syncthreads();
+        float r = smem[0];
+#pragma unroll
+        for (int i = 1; i < NW; ++i) r += smem[i];
+        v = r;
+    }
+    return v;
+}
+
+__device__ __forceinline__ void unpack8(uint4 q, float* f) {
+    const uint32_t w[4] = {q.x, q.y, q.z, q.w};
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+        f[2 * i] = bf16_bits_to_f32(w[i] & 0xFFFFu);
+        f[2 * i + 1] = __uint_as_float(w[i] & 0xFFFF0000u);
+    }
+}
+
+// One workgroup per row, the row in registers: sum of squares (fp32), normalise, affine, round to
+// bf16 - the tensor the reference's norm kernel would have written - and, on those bf16 values,
+// the per-token quantizer (row absmax, scale, codes) of quant_rows_reg_kernel.
+template <int THREADS, int CHUNKS, bool ADAPTIVE>
+__global__ __launch_bounds__(THREADS) void norm_quant_kernel(const NormQuantArgs p) {
+    __shared__ float ssum[THREADS / kWave];
+    __shared__ uint32_t smax[THREADS / kWave];
+    const int64_t row = blockIdx.x;
+    const uint16_t* xr = p.x + row * p.ldx;
+    float xf[CHUNKS][8];
+    float ss = 0.f;
+#pragma unroll
+    for (int c = 0; c < CHUNKS; ++c) {
+        const int k = (c * THREADS + threadIdx.x) * 8;
+        uint4 v = make_uint4(0, 0, 0, 0);
+        if (k < p.D) v = *reinterpret_cast<const uint4*>(xr + k);
+        unpack8(v, xf[c]);
+#pragma unroll
+        for (int e = 0; e < 8; ++e) ss += xf[c][e] * xf[c][e];
+    }
+    ss = block_sum_f32<THREADS>(ss, ssum);
+    const float rstd = 1.0f / sqrtf(ss / (float)p.D + p.eps);
+
+    const int64_t mrow = ADAPTIVE ? row / p.group : 0;
+    const uint16_t* mr = ADAPTIVE ? p.mod + mrow * p.ld_mod : nullptr;
+    uint4 ob[CHUNKS];
+    uint32_t m = 0;
+#pragma unroll
+    for (int c = 0; c < CHUNKS; ++c) {
+        const int k = (c * THREADS + threadIdx.x) * 8;
+        ob[c] = make_uint4(0, 0, 0, 0);
+        if (k < p.D) {
+            float o[8];
+            if constexpr (ADAPTIVE) {
+                float sc[8], sh[8];
+                unpack8(*reinterpret_cast<const uint4*>(mr + k), sc);
+                unpack8(*reinterpret_cast<const uint4*>(mr + p.D + k), sh);
+#pragma unroll
+                for (int e = 0; e < 8; ++e) o[e] = (xf[c][e] * rstd) * (1.0f + sc[e]) + sh[e];
+                if (p.gate != nullptr && row % p.group == 0)
+                    *reinterpret_cast<uint4*>(p.gate + mrow * p.ld_gate + k) =
+                        *reinterpret_cast<const uint4*>(mr + 2 * p.D + k);
+            } else {
+                float w[8];
+                unpack8(*reinterpret_cast<const uint4*>(p.weight + k), w);
+#pragma unroll
+                for (int e = 0; e < 8; ++e) o[e] = (xf[c][e] * rstd) * (p.gemma ? w[e] + 1.0f : w[e]);
+            }
+            ob[c].x = f32_to_bf16_bits(o[0]) | (f32_to_bf16_bits(o[1]) << 16);
+            ob[c].y = f32_to_bf16_bits(o[2]) | (f32_to_bf16_bits(o[3]) << 16);
+            ob[c].z = f32_to_bf16_bits(o[4]) | (f32_to_bf16_bits(o[5]) << 16);
+            ob[c].w = f32_to_bf16_bits(o[6]) | (f32_to_bf16_bits(o[7]) << 16);
+            if (p.out != nullptr) *reinterpret_cast<uint4*>(p.out + row * p.ldo + k) = ob[c];
+        }
+        m = absmax8(ob[c], m);
+    }
+    if (p.xq == nullptr) return;
+    m = block_max_u32<THREADS>(m, smax);
+    const float s = scale_from_amax_bits<QUANT_ACT_DYNAMIC>(m);
+    if (threadIdx.x == 0) p.scale[row] = s;
+    const RowDivisor d = make_divisor(s);
+    uint8_t* qr = p.xq + row * (int64_t)p.D;
+#pragma unroll
+    for (int c = 0; c < CHUNKS; ++c) {
+        const int k = (c * THREADS + threadIdx.x) * 8;
+        if (k < p.D) *reinterpret_cast<uint2*>(qr + k) = encode8<QUANT_ACT_DYNAMIC>(ob[c], d);
+    }
+}
+
+template <bool ADAPTIVE>
+static int launch_norm_quant_t(const NormQuantArgs& a, int64_t M, hipStream_t st) {
+    const dim3 grid((unsigned)M);
+#define PHYAI_NQ(T, C) hipLaunchKernelGGL((norm_quant_kernel<T, C, ADAPTIVE>), grid, dim3(T), 0, st, a)
+    if (a.D <= 512) PHYAI_NQ(64, 1);
+    else if (a.D <= 1024) PHYAI_NQ(128, 1);
+    else if (a.D <= 2048) PHYAI_NQ(256, 1);
+    else if (a.D <= 4096) PHYAI_NQ(256, 2);
+    else if (a.D <= 8192) PHYAI_NQ(256, 4);
+    else return -2;
+#undef PHYAI_NQ
+    return 0;
+}
+
+int launch_norm_quant(const NormQuantArgs& a, int64_t M, bool adaptive, hipStream_t st) {
+    if (M == 0) return 0;
+    return adaptive ? launch_norm_quant_t<true>(a, M, st) : launch_norm_quant_t<false>(a, M, st);
+}
+
 int launch_quant_static(const void* x, int64_t M, int64_t K, int64_t ldx, const float* input_scale,
                         void* xq, hipStream_t st) {
     if (M == 0) return 0;

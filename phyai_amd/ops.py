@@ -129,6 +129,113 @@ def fp8_quant_rowwise(x: torch.Tensor, *, out: torch.Tensor | None = None,
     return out, scale_out
 
 
+# ---- norms with the quantizer fused behind them ------------------------------
+
+def _norm_outputs(op: str, x: torch.Tensor, out, quantize: bool, want_out: bool):
+    """Allocate / validate the bf16 output and the (codes, scale) pair of a fused norm."""
+    if out is not None and (out.shape != x.shape or out.dtype != x.dtype or not out.is_contiguous()):
+        raise _err(op, "`out` must be contiguous and match input shape and dtype")
+    if out is None and want_out:
+        out = torch.empty(x.shape, dtype=x.dtype, device=x.device)
+    xq = xs = None
+    if quantize:
+        xq = torch.empty(x.shape, dtype=torch.float8_e4m3fn, device=x.device)
+        xs = torch.empty((*x.shape[:-1], 1), dtype=torch.float32, device=x.device)
+    return out, xq, xs
+
+
+def _rmsnorm(op: str, x, weight, eps, out, gemma: bool, quantize: bool, want_out: bool):
+    x2 = _as_rows(op, x, "x", torch.bfloat16)
+    M, D = x2.shape
+    if not (isinstance(weight, torch.Tensor) and weight.is_cuda and weight.dtype == torch.bfloat16
+            and weight.shape == (D,) and weight.is_contiguous()):
+        raise _err(op, f"weight must be a contiguous bfloat16 GPU tensor of shape ({D},)")
+    if D % 8 != 0 or D > 8192:
+        raise _err(op, f"last dim {D} must be a multiple of 8 and at most 8192")
+    out, xq, xs = _norm_outputs(op, x, out, quantize, want_out)
+    if M == 0:
+        return out, xq, xs
+    ld = x2.stride(0) if M > 1 else D
+    rc = _lib.load().phyai_fp8_rmsnorm_quant(
+        x2.data_ptr(), ld, weight.data_ptr(), 1 if gemma else 0, M, D, float(eps),
+        out.data_ptr() if out is not None else None, D,
+        xq.data_ptr() if xq is not None else None, xs.data_ptr() if xs is not None else None, _stream_ptr())
+    _lib.check(rc, op)
+    return out, xq, xs
+
+
+def rmsnorm(x: torch.Tensor, weight: torch.Tensor, eps: float = 1e-6,
+            out: torch.Tensor | None = None) -> torch.Tensor:
+    """``(rsqrt(mean(x^2) + eps) * x * weight).to(x.dtype)``, fp32 inside - the reference's
+    ``phyai_kernel.triton.rmsnorm`` (``phyai-kernel/phyai_kernel/triton/rms_norm.py:348-371``)."""
+    return _rmsnorm("rmsnorm", x, weight, eps, out, False, False, True)[0]
+
+
+def gemma_rmsnorm(x: torch.Tensor, weight: torch.Tensor, eps: float = 1e-6,
+                  out: torch.Tensor | None = None) -> torch.Tensor:
+    """RMSNorm with the Gemma ``(1 + weight)`` affine (``rms_norm.py:13,63-65``)."""
+    return _rmsnorm("gemma_rmsnorm", x, weight, eps, out, True, False, True)[0]
+
+
+def rmsnorm_fp8(x: torch.Tensor, weight: torch.Tensor, eps: float = 1e-6, *, gemma: bool = False,
+                out: torch.Tensor | None = None, want_out: bool = False):
+    """RMSNorm whose bf16 result goes straight into the per-token quantizer.
+
+    Returns ``(codes, scale)`` - what ``Fp8Spec.quantize_activation`` gives on the norm's output -
+    or ``(codes, scale, out)`` when the bf16 tensor is wanted too (``out=`` or ``want_out``)."""
+    o, xq, xs = _rmsnorm("rmsnorm_fp8", x, weight, eps, out, gemma, True, want_out or out is not None)
+    return (xq, xs) if o is None else (xq, xs, o)
+
+
+def _adarmsnorm(op: str, x, modulation, eps, out, gate_out, quantize: bool, want_out: bool):
+    if not (isinstance(modulation, torch.Tensor) and modulation.is_cuda):
+        raise _err(op, "tensors must live on the GPU")
+    if x.shape[-1] * 3 != modulation.shape[-1]:
+        raise _err(op, f"modulation last dim ({modulation.shape[-1]}) must be 3x x last dim ({x.shape[-1]})")
+    x2 = _as_rows(op, x, "x", torch.bfloat16)
+    M, D = x2.shape
+    mod2 = _as_rows(op, modulation, "modulation", torch.bfloat16)
+    n_mod = mod2.shape[0]
+    if D % 8 != 0 or D > 8192:
+        raise _err(op, f"last dim {D} must be a multiple of 8 and at most 8192")
+    out, xq, xs = _norm_outputs(op, x, out, quantize, want_out)
+    gate_shape = (*modulation.shape[:-1], D)
+    if gate_out is None:
+        gate_out = torch.empty(gate_shape, dtype=x.dtype, device=x.device)
+    elif tuple(gate_out.shape) != tuple(gate_shape) or gate_out.dtype != x.dtype or not gate_out.is_contiguous():
+        raise _err(op, f"`gate_out` must be contiguous with shape {tuple(gate_shape)} and dtype {x.dtype}")
+    if M == 0:
+        return out, xq, xs, gate_out
+    if n_mod == 0 or M % n_mod != 0:
+        raise _err(op, f"x rows ({M}) must be a non-zero multiple of modulation rows ({n_mod})")
+    rc = _lib.load().phyai_fp8_adarmsnorm_quant(
+        x2.data_ptr(), x2.stride(0) if M > 1 else D, mod2.data_ptr(), mod2.stride(0) if n_mod > 1 else 3 * D,
+        n_mod, M, D, float(eps), out.data_ptr() if out is not None else None, D, gate_out.data_ptr(), D,
+        xq.data_ptr() if xq is not None else None, xs.data_ptr() if xs is not None else None, _stream_ptr())
+    _lib.check(rc, op)
+    return out, xq, xs, gate_out
+
+
+def adarmsnorm(x: torch.Tensor, modulation: torch.Tensor, eps: float = 1e-6, *,
+               out: torch.Tensor | None = None, gate_out: torch.Tensor | None = None):
+    """Adaptive RMSNorm, ``(out, gate)`` - the reference's ``phyai_kernel.triton.adarmsnorm``
+    (``phyai-kernel/phyai_kernel/triton/ada_rms_norm.py:214-221``): ``scale | shift | gate =
+    modulation``; ``out = (x * rsqrt(mean(x^2) + eps) * (1 + scale) + shift).to(x.dtype)``; each
+    modulation row serves ``rows(x) / rows(modulation)`` consecutive rows of ``x``."""
+    o, _, _, g = _adarmsnorm("adarmsnorm", x, modulation, eps, out, gate_out, False, True)
+    return o, g
+
+
+def adarmsnorm_fp8(x: torch.Tensor, modulation: torch.Tensor, eps: float = 1e-6, *,
+                   out: torch.Tensor | None = None, gate_out: torch.Tensor | None = None,
+                   want_out: bool = False):
+    """Adaptive RMSNorm feeding the per-token quantizer: ``(codes, scale, gate)`` or
+    ``(codes, scale, gate, out)`` when the bf16 tensor is wanted too."""
+    o, xq, xs, g = _adarmsnorm("adarmsnorm_fp8", x, modulation, eps, out, gate_out, True,
+                               want_out or out is not None)
+    return (xq, xs, g) if o is None else (xq, xs, g, o)
+
+
 def fp8_quant_static(x: torch.Tensor, input_scale: torch.Tensor, *,
                      out: torch.Tensor | None = None) -> torch.Tensor:
     """Static per-tensor quantization (reference ``layers/quant/fp8.py:142-148``)."""

@@ -281,3 +281,53 @@ def test_golden_fixture_regenerates_identically(tmp_path):
     assert sorted(a.files) == sorted(b.files)
     for k in a.files:
         np.testing.assert_array_equal(a[k], b[k], err_msg=k)
+
+
+# ---- norm restatements (phyai-kernel triton/rms_norm.py, ada_rms_norm.py) -----------------------
+
+def _bf16_ulp_diff(a: torch.Tensor, b: torch.Tensor) -> torch.Tensor:
+    """Distance in bf16 steps between two bf16 tensors (sign-magnitude order)."""
+    def key(t):
+        u = t.view(torch.int16).to(torch.int32) & 0xFFFF
+        return torch.where(u >= 0x8000, 0x8000 - u, u)
+    return (key(a) - key(b)).abs()
+
+
+@pytest.mark.parametrize("gemma", [False, True])
+@pytest.mark.parametrize("D", [256, 1024, 3072])
+def test_rmsnorm_oracle_against_float64_closed_form(D, gemma):
+    x = seeded((17, D), seed=D, scale=0.5)
+    w = seeded((D,), seed=D + 1, scale=0.3)
+    got = ref.rmsnorm(x, w, 1e-6, gemma)
+    x64, w64 = x.double(), w.double() + (1.0 if gemma else 0.0)
+    want = (x64 / torch.sqrt((x64 * x64).mean(-1, keepdim=True) + 1e-6) * w64)
+    d = _bf16_ulp_diff(got, want.to(torch.bfloat16))
+    assert int(d.max()) <= 1 and float((d == 0).float().mean()) > 0.995
+    # invariant: unit weight gives unit mean square
+    ones = torch.ones(D, dtype=torch.bfloat16)
+    o = ref.rmsnorm(x, ones if not gemma else torch.zeros(D, dtype=torch.bfloat16), 1e-6, gemma).double()
+    assert torch.allclose((o * o).mean(-1), torch.ones(17, dtype=torch.float64), atol=5e-3)
+
+
+def test_adarmsnorm_oracle_properties():
+    D = 1024
+    x = seeded((4, 13, D), seed=5, scale=0.5)
+    mod = seeded((4, 3 * D), seed=6, scale=0.1)
+    out, gate = ref.adarmsnorm(x, mod, 1e-6)
+    assert out.shape == x.shape and gate.shape == (4, D)
+    assert torch.equal(gate, mod[:, 2 * D:])                              # gate is a copy
+    # float64 closed form, modulation row b serving x[b, :, :]
+    x64 = x.double()
+    sc, sh = mod[:, None, :D].double(), mod[:, None, D:2 * D].double()
+    want = x64 / torch.sqrt((x64 * x64).mean(-1, keepdim=True) + 1e-6) * (1.0 + sc) + sh
+    d = _bf16_ulp_diff(out, want.to(torch.bfloat16))
+    assert int(d.max()) <= 1 and float((d == 0).float().mean()) > 0.995
+    # zero modulation reduces to the plain norm with unit weight
+    z = torch.zeros(4, 3 * D, dtype=torch.bfloat16)
+    o0, g0 = ref.adarmsnorm(x, z, 1e-6)
+    assert torch.equal(o0, ref.rmsnorm(x, torch.ones(D, dtype=torch.bfloat16), 1e-6, False))
+    assert not bool(g0.any())
+    # per-token mapping (one modulation row per x row) differs from the broadcast one only in rows
+    mod_tok = mod.repeat_interleave(13, dim=0).reshape(4, 13, 3 * D)
+    o_tok, g_tok = ref.adarmsnorm(x, mod_tok, 1e-6)
+    assert torch.equal(o_tok, out) and g_tok.shape == (4, 13, D)
