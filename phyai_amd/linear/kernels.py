@@ -19,6 +19,7 @@ import torch.nn.functional as F
 
 from phyai_amd.linear.backend import KernelProbe
 from phyai_amd.linear.registry import register_linear_kernel
+from phyai_amd.quant.types import ActivationView, Granularity
 
 _FP8_SPECS = ("fp8_per_channel", "fp8_per_tensor")
 _MIN_SM = 89   # same gate as the reference; gfx950 reports 95
@@ -48,6 +49,12 @@ class HipFp8Kernel:
         from phyai_amd import ops
 
         spec_id = layer.spec.spec_id
+        if isinstance(x, ActivationView):
+            # already quantized per token by the producer (a norm with the quantizer fused in)
+            if spec_id != "fp8_per_channel" or x.granularity is not Granularity.PER_CHANNEL or x.x_scale is None:
+                raise RuntimeError(f"HipFp8Kernel: pre-quantized activations need per-token scales and an "
+                                   f"fp8_per_channel layer, got spec_id={spec_id!r}, granularity={x.granularity}")
+            return ops.fp8_gemm(x.x, x.x_scale, layer.weight, layer.weight_scale, bias, epilogue=epilogue)
         if spec_id == "fp8_per_channel":
             return ops.fp8_linear(x, layer.weight, layer.weight_scale, bias, epilogue=epilogue)
         if spec_id == "fp8_per_tensor":

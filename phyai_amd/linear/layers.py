@@ -23,9 +23,12 @@ import torch.nn as nn
 
 from phyai_amd.linear.dispatch import get_linear_dispatcher
 from phyai_amd.quant import AllocationRequest, Bf16Spec
+from phyai_amd.quant.types import ActivationView
 
 
-def _M_of(x: torch.Tensor) -> int:
+def _M_of(x) -> int:
+    if isinstance(x, ActivationView):
+        x = x.x
     """Number of token rows: product of every dim but the last."""
     m = 1
     for s in x.shape[:-1]:
@@ -101,10 +104,17 @@ class LinearBase(nn.Module):
             hook(self)
 
     # -- the hot call -----------------------------------------------------------------
-    def _run(self, x: torch.Tensor, add_bias: bool = True, **kernel_kwargs) -> torch.Tensor:
+    def _run(self, x, add_bias: bool = True, **kernel_kwargs) -> torch.Tensor:
+        """``x`` is the bf16 activations or, for an fp8 layer, an ``ActivationView`` that a norm
+        already quantized per token (``phyai_amd.norm``): then the layer's own quantizer is skipped."""
+        quantized = isinstance(x, ActivationView)
+        if quantized and not getattr(self.spec, "needs_act_quant", False):
+            raise RuntimeError(f"{type(self).__name__}: got quantized activations but spec "
+                               f"{self.spec.spec_id!r} does not quantize its input")
         kernel = get_linear_dispatcher().select(
             spec_id=self.spec.spec_id, M=_M_of(x), N=self.output_size_per_partition,
-            K=self.input_size_per_partition, in_dtype=x.dtype, out_dtype=self.params_dtype)
+            K=self.input_size_per_partition, in_dtype=self.params_dtype if quantized else x.dtype,
+            out_dtype=self.params_dtype)
         bias = self.bias if (add_bias and not self.skip_bias_add) else None
         return kernel.apply(self, x, bias, **kernel_kwargs)
 
@@ -118,10 +128,11 @@ class LinearBase(nn.Module):
         :func:`supports_fused_epilogue` first."""
         return self._run(x, epilogue=epilogue)
 
-    def supports_fused_epilogue(self, x: torch.Tensor) -> bool:
+    def supports_fused_epilogue(self, x) -> bool:
         kernel = get_linear_dispatcher().select(
             spec_id=self.spec.spec_id, M=_M_of(x), N=self.output_size_per_partition,
-            K=self.input_size_per_partition, in_dtype=x.dtype, out_dtype=self.params_dtype)
+            K=self.input_size_per_partition,
+            in_dtype=self.params_dtype if isinstance(x, ActivationView) else x.dtype, out_dtype=self.params_dtype)
         return getattr(kernel, "name", "") == "hip_fp8" and not self.skip_bias_add
 
 

@@ -111,3 +111,53 @@ def test_norm_argument_errors(dev):
                     torch.zeros(12288, dtype=torch.bfloat16, device=dev))
     empty, g = ops.adarmsnorm(x[:0], torch.zeros(0, 192, dtype=torch.bfloat16, device=dev))
     assert empty.shape == (0, 64) and g.shape == (0, 64)
+
+
+def test_norm_modules_feed_fp8_layers(dev):
+    """GemmaRMSNorm / AdaRMSNorm ``forward_fp8`` -> fp8 layer == bf16 norm -> same layer, bit for bit,
+    and DenseMLP takes the quantized view through its fused gate_up epilogue."""
+    import phyai_amd.linear as L
+    from phyai_amd.linear.layers import ColumnParallelLinear
+    from phyai_amd.mlp import DenseMLP
+    from phyai_amd.norm import AdaRMSNorm, GemmaRMSNorm
+    from phyai_amd.quant import Fp8Spec
+    from phyai_amd.quant.types import ActivationView, Granularity
+
+    torch.cuda.set_device(dev)
+    L.init()
+    try:
+        _norm_modules_body(dev, GemmaRMSNorm, AdaRMSNorm, ColumnParallelLinear, DenseMLP, Fp8Spec,
+                           ActivationView, Granularity)
+    finally:
+        L._reset_for_test()
+
+
+def _norm_modules_body(dev, GemmaRMSNorm, AdaRMSNorm, ColumnParallelLinear, DenseMLP, Fp8Spec,
+                       ActivationView, Granularity):
+    D, N, M = 1024, 2560, 50
+    torch.manual_seed(4)
+    norm = GemmaRMSNorm(D, device=dev, prefix="layers.0.input_layernorm")
+    norm.weight.data.copy_((torch.randn(D) * 0.1).to(torch.bfloat16))
+    layer = ColumnParallelLinear(D, N, bias=False, params_dtype=torch.bfloat16, spec=Fp8Spec(), device=dev)
+    layer.spec.quantize_weight_(layer, (torch.randn(N, D) * 0.02).to(torch.bfloat16).to(dev))
+    x = (torch.randn(M, D) * 0.8).to(torch.bfloat16).to(dev)
+    view = norm.forward_fp8(x)
+    assert isinstance(view, ActivationView) and view.granularity is Granularity.PER_CHANNEL
+    y_fused, _ = layer(view)
+    y_plain, _ = layer(norm(x))
+    assert torch.equal(y_fused, y_plain)
+
+    ada = AdaRMSNorm(D, 1024, device=dev)
+    ada.dense.weight.data.copy_((torch.randn(3 * D, 1024) * 0.01).to(torch.bfloat16))
+    cond = torch.randn(1, 1024).to(torch.bfloat16).to(dev)
+    table = ada.project_modulation(cond)
+    v2, gate = ada.forward_fp8(x, modulation=table)
+    n2, gate2 = ada(x, modulation=table)
+    assert torch.equal(gate, gate2) and gate.shape == (1, D)
+    assert torch.equal(layer(v2)[0], layer(n2)[0])
+
+    mlp = DenseMLP(D, 4096, activation="gelu_tanh", gated=True, bias=False, params_dtype=torch.bfloat16,
+                   spec_in=Fp8Spec(), spec_out=Fp8Spec())
+    for lin, shape in ((mlp.gate_up_proj, (8192, D)), (mlp.down_proj, (D, 4096))):
+        lin.spec.quantize_weight_(lin, (torch.randn(*shape) * 0.02).to(torch.bfloat16).to(dev))
+    assert torch.equal(mlp(v2), mlp(n2))
