@@ -119,6 +119,27 @@ int phyai_fp8_linear(const void *x, int64_t ldx, const void *w, const float *w_s
                      void *stream);
 
 /*
+ * The same two with the gated residual of a decoder layer fused into the epilogue:
+ *     out[m, n] = bf16( residual[m, n] + bf16(acc * x_scale[m] * w_scale[n] + bias[n]) * gate[m / g, n] )
+ * computed in fp32 and rounded once, i.e. torch.addcmul(residual, linear(x), gate) on bf16
+ * tensors (models/pi05/modeling_pi05.py:822-826,835: `h = torch.addcmul(residual, out, gate)`
+ * after o_proj and after the MLP's down_proj).  residual: [M, N] bf16, row stride ld_res;
+ * gate: [gate_rows, N] bf16, row stride ld_gate, M a multiple of gate_rows and g = M / gate_rows
+ * (the gate of an adaptive norm has one row per modulation row).  No activation epilogue.
+ * out may alias residual.
+ */
+int phyai_fp8_gemm_addcmul(const void *xq, const float *x_scale, int x_scale_is_scalar,
+                           const void *w, const float *w_scale, const void *bias,
+                           const void *residual, int64_t ld_res, const void *gate, int64_t ld_gate,
+                           int64_t gate_rows, void *out, int64_t ldo, int64_t M, int64_t N,
+                           int64_t K, void *workspace, size_t workspace_bytes, void *stream);
+int phyai_fp8_linear_addcmul(const void *x, int64_t ldx, const void *w, const float *w_scale,
+                             const void *bias, const void *residual, int64_t ld_res,
+                             const void *gate, int64_t ld_gate, int64_t gate_rows, void *out,
+                             int64_t ldo, int64_t M, int64_t N, int64_t K, void *workspace,
+                             size_t workspace_bytes, void *stream);
+
+/*
  * RMSNorm whose output feeds the quantizer without a round trip through memory.
  * Replaces phyai_kernel.triton.rmsnorm / gemma_rmsnorm
  * (phyai-kernel/phyai_kernel/triton/rms_norm.py:42-75: fp32 reduction,

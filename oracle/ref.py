@@ -129,3 +129,12 @@ def adarmsnorm(x: torch.Tensor, modulation: torch.Tensor, eps: float = 1e-6) -> 
     out = (x_hat * (1.0 + scale) + shift).to(x.dtype).reshape(x.shape)
     gate = modulation[..., 2 * D:].to(x.dtype).contiguous()
     return out, gate
+
+
+def addcmul(residual: torch.Tensor, y: torch.Tensor, gate: torch.Tensor) -> torch.Tensor:
+    """``residual + y * gate`` on bf16 tensors, fp32 inside, one rounding - torch.addcmul as the
+    decoder layer calls it (models/pi05/modeling_pi05.py:826,835); ``gate`` broadcasts over rows."""
+    g = gate
+    if g.shape != y.shape:
+        g = g.reshape(-1, g.shape[-1]).repeat_interleave(y.reshape(-1, y.shape[-1]).shape[0] // g.reshape(-1, g.shape[-1]).shape[0], dim=0).reshape(y.shape)
+    return (residual.float() + y.float() * g.float()).to(residual.dtype)

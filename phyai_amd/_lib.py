@@ -26,6 +26,10 @@ SIGNATURES: dict[str, tuple[object, list[object]]] = {
     "phyai_fp8_linear_workspace_bytes": (_sz, [_i64, _i64, _i64, _int]),
     "phyai_fp8_gemm": (_int, [_vp, _vp, _int, _vp, _vp, _vp, _vp, _i64, _i64, _i64, _i64, _int, _vp, _sz, _vp]),
     "phyai_fp8_linear": (_int, [_vp, _i64, _vp, _vp, _vp, _vp, _i64, _i64, _i64, _i64, _int, _vp, _sz, _vp]),
+    "phyai_fp8_gemm_addcmul": (_int, [_vp, _vp, _int, _vp, _vp, _vp, _vp, _i64, _vp, _i64, _i64, _vp, _i64, _i64, _i64,
+                                      _i64, _vp, _sz, _vp]),
+    "phyai_fp8_linear_addcmul": (_int, [_vp, _i64, _vp, _vp, _vp, _vp, _i64, _vp, _i64, _i64, _vp, _i64, _i64, _i64,
+                                        _i64, _vp, _sz, _vp]),
     "phyai_fp8_rmsnorm_quant": (_int, [_vp, _i64, _vp, _int, _i64, _i64, ctypes.c_float, _vp, _i64, _vp, _vp, _vp]),
     "phyai_fp8_adarmsnorm_quant": (_int, [_vp, _i64, _vp, _i64, _i64, _i64, _i64, ctypes.c_float, _vp, _i64, _vp,
                                           _i64, _vp, _vp, _vp]),

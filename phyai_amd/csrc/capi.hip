@@ -109,25 +109,46 @@ size_t phyai_fp8_linear_workspace_bytes(int64_t M, int64_t N, int64_t K, int epi
     return carve(M, N, K, epilogue).total;
 }
 
-int phyai_fp8_gemm(const void* xq, const float* x_scale, int x_scale_is_scalar, const void* w,
-                   const float* w_scale, const void* bias, void* out, int64_t ldo, int64_t M,
-                   int64_t N, int64_t K, int epilogue, void* workspace, size_t workspace_bytes,
-                   void* stream) {
+namespace {
+// Gated residual of phyai_fp8_gemm_addcmul / phyai_fp8_linear_addcmul; all null for the plain forms.
+struct ResidualSpec {
+    const void* residual;
+    int64_t ld_res;
+    const void* gate;
+    int64_t ld_gate;
+    int64_t gate_rows;
+};
+
+int check_residual(const char* fn, const ResidualSpec& r, int64_t M, int64_t N, int epilogue) {
+    if (!r.residual && !r.gate) return 0;
+    if (!r.residual || !r.gate) return fail(PHYAI_FP8_EINVAL, "%s: residual and gate go together", fn);
+    if (epilogue != PHYAI_FP8_EPI_NONE) return fail(PHYAI_FP8_EINVAL, "%s: a gated residual excludes an activation epilogue", fn);
+    if (!aligned(r.residual, 16) || !aligned(r.gate, 16) || r.ld_res < N || r.ld_gate < N || r.ld_res % 8 != 0 || r.ld_gate % 8 != 0)
+        return fail(PHYAI_FP8_EINVAL, "%s: residual and gate must be 16-byte aligned with row strides >= N, multiples of 8", fn);
+    if (r.gate_rows <= 0 || (M > 0 && M % r.gate_rows != 0))
+        return fail(PHYAI_FP8_EINVAL, "%s: M=%lld must be a multiple of the gate rows (%lld)", fn, (long long)M, (long long)r.gate_rows);
+    return 0;
+}
+
+int run_gemm(const char* fn, const void* xq, const float* x_scale, int x_scale_is_scalar, const void* w,
+             const float* w_scale, const void* bias, const ResidualSpec& res, void* out, int64_t ldo, int64_t M,
+             int64_t N, int64_t K, int epilogue, void* workspace, size_t workspace_bytes, void* stream) {
     if (M < 0 || N <= 0 || K <= 0)
-        return fail(PHYAI_FP8_EINVAL, "phyai_fp8_gemm: bad shape M=%lld N=%lld K=%lld", (long long)M, (long long)N, (long long)K);
+        return fail(PHYAI_FP8_EINVAL, "%s: bad shape M=%lld N=%lld K=%lld", fn, (long long)M, (long long)N, (long long)K);
     if (int rc = check_epilogue(epilogue, N)) return rc;
     if (K % 16 != 0 || N % 16 != 0)
-        return fail(PHYAI_FP8_EUNSUPPORTED, "phyai_fp8_gemm: K=%lld and N=%lld must be multiples of 16", (long long)K, (long long)N);
+        return fail(PHYAI_FP8_EUNSUPPORTED, "%s: K=%lld and N=%lld must be multiples of 16", fn, (long long)K, (long long)N);
+    if (int rc = check_residual(fn, res, M, N, epilogue)) return rc;
     if (M == 0) return PHYAI_FP8_OK;
-    if (!xq || !x_scale || !w || !w_scale || !out) return fail(PHYAI_FP8_EINVAL, "phyai_fp8_gemm: null pointer");
-    if (!aligned(xq, 16) || !aligned(w, 16)) return fail(PHYAI_FP8_EINVAL, "phyai_fp8_gemm: xq and w must be 16-byte aligned");
+    if (!xq || !x_scale || !w || !w_scale || !out) return fail(PHYAI_FP8_EINVAL, "%s: null pointer", fn);
+    if (!aligned(xq, 16) || !aligned(w, 16)) return fail(PHYAI_FP8_EINVAL, "%s: xq and w must be 16-byte aligned", fn);
     const int64_t n_out = phyai::epi_is_gated(epilogue) ? N / 2 : N;
-    if (ldo < n_out) return fail(PHYAI_FP8_EINVAL, "phyai_fp8_gemm: ldo=%lld < output width %lld", (long long)ldo, (long long)n_out);
+    if (ldo < n_out) return fail(PHYAI_FP8_EINVAL, "%s: ldo=%lld < output width %lld", fn, (long long)ldo, (long long)n_out);
     if (M * K >= kMaxElems || N * K >= kMaxElems || M * ldo >= kMaxElems * 2)
-        return fail(PHYAI_FP8_EUNSUPPORTED, "phyai_fp8_gemm: operand larger than 2^31 elements");
-    if (workspace && !aligned(workspace, 256)) return fail(PHYAI_FP8_EINVAL, "phyai_fp8_gemm: workspace must be 256-byte aligned");
+        return fail(PHYAI_FP8_EUNSUPPORTED, "%s: operand larger than 2^31 elements", fn);
+    if (workspace && !aligned(workspace, 256)) return fail(PHYAI_FP8_EINVAL, "%s: workspace must be 256-byte aligned", fn);
 
-    phyai::GemmProblem g;
+    phyai::GemmProblem g = {};
     g.xq = static_cast<const uint8_t*>(xq);
     g.x_scale = x_scale;
     g.x_scale_is_scalar = x_scale_is_scalar ? 1 : 0;
@@ -140,31 +161,75 @@ int phyai_fp8_gemm(const void* xq, const float* x_scale, int x_scale_is_scalar, 
     g.epilogue = epilogue;
     g.workspace = workspace;
     g.workspace_bytes = workspace_bytes;
+    g.gate_group = 1;
+    if (res.residual) {
+        g.residual = static_cast<const uint16_t*>(res.residual);
+        g.ld_res = res.ld_res;
+        g.gate = static_cast<const uint16_t*>(res.gate);
+        g.ld_gate = res.ld_gate;
+        g.gate_group = (int)(M / res.gate_rows);
+    }
     const int rc = phyai::launch_gemm(g, static_cast<hipStream_t>(stream));
     if (rc == -3)
-        return fail(PHYAI_FP8_EWORKSPACE, "phyai_fp8_gemm: workspace of %zu bytes is too small, need %zu",
+        return fail(PHYAI_FP8_EWORKSPACE, "%s: workspace of %zu bytes is too small, need %zu", fn,
                     workspace ? workspace_bytes : (size_t)0, phyai::gemm_workspace_bytes(M, N, K, epilogue, ldo));
-    if (rc != 0) return fail(PHYAI_FP8_EUNSUPPORTED, "phyai_fp8_gemm: no kernel for this problem (rc=%d)", rc);
-    return check_launch("phyai_fp8_gemm");
+    if (rc != 0) return fail(PHYAI_FP8_EUNSUPPORTED, "%s: no kernel for this problem (rc=%d)", fn, rc);
+    return check_launch(fn);
+}
+
+int run_linear(const char* fn, const void* x, int64_t ldx, const void* w, const float* w_scale, const void* bias,
+               const ResidualSpec& res, void* out, int64_t ldo, int64_t M, int64_t N, int64_t K, int epilogue,
+               void* workspace, size_t workspace_bytes, void* stream) {
+    if (M < 0 || N <= 0 || K <= 0)
+        return fail(PHYAI_FP8_EINVAL, "%s: bad shape M=%lld N=%lld K=%lld", fn, (long long)M, (long long)N, (long long)K);
+    if (M == 0) return PHYAI_FP8_OK;
+    const LinearCarve c = carve(M, N, K, epilogue);
+    if (!workspace || workspace_bytes < c.total)
+        return fail(PHYAI_FP8_EWORKSPACE, "%s: workspace of %zu bytes is too small, need %zu", fn,
+                    workspace ? workspace_bytes : (size_t)0, c.total);
+    if (!aligned(workspace, 256)) return fail(PHYAI_FP8_EINVAL, "%s: workspace must be 256-byte aligned", fn);
+    uint8_t* ws = static_cast<uint8_t*>(workspace);
+    void* xq = ws + c.xq_off;
+    float* xs = reinterpret_cast<float*>(ws + c.xs_off);
+    if (int rc = phyai_fp8_quant_rowwise(x, M, K, ldx, xq, xs, stream)) return rc;
+    return run_gemm(fn, xq, xs, 0, w, w_scale, bias, res, out, ldo, M, N, K, epilogue, workspace, c.gemm_bytes, stream);
+}
+}  // namespace
+
+int phyai_fp8_gemm(const void* xq, const float* x_scale, int x_scale_is_scalar, const void* w,
+                   const float* w_scale, const void* bias, void* out, int64_t ldo, int64_t M,
+                   int64_t N, int64_t K, int epilogue, void* workspace, size_t workspace_bytes,
+                   void* stream) {
+    return run_gemm("phyai_fp8_gemm", xq, x_scale, x_scale_is_scalar, w, w_scale, bias, ResidualSpec{}, out, ldo,
+                    M, N, K, epilogue, workspace, workspace_bytes, stream);
+}
+
+int phyai_fp8_gemm_addcmul(const void* xq, const float* x_scale, int x_scale_is_scalar, const void* w,
+                           const float* w_scale, const void* bias, const void* residual, int64_t ld_res,
+                           const void* gate, int64_t ld_gate, int64_t gate_rows, void* out, int64_t ldo,
+                           int64_t M, int64_t N, int64_t K, void* workspace, size_t workspace_bytes,
+                           void* stream) {
+    if (!residual || !gate) return fail(PHYAI_FP8_EINVAL, "phyai_fp8_gemm_addcmul: null residual or gate");
+    const ResidualSpec r = {residual, ld_res, gate, ld_gate, gate_rows};
+    return run_gemm("phyai_fp8_gemm_addcmul", xq, x_scale, x_scale_is_scalar, w, w_scale, bias, r, out, ldo, M, N,
+                    K, PHYAI_FP8_EPI_NONE, workspace, workspace_bytes, stream);
 }
 
 int phyai_fp8_linear(const void* x, int64_t ldx, const void* w, const float* w_scale,
                      const void* bias, void* out, int64_t ldo, int64_t M, int64_t N, int64_t K,
                      int epilogue, void* workspace, size_t workspace_bytes, void* stream) {
-    if (M < 0 || N <= 0 || K <= 0)
-        return fail(PHYAI_FP8_EINVAL, "phyai_fp8_linear: bad shape M=%lld N=%lld K=%lld", (long long)M, (long long)N, (long long)K);
-    if (M == 0) return PHYAI_FP8_OK;
-    const LinearCarve c = carve(M, N, K, epilogue);
-    if (!workspace || workspace_bytes < c.total)
-        return fail(PHYAI_FP8_EWORKSPACE, "phyai_fp8_linear: workspace of %zu bytes is too small, need %zu",
-                    workspace ? workspace_bytes : (size_t)0, c.total);
-    if (!aligned(workspace, 256)) return fail(PHYAI_FP8_EINVAL, "phyai_fp8_linear: workspace must be 256-byte aligned");
-    uint8_t* ws = static_cast<uint8_t*>(workspace);
-    void* xq = ws + c.xq_off;
-    float* xs = reinterpret_cast<float*>(ws + c.xs_off);
-    if (int rc = phyai_fp8_quant_rowwise(x, M, K, ldx, xq, xs, stream)) return rc;
-    return phyai_fp8_gemm(xq, xs, 0, w, w_scale, bias, out, ldo, M, N, K, epilogue, workspace,
-                          c.gemm_bytes, stream);
+    return run_linear("phyai_fp8_linear", x, ldx, w, w_scale, bias, ResidualSpec{}, out, ldo, M, N, K, epilogue,
+                      workspace, workspace_bytes, stream);
+}
+
+int phyai_fp8_linear_addcmul(const void* x, int64_t ldx, const void* w, const float* w_scale,
+                             const void* bias, const void* residual, int64_t ld_res, const void* gate,
+                             int64_t ld_gate, int64_t gate_rows, void* out, int64_t ldo, int64_t M,
+                             int64_t N, int64_t K, void* workspace, size_t workspace_bytes, void* stream) {
+    if (!residual || !gate) return fail(PHYAI_FP8_EINVAL, "phyai_fp8_linear_addcmul: null residual or gate");
+    const ResidualSpec r = {residual, ld_res, gate, ld_gate, gate_rows};
+    return run_linear("phyai_fp8_linear_addcmul", x, ldx, w, w_scale, bias, r, out, ldo, M, N, K,
+                      PHYAI_FP8_EPI_NONE, workspace, workspace_bytes, stream);
 }
 
 namespace {

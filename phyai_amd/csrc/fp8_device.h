@@ -106,6 +106,18 @@ __device__ __forceinline__ float apply_act(float v) {
     else return v;
 }
 
+// residual + y * gate on four consecutive columns; y is the linear's bf16 output.  The product of
+// two bf16 values is exact in fp32, so this equals torch.addcmul's single rounding whether or
+// not the multiply and the add are contracted.
+__device__ __forceinline__ void addcmul4(float* y, uint2 res, uint2 gate) {
+    const float r[4] = {bf16_bits_to_f32(res.x & 0xFFFFu), __uint_as_float(res.x & 0xFFFF0000u),
+                        bf16_bits_to_f32(res.y & 0xFFFFu), __uint_as_float(res.y & 0xFFFF0000u)};
+    const float g[4] = {bf16_bits_to_f32(gate.x & 0xFFFFu), __uint_as_float(gate.x & 0xFFFF0000u),
+                        bf16_bits_to_f32(gate.y & 0xFFFFu), __uint_as_float(gate.y & 0xFFFF0000u)};
+#pragma unroll
+    for (int e = 0; e < 4; ++e) y[e] = r[e] + bf16_bits_to_f32(f32_to_bf16_bits(y[e])) * g[e];
+}
+
 // Round an fp32 value through bf16 (the reference materialises the GEMM output
 // as a bf16 tensor before the activation kernel reads it).
 __device__ __forceinline__ float round_bf16(float v) { return bf16_bits_to_f32(f32_to_bf16_bits(v)); }

@@ -59,6 +59,7 @@ struct BigArgs {
     float* __restrict__ partials;
     int* __restrict__ counters;
     int m_tiles, n_tiles;            // tile grid; the launch is 1-D over it (see big_tile_of)
+    ResidualArgs res;
 };
 
 // Workgroup id -> tile.  Workgroups go to the 8 XCDs round-robin (id % 8) and each XCD has its own
@@ -399,6 +400,17 @@ __global__ __launch_bounds__(256) void gemm_fp8_big_kernel(const BigArgs p) {
                     o[1] = apply_act<EPI>(__uint_as_float(g01 & 0xFFFF0000u));
                     o[2] = apply_act<EPI>(__uint_as_float(g23 << 16));
                     o[3] = apply_act<EPI>(__uint_as_float(g23 & 0xFFFF0000u));
+                } else {
+                    if (p.res.residual != nullptr) {       // out = residual + bf16(linear) * gate
+                        const int m = m0 + wm * WM + row;
+                        const int n = nbase + j * 32 + 8 * g + 4 * h;
+                        if (m < p.M && n < n_lim) {
+                            const uint2 rs = *reinterpret_cast<const uint2*>(p.res.residual + (int64_t)m * p.res.ld_res + n);
+                            const uint2 gt = *reinterpret_cast<const uint2*>(
+                                p.res.gate + (int64_t)(m / p.res.gate_group) * p.res.ld_gate + n);
+                            addcmul4(o, rs, gt);
+                        }
+                    }
                 }
                 uint2 w;
                 w.x = pack_bf16x2(o[0], o[1]);
@@ -503,6 +515,7 @@ int launch_gemm_big(const GemmProblem& g, const BigPlan& pl, hipStream_t st) {
     a.a = g.xq; a.b = g.w; a.a_scale = g.x_scale; a.b_scale = g.w_scale; a.bias = g.bias;
     a.out = g.out; a.ldo = g.ldo; a.M = g.M; a.N = g.N; a.K = g.K;
     a.a_scale_scalar = g.x_scale_is_scalar;
+    a.res = residual_of(g);
     a.k_per_split = g.K / pl.splits;
     a.counters = static_cast<int*>(g.workspace);
     a.partials = g.workspace ? reinterpret_cast<float*>(static_cast<uint8_t*>(g.workspace) + kGemmHeaderBytes) : nullptr;

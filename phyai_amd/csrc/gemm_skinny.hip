@@ -50,6 +50,7 @@ struct SkinnyArgs {
     int M, N, K;
     int x_scale_scalar;
     int rounds;  // K steps are consumed in rounds of SK_WAVES * KPW
+    ResidualArgs res;
 };
 
 constexpr int SK_WAVES = 8;
@@ -100,6 +101,13 @@ __global__ __launch_bounds__(SK_THREADS) void gemm_fp8_skinny_kernel(const Skinn
         if constexpr (GATED) bu2 = *reinterpret_cast<const uint2*>(p.bias + half_n + e_n_safe);
     }
     const float sa = p.x_scale[(p.x_scale_scalar || !e_live) ? 0 : e_m];
+    uint2 res2 = make_uint2(0, 0), gate2 = make_uint2(0, 0);   // gated residual, requested early too
+    if constexpr (EPI == EPI_NONE) {
+        if (p.res.residual != nullptr && e_live) {
+            res2 = *reinterpret_cast<const uint2*>(p.res.residual + (int64_t)e_m * p.res.ld_res + e_n);
+            gate2 = *reinterpret_cast<const uint2*>(p.res.gate + (int64_t)(e_m / p.res.gate_group) * p.res.ld_gate + e_n);
+        }
+    }
 
     // ---- operand row pointers ---------------------------------------------------------
     const uint8_t* wrow[NT];
@@ -187,6 +195,7 @@ __global__ __launch_bounds__(SK_THREADS) void gemm_fp8_skinny_kernel(const Skinn
     const float buf[4] = {bf16_bits_to_f32(bu2.x & 0xFFFFu), bf16_bits_to_f32(bu2.x >> 16),
                           bf16_bits_to_f32(bu2.y & 0xFFFFu), bf16_bits_to_f32(bu2.y >> 16)};
     uint32_t o[4];
+    float vf[4];
 #pragma unroll
     for (int r = 0; r < 4; ++r) {
         float v = g[r] * (sa * sw4[r]) + bwf[r];
@@ -196,8 +205,13 @@ __global__ __launch_bounds__(SK_THREADS) void gemm_fp8_skinny_kernel(const Skinn
         } else if constexpr (EPI != EPI_NONE) {
             v = apply_act<EPI>(round_bf16(v));
         }
-        o[r] = f32_to_bf16_bits(v);
+        vf[r] = v;
     }
+    if constexpr (EPI == EPI_NONE) {
+        if (p.res.residual != nullptr) addcmul4(vf, res2, gate2);
+    }
+#pragma unroll
+    for (int r = 0; r < 4; ++r) o[r] = f32_to_bf16_bits(vf[r]);
     if (e_live)
         *reinterpret_cast<uint2*>(p.out + (int64_t)e_m * p.ldo + e_n) =
             make_uint2(o[0] | (o[1] << 16), o[2] | (o[3] << 16));
@@ -288,6 +302,7 @@ int launch_gemm_skinny(const GemmProblem& g, const SkinnyPlan& pl, hipStream_t s
     a.out = g.out; a.ldo = g.ldo; a.M = g.M; a.N = g.N; a.K = g.K;
     a.x_scale_scalar = g.x_scale_is_scalar;
     a.rounds = pl.rounds;
+    a.res = residual_of(g);
     switch (g.epilogue) {
     case EPI_NONE: return sk_launch_epi<EPI_NONE>(a, pl, st);
     case EPI_GEGLU_TANH: return sk_launch_epi<EPI_GEGLU_TANH>(a, pl, st);

@@ -46,6 +46,7 @@ struct TileArgs {
     int M, N, K;
     int a_scale_scalar;
     int k_tiles_per_split;  // in BK slabs
+    ResidualArgs res;
 };
 
 __device__ __forceinline__ v8i lds_frag(const uint8_t* buf, int row, int ks, int h) {
@@ -232,7 +233,15 @@ __global__ __launch_bounds__(256) void gemm_fp8_tile_kernel(const TileArgs p) {
                 } else if constexpr (EPI != EPI_NONE) {
                     v = apply_act<EPI>(round_bf16(v));
                 }
-                if (m < p.M && n_ok) p.out[(int64_t)m * p.ldo + n_out] = (uint16_t)f32_to_bf16_bits(v);
+                if (m < p.M && n_ok) {
+                    if constexpr (EPI == EPI_NONE) {
+                        if (p.res.residual != nullptr)
+                            v = bf16_bits_to_f32(p.res.residual[(int64_t)m * p.res.ld_res + n_out]) +
+                                round_bf16(v) *
+                                    bf16_bits_to_f32(p.res.gate[(int64_t)(m / p.res.gate_group) * p.res.ld_gate + n_out]);
+                    }
+                    p.out[(int64_t)m * p.ldo + n_out] = (uint16_t)f32_to_bf16_bits(v);
+                }
             }
         }
     }
@@ -370,6 +379,7 @@ int launch_gemm(const GemmProblem& g, hipStream_t st) {
     a.a = g.xq; a.b = g.w; a.a_scale = g.x_scale; a.b_scale = g.w_scale; a.bias = g.bias;
     a.out = g.out; a.ldo = g.ldo; a.M = g.M; a.N = g.N; a.K = g.K;
     a.a_scale_scalar = g.x_scale_is_scalar;
+    a.res = residual_of(g);
     a.counters = static_cast<int*>(g.workspace);
     a.partials = g.workspace ? reinterpret_cast<float*>(static_cast<uint8_t*>(g.workspace) + kHeaderBytes) : nullptr;
     const int slabs = ceil_div(g.K, BK);

@@ -48,7 +48,28 @@ struct GemmProblem {
     int epilogue;
     void* workspace;        // header (counters) + split-K partials
     size_t workspace_bytes;
+    // Gated residual (epilogue NONE only): out = residual + bf16(linear) * gate, in fp32, rounded
+    // once.  gate row of token row m is m / gate_group.  Null residual: plain output.
+    const uint16_t* residual;  // [M, N] bf16
+    int64_t ld_res;
+    const uint16_t* gate;      // [M / gate_group, N] bf16
+    int64_t ld_gate;
+    int gate_group;
 };
+
+// What the kernels need of the above, by value.
+struct ResidualArgs {
+    const uint16_t* residual;
+    const uint16_t* gate;
+    int64_t ld_res, ld_gate;
+    int gate_group;
+};
+inline ResidualArgs residual_of(const GemmProblem& g) {
+    ResidualArgs r;
+    r.residual = g.residual; r.gate = g.gate; r.ld_res = g.ld_res; r.ld_gate = g.ld_gate;
+    r.gate_group = g.gate_group > 0 ? g.gate_group : 1;
+    return r;
+}
 
 constexpr size_t kGemmHeaderBytes = 16384;  // split-K arrival counters (4096 ints) at the workspace start
 

@@ -43,9 +43,11 @@ class HipFp8Kernel:
         return probe.K % 16 == 0 and probe.N % 16 == 0
 
     def apply(self, layer: torch.nn.Module, x: torch.Tensor, bias: torch.Tensor | None,
-              *, epilogue=None) -> torch.Tensor:
-        """``epilogue`` is an extension over the reference protocol: ``DenseMLP`` passes the
-        gated activation here so that it runs inside the GEMM kernel."""
+              *, epilogue=None, residual: torch.Tensor | None = None,
+              gate: torch.Tensor | None = None) -> torch.Tensor:
+        """``epilogue`` / ``residual`` + ``gate`` are extensions over the reference protocol:
+        ``DenseMLP`` passes the gated activation here so that it runs inside the GEMM kernel, and a
+        decoder layer its ``addcmul(residual, out, gate)`` (``forward_addcmul`` of the layers)."""
         from phyai_amd import ops
 
         spec_id = layer.spec.spec_id
@@ -54,13 +56,15 @@ class HipFp8Kernel:
             if spec_id != "fp8_per_channel" or x.granularity is not Granularity.PER_CHANNEL or x.x_scale is None:
                 raise RuntimeError(f"HipFp8Kernel: pre-quantized activations need per-token scales and an "
                                    f"fp8_per_channel layer, got spec_id={spec_id!r}, granularity={x.granularity}")
-            return ops.fp8_gemm(x.x, x.x_scale, layer.weight, layer.weight_scale, bias, epilogue=epilogue)
+            return ops.fp8_gemm(x.x, x.x_scale, layer.weight, layer.weight_scale, bias, epilogue=epilogue,
+                                residual=residual, gate=gate)
         if spec_id == "fp8_per_channel":
-            return ops.fp8_linear(x, layer.weight, layer.weight_scale, bias, epilogue=epilogue)
+            return ops.fp8_linear(x, layer.weight, layer.weight_scale, bias, epilogue=epilogue,
+                                  residual=residual, gate=gate)
         if spec_id == "fp8_per_tensor":
             act = layer.spec.quantize_activation(x, layer)
             return ops.fp8_gemm(act.x, layer.input_scale, layer.weight, layer.weight_scale, bias,
-                                epilogue=epilogue)
+                                epilogue=epilogue, residual=residual, gate=gate)
         raise RuntimeError(f"HipFp8Kernel got unhandled spec_id={spec_id!r}")
 
 

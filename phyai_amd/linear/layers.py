@@ -128,6 +128,16 @@ class LinearBase(nn.Module):
         :func:`supports_fused_epilogue` first."""
         return self._run(x, epilogue=epilogue)
 
+    def forward_addcmul(self, x, residual: torch.Tensor, gate: torch.Tensor) -> torch.Tensor:
+        """``torch.addcmul(residual, self(x)[0], gate)`` with the multiply-add inside the GEMM epilogue
+        (the gated residual after ``o_proj`` / ``down_proj``, reference
+        ``models/pi05/modeling_pi05.py:826,835``).  Falls back to the separate op for kernels
+        without the extension."""
+        if self.supports_fused_epilogue(x):
+            return self._run(x, residual=residual, gate=gate)
+        y, _ = self.forward(x)
+        return torch.addcmul(residual, y, gate)
+
     def supports_fused_epilogue(self, x) -> bool:
         kernel = get_linear_dispatcher().select(
             spec_id=self.spec.spec_id, M=_M_of(x), N=self.output_size_per_partition,

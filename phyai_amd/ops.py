@@ -318,9 +318,38 @@ def _out_for(op: str, lead: tuple[int, ...], n_out: int, out: torch.Tensor | Non
     return out
 
 
+def _check_addcmul(op: str, residual, gate, lead: tuple[int, ...], M: int, N: int, epi: int, device):
+    """Validate the gated-residual pair; returns ``(residual2d, gate2d)`` or ``(None, None)``."""
+    if residual is None and gate is None:
+        return None, None
+    if residual is None or gate is None:
+        raise _err(op, "residual and gate go together")
+    if epi != EPI_NONE:
+        raise _err(op, "a gated residual excludes an activation epilogue")
+    for name, t in (("residual", residual), ("gate", gate)):
+        if not (isinstance(t, torch.Tensor) and t.is_cuda and t.dtype == torch.bfloat16 and t.shape[-1] == N):
+            raise _err(op, f"{name} must be a bfloat16 GPU tensor with last dim {N}")
+    if tuple(residual.shape) != (*lead, N):
+        raise _err(op, f"residual must have shape {(*lead, N)}, got {tuple(residual.shape)}")
+    r2 = residual.reshape(-1, N)
+    g2 = gate.reshape(-1, N)
+    if not r2.is_contiguous():
+        r2 = r2.contiguous()
+    if not g2.is_contiguous():
+        g2 = g2.contiguous()
+    if g2.shape[0] == 0 or M % g2.shape[0] != 0:
+        raise _err(op, f"rows ({M}) must be a non-zero multiple of gate rows ({g2.shape[0]})")
+    return r2, g2
+
+
 def fp8_gemm(xq: torch.Tensor, x_scale: torch.Tensor, weight: torch.Tensor, weight_scale: torch.Tensor,
-             bias: torch.Tensor | None = None, *, epilogue=None, out: torch.Tensor | None = None) -> torch.Tensor:
+             bias: torch.Tensor | None = None, *, epilogue=None, out: torch.Tensor | None = None,
+             residual: torch.Tensor | None = None, gate: torch.Tensor | None = None) -> torch.Tensor:
     """``bf16(act((xq @ weight.T) * x_scale * weight_scale + bias))`` on quantized inputs.
+
+    With ``residual`` and ``gate`` the result is ``torch.addcmul(residual, y, gate)`` of that
+    linear output ``y`` (reference ``models/pi05/modeling_pi05.py:826,835``), in the same kernel;
+    ``gate`` may have fewer rows than ``residual`` (one per modulation row).
 
     ``x_scale`` has one element per token row, or a single element (static
     per-tensor scale).  Replaces the ``torch._scaled_mm`` call at reference
@@ -343,19 +372,27 @@ def fp8_gemm(xq: torch.Tensor, x_scale: torch.Tensor, weight: torch.Tensor, weig
     scalar = 1 if (xs.numel() == 1 and M != 1) else 0
     bias_ptr = _check_bias(op, bias, N)
     n_out = N // 2 if epi in _GATED else N
+    r2, g2 = _check_addcmul(op, residual, gate, tuple(xq.shape[:-1]), M, N, epi, xq.device)
     out = _out_for(op, tuple(xq.shape[:-1]), n_out, out, xq.device)
     if M == 0:
         return out
     ws = _workspace_for(M, N, K, epi, xq.device)
-    rc = _lib.load().phyai_fp8_gemm(x2.data_ptr(), xs.data_ptr(), scalar, weight.data_ptr(),
-                                     weight_scale.data_ptr(), bias_ptr, out.data_ptr(), n_out, M, N, K, epi,
-                                     ws.data_ptr(), ws.numel(), _stream_ptr())
+    if r2 is not None:
+        rc = _lib.load().phyai_fp8_gemm_addcmul(
+            x2.data_ptr(), xs.data_ptr(), scalar, weight.data_ptr(), weight_scale.data_ptr(), bias_ptr,
+            r2.data_ptr(), r2.stride(0) if M > 1 else N, g2.data_ptr(), g2.stride(0) if g2.shape[0] > 1 else N,
+            g2.shape[0], out.data_ptr(), n_out, M, N, K, ws.data_ptr(), ws.numel(), _stream_ptr())
+    else:
+        rc = _lib.load().phyai_fp8_gemm(x2.data_ptr(), xs.data_ptr(), scalar, weight.data_ptr(),
+                                         weight_scale.data_ptr(), bias_ptr, out.data_ptr(), n_out, M, N, K, epi,
+                                         ws.data_ptr(), ws.numel(), _stream_ptr())
     _lib.check(rc, op)
     return out
 
 
 def fp8_linear(x: torch.Tensor, weight: torch.Tensor, weight_scale: torch.Tensor,
-               bias: torch.Tensor | None = None, *, epilogue=None, out: torch.Tensor | None = None) -> torch.Tensor:
+               bias: torch.Tensor | None = None, *, epilogue=None, out: torch.Tensor | None = None,
+               residual: torch.Tensor | None = None, gate: torch.Tensor | None = None) -> torch.Tensor:
     """The whole W8A8 linear on bf16 ``x[..., K]``: per-token quantization, fp8 MFMA
     GEMM, per-channel dequantization, bias and optional activation, bf16 out.
 
@@ -373,13 +410,20 @@ def fp8_linear(x: torch.Tensor, weight: torch.Tensor, weight_scale: torch.Tensor
         raise _err(op, f"gated epilogue needs N % 32 == 0, got {N}")
     bias_ptr = _check_bias(op, bias, N)
     n_out = N // 2 if epi in _GATED else N
+    r2, g2 = _check_addcmul(op, residual, gate, tuple(x.shape[:-1]), M, N, epi, x.device)
     out = _out_for(op, tuple(x.shape[:-1]), n_out, out, x.device)
     if M == 0:
         return out
     ws = _workspace_for(M, N, K, epi, x.device)
-    rc = _lib.load().phyai_fp8_linear(x2.data_ptr(), x2.stride(0) if M > 1 else K, weight.data_ptr(),
-                                       weight_scale.data_ptr(), bias_ptr, out.data_ptr(), n_out, M, N, K, epi,
-                                       ws.data_ptr(), ws.numel(), _stream_ptr())
+    if r2 is not None:
+        rc = _lib.load().phyai_fp8_linear_addcmul(
+            x2.data_ptr(), x2.stride(0) if M > 1 else K, weight.data_ptr(), weight_scale.data_ptr(), bias_ptr,
+            r2.data_ptr(), r2.stride(0) if M > 1 else N, g2.data_ptr(), g2.stride(0) if g2.shape[0] > 1 else N,
+            g2.shape[0], out.data_ptr(), n_out, M, N, K, ws.data_ptr(), ws.numel(), _stream_ptr())
+    else:
+        rc = _lib.load().phyai_fp8_linear(x2.data_ptr(), x2.stride(0) if M > 1 else K, weight.data_ptr(),
+                                           weight_scale.data_ptr(), bias_ptr, out.data_ptr(), n_out, M, N, K, epi,
+                                           ws.data_ptr(), ws.numel(), _stream_ptr())
     _lib.check(rc, op)
     return out
 

@@ -155,6 +155,10 @@ def _norm_modules_body(dev, GemmaRMSNorm, AdaRMSNorm, ColumnParallelLinear, Dens
     n2, gate2 = ada(x, modulation=table)
     assert torch.equal(gate, gate2) and gate.shape == (1, D)
     assert torch.equal(layer(v2)[0], layer(n2)[0])
+    # gated residual fused into the same layer's epilogue, gate of one modulation row
+    res = (torch.randn(M, N) * 0.5).to(torch.bfloat16).to(dev)
+    g_row = (torch.randn(1, N) * 0.3).to(torch.bfloat16).to(dev)
+    assert torch.equal(layer.forward_addcmul(v2, res, g_row), torch.addcmul(res, layer(v2)[0], g_row))
 
     mlp = DenseMLP(D, 4096, activation="gelu_tanh", gated=True, bias=False, params_dtype=torch.bfloat16,
                    spec_in=Fp8Spec(), spec_out=Fp8Spec())

@@ -447,3 +447,47 @@ def test_quant_rowwise_exhaustive_all_values_all_scales(dev):
             raise AssertionError(
                 f"amax bits {int(a[r]):#06x}, x bits {int(x[r, c].view(torch.uint16)):#06x}: "
                 f"got {int(q.view(torch.uint8)[r, c]):#04x} want {int(wq.view(torch.uint8)[r, c]):#04x}")
+
+
+@pytest.mark.parametrize("M,N,K,force,gate_rows", [
+    (50, 1024, 2048, "", 1), (50, 1024, 4096, "", 50), (200, 1024, 4096, "", 4), (70, 192, 272, "", 70),
+    (816, 2048, 2048, "128", 816), (816, 2048, 2048, "256", 1), (300, 384, 4096, "128", 3), (9, 64, 128, "", 9)])
+def test_linear_gated_residual(dev, monkeypatch, M, N, K, force, gate_rows):
+    """out = addcmul(residual, linear(x), gate) inside the GEMM epilogue, every kernel family; the result
+    must equal torch.addcmul applied to the device's own plain linear output bit for bit."""
+    ops = _ops()
+    if force:
+        monkeypatch.setenv("PHYAI_FP8_BIG", force)
+    x, wq, ws, b = _problem(M, N, K, seed=M + N)
+    res = seeded((M, N), seed=5)
+    gate = seeded((gate_rows, N), seed=6, scale=0.5)
+    xd, wd, sd, bd = x.to(dev), wq.to(dev), ws.to(dev), b.to(dev)
+    y = ops.fp8_linear(xd, wd, sd, bd)
+    got = ops.fp8_linear(xd, wd, sd, bd, residual=res.to(dev), gate=gate.to(dev))
+    want = ref.addcmul(res, y.cpu(), gate)
+    assert torch.equal(got.cpu(), want)
+    # and through the quantized-input entry point, writing over the residual
+    xq, xs = ops.fp8_quant_rowwise(xd)
+    buf = res.to(dev).clone()
+    ops.fp8_gemm(xq, xs, wd, sd, bd, residual=buf, gate=gate.to(dev), out=buf)
+    assert torch.equal(buf.cpu(), want)
+    # against the oracle's own linear, to the stated tolerance
+    xq_c, xs_c = ref.quant_rowwise(x)
+    y_ref = ref.gemm_f32(xq_c, xs_c, wq, ws, b)
+    g_full = gate.repeat_interleave(M // gate_rows, dim=0).float()
+    assert_close_to_ref(got, res.float() + y_ref.to(torch.bfloat16).float() * g_full, "gated residual")
+
+
+def test_gated_residual_argument_errors(dev):
+    ops = _ops()
+    x, wq, ws, b = _problem(16, 64, 128, seed=1)
+    xd, wd, sd = x.to(dev), wq.to(dev), ws.to(dev)
+    r = torch.zeros(16, 64, dtype=torch.bfloat16, device=dev)
+    with pytest.raises(RuntimeError, match="go together"):
+        ops.fp8_linear(xd, wd, sd, None, residual=r)
+    with pytest.raises(RuntimeError, match="excludes an activation"):
+        ops.fp8_linear(xd, wd, sd, None, epilogue="gelu", residual=r, gate=r)
+    with pytest.raises(RuntimeError, match="multiple of gate rows"):
+        ops.fp8_linear(xd, wd, sd, None, residual=r, gate=r[:5])
+    with pytest.raises(RuntimeError, match="residual must have shape"):
+        ops.fp8_linear(xd, wd, sd, None, residual=r[:8], gate=r[:8])

@@ -331,3 +331,14 @@ def test_adarmsnorm_oracle_properties():
     mod_tok = mod.repeat_interleave(13, dim=0).reshape(4, 13, 3 * D)
     o_tok, g_tok = ref.adarmsnorm(x, mod_tok, 1e-6)
     assert torch.equal(o_tok, out) and g_tok.shape == (4, 13, D)
+
+
+def test_addcmul_oracle_is_torch_addcmul_and_single_rounding():
+    r, y, g = seeded((33, 64), 1), seeded((33, 64), 2), seeded((33, 64), 3, 0.3)
+    got = ref.addcmul(r, y, g)
+    assert torch.equal(got, torch.addcmul(r, y, g))                       # the library routine the reference calls
+    want = (r.double() + y.double() * g.double()).to(torch.bfloat16)      # exact arithmetic, one rounding
+    assert torch.equal(got, want)
+    gb = seeded((3, 64), 4, 0.3)                                          # one gate row per 11 token rows
+    assert torch.equal(ref.addcmul(r, y, gb), torch.addcmul(r.reshape(3, 11, 64), y.reshape(3, 11, 64),
+                                                            gb.reshape(3, 1, 64)).reshape(33, 64))
