@@ -98,6 +98,57 @@ def run_layers(layers, shapes):
             ops.fp8_linear(t["x"], t["w"], t["ws"], None, epilogue=t["epi"], out=t["out"])
 
 
+def decoder_layer_times(dev, layers, M, denoise_steps, steps, warmup):
+    """The expert layer's linear path WITH its neighbours (adaptive norms before qkv / gate_up, gated
+    residuals after o / down; reference models/pi05/modeling_pi05.py:812-835), two ways on the same
+    tensors: `separate` = norm, quantizer, GEMM and addcmul as their own launches (12 per layer, the
+    reference's structure), `fused` = norm+quantizer in one kernel, addcmul in the GEMM epilogue
+    (6 per layer).  Attention and RoPE are not part of either."""
+    from phyai_amd import ops
+    from phyai_amd.runtime import HipGraph
+
+    D = 1024
+    g = torch.Generator().manual_seed(777)
+    h = torch.randn(M, D, generator=g).to(torch.bfloat16).to(dev)
+    mods = [(torch.randn(1, 3 * D, generator=g) * 0.1).to(torch.bfloat16).to(dev) for _ in range(2)]
+    attn = torch.randn(M, 2048, generator=g).to(torch.bfloat16).to(dev)
+    h1 = torch.empty_like(h)
+    h2 = torch.empty_like(h)
+
+    def separate():
+        for _ in range(denoise_steps):
+            for layer in layers:
+                q, o, gu, dn = layer["qkv"], layer["o"], layer["gate_up"], layer["down"]
+                n, gate = ops.adarmsnorm(h, mods[0], 1e-6)
+                ops.fp8_linear(n, q["w"], q["ws"], None, out=q["out"])
+                y = ops.fp8_linear(attn, o["w"], o["ws"], None, out=o["out"])
+                torch.addcmul(h, y, gate, out=h1)
+                m, gate2 = ops.adarmsnorm(h1, mods[1], 1e-6)
+                a = ops.fp8_linear(m, gu["w"], gu["ws"], None, epilogue="geglu_tanh", out=gu["out"])
+                y2 = ops.fp8_linear(a, dn["w"], dn["ws"], None, out=dn["out"])
+                torch.addcmul(h1, y2, gate2, out=h2)
+
+    def fused():
+        for _ in range(denoise_steps):
+            for layer in layers:
+                q, o, gu, dn = layer["qkv"], layer["o"], layer["gate_up"], layer["down"]
+                nq, ns, gate = ops.adarmsnorm_fp8(h, mods[0], 1e-6)
+                ops.fp8_gemm(nq, ns, q["w"], q["ws"], None, out=q["out"])
+                ops.fp8_linear(attn, o["w"], o["ws"], None, residual=h, gate=gate, out=h1)
+                mq, ms, gate2 = ops.adarmsnorm_fp8(h1, mods[1], 1e-6)
+                a = ops.fp8_gemm(mq, ms, gu["w"], gu["ws"], None, epilogue="geglu_tanh", out=gu["out"])
+                ops.fp8_linear(a, dn["w"], dn["ws"], None, residual=h1, gate=gate2, out=h2)
+
+    res = {}
+    for name, fn in (("separate", separate), ("fused", fused)):
+        gr = HipGraph()
+        gr.capture(fn, {})
+        ts, _ = time_replays(gr, steps, warmup)
+        res[name] = round(statistics.median(ts) * 1e3 / denoise_steps, 2)
+        del gr
+    return res
+
+
 def time_replays(graph, n, warmup):
     """HIP events around each replay, on the stream the replays are launched on."""
     for _ in range(warmup):
@@ -312,6 +363,10 @@ def main() -> int:
                                  "TFLOP/s": round(flops / (p_layer_us * 1e-6) / 1e12, 1),
                                  "frac_fp8_peak": round(flops / (p_layer_us * 1e-6) / 1e12 / FP8_PEAK_TFLOPS, 4)}
         del pl, pg
+    dl = decoder_layer_times(dev, layers, M, denoise_steps, max(20, args.steps // 4), 5)
+    extra["expert_step_with_norms_and_residuals_us"] = {
+        **dl, "note": "per denoise step, 18 layers: adaptive norm -> qkv, o -> gated residual, adaptive norm -> "
+                      "gate_up+GeGLU, down -> gated residual; separate = 12 launches per layer, fused = 6"}
     if args.sweep:
         extra["batched_sweep"] = sweep(dev)
 
