@@ -98,6 +98,45 @@ def run_layers(layers, shapes):
             ops.fp8_linear(t["x"], t["w"], t["ws"], None, epilogue=t["epi"], out=t["out"])
 
 
+def torch_reference_times(dev, layers, shapes, denoise_steps, steps, warmup):
+    """The reference's own GPU path for the same linears, as far as this image can run it: the
+    quantizer's torch expressions (layers/quant/fp8.py:152-154) and torch._scaled_mm
+    (layers/linear/backends/torch.py:166-175; hipBLASLt underneath on ROCm), the gated activation as
+    torch ops because flashinfer is not installed.  Same tensors, same graph shape.  Returns us per
+    denoise step, or a reason string when torch._scaled_mm does not run here."""
+    import torch.nn.functional as F
+
+    from phyai_amd.runtime import HipGraph
+
+    def linear(t):
+        x = t["x"]
+        a = x.abs().amax(dim=-1, keepdim=True).clamp_min(1e-12)
+        s = (a / 448.0).to(torch.float32)
+        xq = (x / s).to(torch.float8_e4m3fn)
+        y = torch._scaled_mm(xq, t["w"].t(), scale_a=s, scale_b=t["ws"].reshape(1, -1), out_dtype=torch.bfloat16)
+        if t["epi"]:
+            half = y.shape[-1] // 2
+            y = F.gelu(y[:, :half], approximate="tanh") * y[:, half:]
+        return y
+
+    try:
+        linear(layers[0][shapes[0][0]])
+        torch.cuda.synchronize()
+    except Exception as e:  # noqa: BLE001 - any failure means "not runnable on this image"
+        return f"torch._scaled_mm unavailable: {str(e)[:120]}"
+
+    def chunk():
+        for _ in range(denoise_steps):
+            for layer in layers:
+                for name, _, _, _ in shapes:
+                    linear(layer[name])
+
+    g = HipGraph()
+    g.capture(chunk, {})
+    ts, _ = time_replays(g, steps, warmup)
+    return round(statistics.median(ts) * 1e3 / denoise_steps, 2)
+
+
 def decoder_layer_times(dev, layers, M, denoise_steps, steps, warmup):
     """The expert layer's linear path WITH its neighbours (adaptive norms before qkv / gate_up, gated
     residuals after o / down; reference models/pi05/modeling_pi05.py:812-835), two ways on the same
@@ -359,7 +398,9 @@ def main() -> int:
         pts, _ = time_replays(pg, 30, 3)
         p_layer_us = statistics.median(pts) * 1e3 / len(pl)
         flops = sum(2 * 816 * N * K for _, N, K, _ in PREFILL_SET)
-        extra["prefill_M816"] = {"us_per_layer": round(p_layer_us, 2),
+        tref = torch_reference_times(dev, pl, PREFILL_SET, 1, 10, 3)
+        extra["prefill_M816"] = {"torch_reference_path_us_per_layer": (round(tref / len(pl), 2) if not isinstance(tref, str) else tref),
+                                 "us_per_layer": round(p_layer_us, 2),
                                  "TFLOP/s": round(flops / (p_layer_us * 1e-6) / 1e12, 1),
                                  "frac_fp8_peak": round(flops / (p_layer_us * 1e-6) / 1e12 / FP8_PEAK_TFLOPS, 4)}
         del pl, pg
@@ -367,6 +408,10 @@ def main() -> int:
     extra["expert_step_with_norms_and_residuals_us"] = {
         **dl, "note": "per denoise step, 18 layers: adaptive norm -> qkv, o -> gated residual, adaptive norm -> "
                       "gate_up+GeGLU, down -> gated residual; separate = 12 launches per layer, fused = 6"}
+    extra["torch_reference_path_us"] = {
+        "expert_step": torch_reference_times(dev, layers, EXPERT_SET, denoise_steps, max(10, args.steps // 10), 3),
+        "note": "same linears through the reference's own arithmetic on this GPU: torch-op quantizer + "
+                "torch._scaled_mm (+ torch GELU*up); compare with `value`"}
     if args.sweep:
         extra["batched_sweep"] = sweep(dev)
 

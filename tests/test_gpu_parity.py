@@ -491,3 +491,49 @@ def test_gated_residual_argument_errors(dev):
         ops.fp8_linear(xd, wd, sd, None, residual=r, gate=r[:5])
     with pytest.raises(RuntimeError, match="residual must have shape"):
         ops.fp8_linear(xd, wd, sd, None, residual=r[:8], gate=r[:8])
+
+
+# ---- against the reference's own GPU arithmetic (torch ops + torch._scaled_mm on this device) ----
+
+def _torch_quantize_activation(x: torch.Tensor):
+    """The three lines of Fp8Spec.quantize_activation (reference layers/quant/fp8.py:152-154), on the GPU."""
+    a = x.abs().amax(dim=-1, keepdim=True).clamp_min(1e-12)
+    s = (a / 448.0).to(torch.float32)
+    return (x / s).to(torch.float8_e4m3fn), s
+
+
+@pytest.mark.parametrize("shape", [(50, 1024), (816, 2048), (7, 4096), (300, 16384)])
+def test_quantizer_bit_exact_with_reference_expressions_on_device(dev, shape):
+    ops = _ops()
+    x = seeded(shape, seed=shape[0], scale=1.5).to(dev)
+    x[0, :16] = 0.0
+    x[1 % shape[0], 3] = 300.0                                          # an outlier channel
+    q_ref, s_ref = _torch_quantize_activation(x)
+    q, s = ops.fp8_quant_rowwise(x)
+    assert torch.equal(s, s_ref)
+    assert torch.equal(q.view(torch.uint8), q_ref.view(torch.uint8))
+
+
+@pytest.mark.parametrize("M,N,K,force", [(50, 2560, 1024, ""), (50, 1024, 4096, ""), (200, 1024, 2048, ""),
+                                         (816, 2560, 2048, ""), (816, 2048, 16384, ""), (816, 4096, 2048, "256"),
+                                         (70, 192, 272, "")])
+def test_gemm_against_torch_scaled_mm(dev, monkeypatch, M, N, K, force):
+    """torch._scaled_mm with row-wise scales is the GEMM the reference calls
+    (layers/linear/backends/torch.py:166-175).  Same codes, same scales, same bias on this GPU: the
+    outputs must agree to the stated tolerance, and nearly all of them bit for bit."""
+    ops = _ops()
+    if force:
+        monkeypatch.setenv("PHYAI_FP8_BIG", force)
+    x, wq, ws, b = _problem(M, N, K, seed=M * 7 + N)
+    xd, wd, sd, bd = x.to(dev), wq.to(dev), ws.to(dev), b.to(dev)
+    xq, xs = ops.fp8_quant_rowwise(xd)
+    try:
+        want = torch._scaled_mm(xq, wd.t(), scale_a=xs, scale_b=sd.reshape(1, -1), bias=bd, out_dtype=torch.bfloat16)
+        torch.cuda.synchronize()
+    except Exception as e:  # noqa: BLE001
+        pytest.skip(f"torch._scaled_mm does not run on this image: {str(e)[:100]}")
+    got = ops.fp8_gemm(xq, xs, wd, sd, bd)
+    assert_close_to_ref(got, want.float().cpu(), f"vs torch._scaled_mm {M}x{N}x{K}")
+    step = want.float().abs().clamp_min(2.0 ** -126) * 2.0 ** -7
+    assert bool(((got.float() - want.float()).abs() <= step).all()), "more than one bf16 step from torch._scaled_mm"
+    assert float((got == want).float().mean()) > 0.97
