@@ -456,7 +456,7 @@ BigPlan big_plan(int M, int N, int K, int epilogue) {
     if (forced == 256 || forced == 128) pl.tile = forced;
     else if (M < 128) return pl;
     else if (big_tiles(M, N, epilogue, 256, 256) >= 200) pl.tile = 256;
-    else if (big_tiles(M, N, epilogue, 128, 128) >= 48) pl.tile = 128;
+    else if (big_tiles(M, N, epilogue, 128, 128) >= 32) pl.tile = 128;   // fewer: the weight-streaming kernel wins
     else return pl;
     const int tiles = big_tiles(M, N, epilogue, pl.tile, pl.tile);
     if (pl.tile == 128) {
