@@ -36,6 +36,17 @@ def _M_of(x) -> int:
     return m
 
 
+def _max_of_legs():
+    seen: list = []
+
+    def load(param: nn.Parameter, loaded: torch.Tensor, _shard_id=None) -> None:
+        v = loaded.reshape(-1)[0].to(param.dtype)
+        param.data.fill_(max([v.item()] + seen))
+        seen.append(v.item())
+
+    return load
+
+
 def _default_device() -> torch.device:
     return torch.device("cuda", torch.cuda.current_device()) if torch.cuda.is_available() else torch.device("cpu")
 
@@ -88,15 +99,36 @@ class LinearBase(nn.Module):
         """
         if not self.prefix:
             return
-        legs = list(legs) if legs is not None else [(self.prefix, None)]
+        from phyai_amd import weights as W
+
+        fused = legs is not None
+        legs = list(legs) if fused else [(self.prefix, None)]
+        # row range of every leg in the fused parameter
+        offsets, off = {}, 0
+        for (_, sid), width in zip(legs, getattr(self, "output_partition_sizes", [self.output_size_per_partition])):
+            offsets[sid] = (off, width)
+            off += width
+        rows = W.fused_rows(offsets) if fused else W.replicated()
         self.weight.hf_keys = [(f"{base}.weight", sid) for base, sid in legs]
+        self.weight.weight_loader = rows
         if self.bias is not None:
             self.bias.hf_keys = [(f"{base}.bias", sid) for base, sid in legs]
+            self.bias.weight_loader = rows
         for name in ("weight_scale", "input_scale", "weight_global_scale"):
             p = getattr(self, name, None)
             if isinstance(p, nn.Parameter):
                 p.hf_keys = [(f"{base}.{name}", sid) for base, sid in legs]
                 p.optional = True
+                if not fused:
+                    p.weight_loader = W.replicated()
+                elif p.shape[0] == self.output_size_per_partition:
+                    p.weight_loader = rows                                    # one scale per output row
+                elif p.shape[0] == len(legs):
+                    p.weight_loader = W.leg_slots([sid for _, sid in legs])   # one scale per leg
+                else:
+                    # one value for the whole fused layer (a static activation scale): every leg
+                    # of a checkpoint carries its own; the largest is the safe common choice
+                    p.weight_loader = _max_of_legs()
 
     def post_load(self) -> None:
         hook = getattr(self.spec, "process_after_loading", None)

@@ -22,19 +22,41 @@ from phyai_amd.quant import Bf16Spec, Fp8Spec, Granularity
 SpecFactory = Callable[[], object]
 
 
+def _lower(target) -> object | None:
+    """A rule's right-hand side -> spec: ``None`` (skip), a spec factory, or a semantic
+    ``QuantScheme`` (lowered as the reference's ``materialize`` does)."""
+    if target is None:
+        return None
+    if callable(target):
+        return target()
+    from phyai_amd.quant.scheme import QuantScheme, materialize
+
+    if isinstance(target, QuantScheme):
+        return materialize(target)
+    return target
+
+
 @dataclasses.dataclass
 class QuantPlan:
-    rules: list[tuple[str, SpecFactory]] = dataclasses.field(default_factory=list)
-    default: SpecFactory | None = None
+    """Ordered rule table; the first matching rule decides (reference ``plan.py:43-70``).  A rule is
+    a ``Rule(Matcher, QuantScheme | None)`` - what the config importers produce - or, as a
+    shorthand, ``(glob over the layer prefix, spec factory)``; ``ignore`` globs are checked first."""
+
+    rules: list = dataclasses.field(default_factory=list)
+    default: object | None = None
     ignore: list[str] = dataclasses.field(default_factory=list)
 
     def resolve(self, prefix: str, layer_cls: type | None = None) -> object | None:
         if any(fnmatch.fnmatchcase(prefix, pat) for pat in self.ignore):
             return None
-        for pat, factory in self.rules:
-            if fnmatch.fnmatchcase(prefix, pat):
-                return factory()
-        return self.default() if self.default is not None else None
+        for rule in self.rules:
+            if isinstance(rule, tuple):
+                pat, target = rule
+                if fnmatch.fnmatchcase(prefix, pat):
+                    return _lower(target)
+            elif rule.matcher.matches(prefix, layer_cls):
+                return _lower(rule.scheme)
+        return _lower(self.default)
 
     @staticmethod
     def fp8_per_channel(ignore: list[str] | None = None) -> "QuantPlan":
