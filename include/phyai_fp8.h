@@ -147,8 +147,9 @@ int phyai_fp8_linear_addcmul(const void *x, int64_t ldx, const void *w, const fl
  * by Fp8Spec.quantize_activation (layers/quant/fp8.py:150-155) on that bf16
  * output.  x: [M, D] bf16, row stride ldx; weight: [D] bf16.  out ([M, D] bf16,
  * row stride ldo) may be NULL when only the codes are wanted; xq / x_scale may
- * both be NULL when only the normalised bf16 tensor is wanted.  D % 8 == 0,
- * D <= 8192 (the reference's single-block limit).
+ * both be NULL when only the normalised bf16 tensor is wanted.  D % 8 == 0; rows up
+ * to 8192 elements stay in registers, longer ones are re-read per pass (the
+ * reference's two-pass kernels, rms_norm.py:125-167).
  */
 int phyai_fp8_rmsnorm_quant(const void *x, int64_t ldx, const void *weight, int gemma,
                             int64_t M, int64_t D, float eps, void *out, int64_t ldo,

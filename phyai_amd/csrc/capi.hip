@@ -241,7 +241,7 @@ int check_norm_args(const char* fn, const void* x, int64_t ldx, int64_t M, int64
     if (!out && !xq) return fail(PHYAI_FP8_EINVAL, "%s: neither out nor xq given", fn);
     if ((xq == nullptr) != (x_scale == nullptr)) return fail(PHYAI_FP8_EINVAL, "%s: xq and x_scale go together", fn);
     if (D % 8 != 0) return fail(PHYAI_FP8_EUNSUPPORTED, "%s: D=%lld must be a multiple of 8", fn, (long long)D);
-    if (D > 8192) return fail(PHYAI_FP8_EUNSUPPORTED, "%s: D=%lld exceeds 8192", fn, (long long)D);
+    if (D > (1 << 20)) return fail(PHYAI_FP8_EUNSUPPORTED, "%s: D=%lld exceeds 2^20", fn, (long long)D);
     if (ldx < D || ldx % 8 != 0 || (out && (ldo < D || ldo % 8 != 0)))
         return fail(PHYAI_FP8_EINVAL, "%s: row strides must be >= D and multiples of 8", fn);
     if (!aligned(x, 16) || (out && !aligned(out, 16)) || (xq && !aligned(xq, 8)))

@@ -319,6 +319,67 @@ __global__ __launch_bounds__(THREADS) void norm_quant_kernel(const NormQuantArgs
     }
 }
 
+// Rows too long for registers (D > 8192, the reference's two-pass kernels): the row is read again
+// for every pass - sum of squares, then the bf16 result and its absmax, then the codes.
+template <bool ADAPTIVE>
+__global__ __launch_bounds__(256) void norm_quant_loop_kernel(const NormQuantArgs p) {
+    __shared__ float ssum[256 / kWave];
+    __shared__ uint32_t smax[256 / kWave];
+    const int64_t row = blockIdx.x;
+    const uint16_t* xr = p.x + row * p.ldx;
+    float ss = 0.f;
+    for (int k = threadIdx.x * 8; k < p.D; k += 256 * 8) {
+        float f[8];
+        unpack8(*reinterpret_cast<const uint4*>(xr + k), f);
+#pragma unroll
+        for (int e = 0; e < 8; ++e) ss += f[e] * f[e];
+    }
+    ss = block_sum_f32<256>(ss, ssum);
+    const float rstd = 1.0f / sqrtf(ss / (float)p.D + p.eps);
+    const int64_t mrow = ADAPTIVE ? row / p.group : 0;
+    const uint16_t* mr = ADAPTIVE ? p.mod + mrow * p.ld_mod : nullptr;
+    auto result8 = [&](int k) -> uint4 {
+        float f[8], o[8];
+        unpack8(*reinterpret_cast<const uint4*>(xr + k), f);
+        if constexpr (ADAPTIVE) {
+            float sc[8], sh[8];
+            unpack8(*reinterpret_cast<const uint4*>(mr + k), sc);
+            unpack8(*reinterpret_cast<const uint4*>(mr + p.D + k), sh);
+#pragma unroll
+            for (int e = 0; e < 8; ++e) o[e] = (f[e] * rstd) * (1.0f + sc[e]) + sh[e];
+        } else {
+            float w[8];
+            unpack8(*reinterpret_cast<const uint4*>(p.weight + k), w);
+#pragma unroll
+            for (int e = 0; e < 8; ++e) o[e] = (f[e] * rstd) * (p.gemma ? w[e] + 1.0f : w[e]);
+        }
+        uint4 b;
+        b.x = f32_to_bf16_bits(o[0]) | (f32_to_bf16_bits(o[1]) << 16);
+        b.y = f32_to_bf16_bits(o[2]) | (f32_to_bf16_bits(o[3]) << 16);
+        b.z = f32_to_bf16_bits(o[4]) | (f32_to_bf16_bits(o[5]) << 16);
+        b.w = f32_to_bf16_bits(o[6]) | (f32_to_bf16_bits(o[7]) << 16);
+        return b;
+    };
+    uint32_t m = 0;
+    for (int k = threadIdx.x * 8; k < p.D; k += 256 * 8) {
+        const uint4 b = result8(k);
+        if (p.out != nullptr) *reinterpret_cast<uint4*>(p.out + row * p.ldo + k) = b;
+        if constexpr (ADAPTIVE) {
+            if (p.gate != nullptr && row % p.group == 0)
+                *reinterpret_cast<uint4*>(p.gate + mrow * p.ld_gate + k) = *reinterpret_cast<const uint4*>(mr + 2 * p.D + k);
+        }
+        m = absmax8(b, m);
+    }
+    if (p.xq == nullptr) return;
+    m = block_max_u32<256>(m, smax);
+    const float s = scale_from_amax_bits<QUANT_ACT_DYNAMIC>(m);
+    if (threadIdx.x == 0) p.scale[row] = s;
+    const RowDivisor d = make_divisor(s);
+    uint8_t* qr = p.xq + row * (int64_t)p.D;
+    for (int k = threadIdx.x * 8; k < p.D; k += 256 * 8)
+        *reinterpret_cast<uint2*>(qr + k) = encode8<QUANT_ACT_DYNAMIC>(result8(k), d);
+}
+
 template <bool ADAPTIVE>
 static int launch_norm_quant_t(const NormQuantArgs& a, int64_t M, hipStream_t st) {
     const dim3 grid((unsigned)M);
@@ -328,7 +389,7 @@ static int launch_norm_quant_t(const NormQuantArgs& a, int64_t M, hipStream_t st
     else if (a.D <= 2048) PHYAI_NQ(256, 1);
     else if (a.D <= 4096) PHYAI_NQ(256, 2);
     else if (a.D <= 8192) PHYAI_NQ(256, 4);
-    else return -2;
+    else hipLaunchKernelGGL((norm_quant_loop_kernel<ADAPTIVE>), grid, dim3(256), 0, st, a);
 #undef PHYAI_NQ
     return 0;
 }

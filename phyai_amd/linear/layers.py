@@ -36,13 +36,14 @@ def _M_of(x) -> int:
     return m
 
 
-def _max_of_legs():
-    seen: list = []
+def _max_of_legs(layer: nn.Module):
+    """Loader of a scalar that every leg of a fused layer brings its own copy of: keep the largest
+    of one load (``post_load`` forgets what was seen, so a reload starts afresh)."""
 
     def load(param: nn.Parameter, loaded: torch.Tensor, _shard_id=None) -> None:
-        v = loaded.reshape(-1)[0].to(param.dtype)
-        param.data.fill_(max([v.item()] + seen))
-        seen.append(v.item())
+        v = float(loaded.reshape(-1)[0])
+        layer._fused_scalar_seen.append(v)
+        param.data.fill_(max(layer._fused_scalar_seen))
 
     return load
 
@@ -128,9 +129,12 @@ class LinearBase(nn.Module):
                 else:
                     # one value for the whole fused layer (a static activation scale): every leg
                     # of a checkpoint carries its own; the largest is the safe common choice
-                    p.weight_loader = _max_of_legs()
+                    self._fused_scalar_seen = []
+                    p.weight_loader = _max_of_legs(self)
 
     def post_load(self) -> None:
+        if hasattr(self, "_fused_scalar_seen"):
+            self._fused_scalar_seen = []
         hook = getattr(self.spec, "process_after_loading", None)
         if callable(hook):
             hook(self)

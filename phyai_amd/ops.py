@@ -150,8 +150,8 @@ def _rmsnorm(op: str, x, weight, eps, out, gemma: bool, quantize: bool, want_out
     if not (isinstance(weight, torch.Tensor) and weight.is_cuda and weight.dtype == torch.bfloat16
             and weight.shape == (D,) and weight.is_contiguous()):
         raise _err(op, f"weight must be a contiguous bfloat16 GPU tensor of shape ({D},)")
-    if D % 8 != 0 or D > 8192:
-        raise _err(op, f"last dim {D} must be a multiple of 8 and at most 8192")
+    if D % 8 != 0:
+        raise _err(op, f"last dim {D} must be a multiple of 8")
     out, xq, xs = _norm_outputs(op, x, out, quantize, want_out)
     if M == 0:
         return out, xq, xs
@@ -196,8 +196,8 @@ def _adarmsnorm(op: str, x, modulation, eps, out, gate_out, quantize: bool, want
     M, D = x2.shape
     mod2 = _as_rows(op, modulation, "modulation", torch.bfloat16)
     n_mod = mod2.shape[0]
-    if D % 8 != 0 or D > 8192:
-        raise _err(op, f"last dim {D} must be a multiple of 8 and at most 8192")
+    if D % 8 != 0:
+        raise _err(op, f"last dim {D} must be a multiple of 8")
     out, xq, xs = _norm_outputs(op, x, out, quantize, want_out)
     gate_shape = (*modulation.shape[:-1], D)
     if gate_out is None:
