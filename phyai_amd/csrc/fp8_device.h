@@ -54,6 +54,21 @@ __device__ __forceinline__ uint32_t wave_max_u32(uint32_t v) {
     return v;
 }
 
+// One 16-byte chunk per lane from global memory straight into LDS: lane i's chunk lands at
+// lds_wave_base + 16*i.  Issued as inline assembly so that the compiler does not order its own
+// LDS reads behind copies that are still in flight; the waits are placed by hand below.
+__device__ __forceinline__ void copy16_to_lds(const uint8_t* base, uint32_t lane_offset, uint32_t lds_wave_base) {
+    asm volatile("s_mov_b32 m0, %2\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, %1"
+                 :: "v"(lane_offset), "s"(base), "s"(lds_wave_base) : "memory", "m0");
+}
+
+// s_waitcnt vmcnt(N) with a compile-time N: at most N of this wavefront's copies still in flight.
+template <int N>
+__device__ __forceinline__ void wait_copies() {
+    static_assert(N >= 0 && N < 64, "vmcnt is a 6-bit counter");
+    asm volatile("s_waitcnt vmcnt(%0)" ::"n"(N) : "memory");
+}
+
 // ---- epilogue activations (fp32 math) ------------------------------------
 // gelu_tanh(v) = 0.5 v (1 + tanh u), u = k0 (v + k1 v^3).  With tanh u = 1 - 2 / (exp(2u) + 1) this
 // is v - v / (exp(2u) + 1): exact limits (v and 0) when the exponential overflows or underflows,

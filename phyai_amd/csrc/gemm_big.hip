@@ -81,21 +81,6 @@ __device__ __forceinline__ BigTile big_tile_of(int id, int m_tiles, int n_tiles)
     return t;
 }
 
-// One 16-byte chunk per lane from global memory straight into LDS: lane i's chunk lands at
-// lds_wave_base + 16*i.  Issued as inline assembly so that the compiler does not order its own
-// LDS reads behind copies that are still in flight; the waits are placed by hand below.
-__device__ __forceinline__ void copy16_to_lds(const uint8_t* base, uint32_t lane_offset, uint32_t lds_wave_base) {
-    asm volatile("s_mov_b32 m0, %2\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, %1"
-                 :: "v"(lane_offset), "s"(base), "s"(lds_wave_base) : "memory", "m0");
-}
-
-// s_waitcnt vmcnt(N) with a compile-time N: at most N of this wavefront's copies still in flight.
-template <int N>
-__device__ __forceinline__ void wait_copies() {
-    static_assert(N >= 0 && N < 64, "vmcnt is a 6-bit counter");
-    asm volatile("s_waitcnt vmcnt(%0)" ::"n"(N) : "memory");
-}
-
 // Swizzle of the eight 16-byte chunks of a 128-byte row.  LDS has 64 banks of 4 bytes, so one
 // pass over the banks spans two rows and a 128-bit read is served 16 lanes at a time: the eight
 // rows of equal parity among 16 consecutive ones must land in different chunk columns.

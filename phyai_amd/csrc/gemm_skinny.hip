@@ -65,12 +65,29 @@ __device__ __forceinline__ v8i join(v4i lo, v4i hi) {
 
 // MB: 16-row token blocks per workgroup (grid.y workgroups cover M); NT: 16-row weight
 // tiles per workgroup; KPW: K steps per wavefront per round.
-template <int MB, int NT, int KPW, int EPI>
+//
+// STAGED: the operands reach the MFMA layout through the wavefront's own slice of LDS instead of
+// directly.  A direct load gives each operand row 64 contiguous bytes per instruction (4 lanes
+// per row); the copy into LDS is free to give it the whole 128-byte step (8 lanes per row), i.e.
+// one L2 line per request.  A CU pulls about twice the bytes per second that way, and the load
+// phase of this kernel is bound by exactly that rate (every workgroup needs its weight tiles
+// AND all of the activation codes of its token rows).  Nobody but the wavefront itself reads
+// what it staged, so there is still no barrier before the math: copies, s_waitcnt, ds_read.
+template <int MB, int NT, int KPW, int EPI, bool STAGED>
 __global__ __launch_bounds__(SK_THREADS) void gemm_fp8_skinny_kernel(const SkinnyArgs p) {
     constexpr bool GATED = epi_is_gated(EPI);
     constexpr int COLS_PER_TILE = GATED ? 8 : 16;  // output columns per 16-row weight tile
+    constexpr int BLOCKS = NT + MB;                // 16-row operand blocks (2 KB each) per K step
+    constexpr int RED_PER_WAVE = NT * MB * kWave * (int)sizeof(v4f);
+    constexpr int STAGE_PER_WAVE = KPW * BLOCKS * 2048;
+    constexpr int PER_WAVE = STAGED ? (STAGE_PER_WAVE > RED_PER_WAVE ? STAGE_PER_WAVE : RED_PER_WAVE) : RED_PER_WAVE;
+    static_assert(SK_WAVES * PER_WAVE <= 160 * 1024, "staging does not fit the LDS");
 
-    __shared__ v4f red[SK_WAVES][NT][MB][kWave];
+    // per wavefront: staging of its K steps, later its partial sums (red[wave][nt][mb][lane])
+    __shared__ __attribute__((aligned(1024))) uint8_t smem[SK_WAVES * PER_WAVE];
+    auto red = [&](int w, int nt, int mb, int l) -> v4f& {
+        return reinterpret_cast<v4f*>(smem + w * PER_WAVE)[(nt * MB + mb) * kWave + l];
+    };
 
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     const int l16 = lane & 15, q = lane >> 4;
@@ -109,27 +126,21 @@ __global__ __launch_bounds__(SK_THREADS) void gemm_fp8_skinny_kernel(const Skinn
         }
     }
 
-    // ---- operand row pointers ---------------------------------------------------------
-    const uint8_t* wrow[NT];
-#pragma unroll
-    for (int nt = 0; nt < NT; ++nt) {
-        int r;
+    // ---- operand rows ----------------------------------------------------------------------
+    // weight row of operand row r16 (0..15) of tile nt, token row of operand row r16 of block mb
+    auto w_row = [&](int nt, int r16) -> int {
         if constexpr (GATED) {
-            const int g = col0 + nt * 8 + (l16 & 7);
-            r = (l16 < 8 ? 0 : half_n) + (g < half_n ? g : half_n - 1);
+            const int g = col0 + nt * 8 + (r16 & 7);
+            return (r16 < 8 ? 0 : half_n) + (g < half_n ? g : half_n - 1);
         } else {
-            r = col0 + nt * 16 + l16;
-            r = r < p.N ? r : p.N - 1;
+            const int r = col0 + nt * 16 + r16;
+            return r < p.N ? r : p.N - 1;
         }
-        wrow[nt] = p.w + (size_t)r * p.K + q * 16;
-    }
-    const uint8_t* xrow[MB];
-#pragma unroll
-    for (int mb = 0; mb < MB; ++mb) {
-        int r = m_base + mb * 16 + l16;
-        r = r < p.M ? r : p.M - 1;  // rows past M only feed outputs that are never stored
-        xrow[mb] = p.xq + (size_t)r * p.K + q * 16;
-    }
+    };
+    auto x_row = [&](int mb, int r16) -> int {
+        const int r = m_base + mb * 16 + r16;
+        return r < p.M ? r : p.M - 1;  // rows past M only feed outputs that are never stored
+    };
 
     v4f acc[NT][MB];
 #pragma unroll
@@ -137,56 +148,131 @@ __global__ __launch_bounds__(SK_THREADS) void gemm_fp8_skinny_kernel(const Skinn
 #pragma unroll
         for (int mb = 0; mb < MB; ++mb) acc[nt][mb] = v4f{0.f, 0.f, 0.f, 0.f};
 
-    for (int rnd = 0; rnd < p.rounds; ++rnd) {
-        v4i wlo[KPW][NT], whi[KPW][NT], xlo[KPW][MB], xhi[KPW][MB];
-        bool live[KPW];
-        // ---- 1. request every byte of this round ------------------------------------
+    if constexpr (!STAGED) {
+        const uint8_t* wrow[NT];
 #pragma unroll
-        for (int j = 0; j < KPW; ++j) {
-            const int s = (rnd * KPW + j) * SK_WAVES + wave;  // wave-uniform
-            live[j] = s < total_steps;
-            const int off = (live[j] ? s : total_steps - 1) << 7;
+        for (int nt = 0; nt < NT; ++nt) wrow[nt] = p.w + (size_t)w_row(nt, l16) * p.K + q * 16;
+        const uint8_t* xrow[MB];
 #pragma unroll
-            for (int nt = 0; nt < NT; ++nt) {
-                wlo[j][nt] = *reinterpret_cast<const v4i*>(wrow[nt] + off);
-                whi[j][nt] = *reinterpret_cast<const v4i*>(wrow[nt] + off + 64);
+        for (int mb = 0; mb < MB; ++mb) xrow[mb] = p.xq + (size_t)x_row(mb, l16) * p.K + q * 16;
+
+        for (int rnd = 0; rnd < p.rounds; ++rnd) {
+            v4i wlo[KPW][NT], whi[KPW][NT], xlo[KPW][MB], xhi[KPW][MB];
+            bool live[KPW];
+            // ---- 1. request every byte of this round ------------------------------------
+#pragma unroll
+            for (int j = 0; j < KPW; ++j) {
+                const int s = (rnd * KPW + j) * SK_WAVES + wave;  // wave-uniform
+                live[j] = s < total_steps;
+                const int off = (live[j] ? s : total_steps - 1) << 7;
+#pragma unroll
+                for (int nt = 0; nt < NT; ++nt) {
+                    wlo[j][nt] = *reinterpret_cast<const v4i*>(wrow[nt] + off);
+                    whi[j][nt] = *reinterpret_cast<const v4i*>(wrow[nt] + off + 64);
+                }
+#pragma unroll
+                for (int mb = 0; mb < MB; ++mb) {
+                    xlo[j][mb] = *reinterpret_cast<const v4i*>(xrow[mb] + off);
+                    xhi[j][mb] = *reinterpret_cast<const v4i*>(xrow[mb] + off + 64);
+                }
             }
+            // ---- 2. MFMA ---------------------------------------------------------------------
 #pragma unroll
-            for (int mb = 0; mb < MB; ++mb) {
-                xlo[j][mb] = *reinterpret_cast<const v4i*>(xrow[mb] + off);
-                xhi[j][mb] = *reinterpret_cast<const v4i*>(xrow[mb] + off + 64);
+            for (int j = 0; j < KPW; ++j) {
+#pragma unroll
+                for (int nt = 0; nt < NT; ++nt) {
+                    v8i a = join(wlo[j][nt], whi[j][nt]);
+                    if (!live[j]) a = v8i{0, 0, 0, 0, 0, 0, 0, 0};  // a step past K adds nothing
+#pragma unroll
+                    for (int mb = 0; mb < MB; ++mb)
+                        acc[nt][mb] = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(
+                            a, join(xlo[j][mb], xhi[j][mb]), acc[nt][mb], 0, 0, 0, 0, 0, 0);
+                }
             }
         }
-        // ---- 2. MFMA ---------------------------------------------------------------------
+    } else {
+        // Copy geometry: one instruction moves 8 operand rows x 128 bytes; lane i fills slot i%8 of
+        // row i/8 with chunk (i%8) ^ swz(row), swz(r) = (r/2)%8, which keeps the 128-bit reads of
+        // the MFMA layout (lane (l16, q): chunks q and 4+q of row l16) off each other's banks.
+        const int c_row = lane >> 3, c_slot = lane & 7;
+        uint32_t woff[NT][2], xoff[MB][2];
 #pragma unroll
-        for (int j = 0; j < KPW; ++j) {
+        for (int hf = 0; hf < 2; ++hf) {
+            const int r16 = hf * 8 + c_row;
+            const uint32_t chunk = (uint32_t)((c_slot ^ ((r16 >> 1) & 7)) << 4);
 #pragma unroll
-            for (int nt = 0; nt < NT; ++nt) {
-                v8i a = join(wlo[j][nt], whi[j][nt]);
-                if (!live[j]) a = v8i{0, 0, 0, 0, 0, 0, 0, 0};  // a step past K adds nothing
+            for (int nt = 0; nt < NT; ++nt) woff[nt][hf] = (uint32_t)w_row(nt, r16) * (uint32_t)p.K + chunk;
 #pragma unroll
-                for (int mb = 0; mb < MB; ++mb)
-                    acc[nt][mb] = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(
-                        a, join(xlo[j][mb], xhi[j][mb]), acc[nt][mb], 0, 0, 0, 0, 0, 0);
+            for (int mb = 0; mb < MB; ++mb) xoff[mb][hf] = (uint32_t)x_row(mb, r16) * (uint32_t)p.K + chunk;
+        }
+        const uint32_t lds_wave = __builtin_amdgcn_readfirstlane((uint32_t)(uintptr_t)smem + wave * PER_WAVE);
+        const uint8_t* my_stage = smem + wave * PER_WAVE;
+        const int swz = (l16 >> 1) & 7;
+        const int rd_lo = l16 * 128 + ((q ^ swz) << 4), rd_hi = l16 * 128 + (((4 + q) ^ swz) << 4);
+
+        for (int rnd = 0; rnd < p.rounds; ++rnd) {
+            if (rnd > 0) asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");   // last round's reads have landed
+            // ---- 1. request every byte of this round ------------------------------------
+#pragma unroll
+            for (int j = 0; j < KPW; ++j) {
+                const int s = __builtin_amdgcn_readfirstlane((rnd * KPW + j) * SK_WAVES + wave);
+                if (s < total_steps) {
+                    const uint32_t dst = lds_wave + j * (BLOCKS * 2048);
+#pragma unroll
+                    for (int nt = 0; nt < NT; ++nt)
+#pragma unroll
+                        for (int hf = 0; hf < 2; ++hf)
+                            copy16_to_lds(p.w + ((size_t)s << 7), woff[nt][hf], dst + (nt * 2 + hf) * 1024);
+#pragma unroll
+                    for (int mb = 0; mb < MB; ++mb)
+#pragma unroll
+                        for (int hf = 0; hf < 2; ++hf)
+                            copy16_to_lds(p.xq + ((size_t)s << 7), xoff[mb][hf], dst + ((NT + mb) * 2 + hf) * 1024);
+                }
+            }
+            wait_copies<0>();   // everything this wavefront asked for (epilogue operands included)
+            // ---- 2. MFMA ---------------------------------------------------------------------
+#pragma unroll
+            for (int j = 0; j < KPW; ++j) {
+                const int s = __builtin_amdgcn_readfirstlane((rnd * KPW + j) * SK_WAVES + wave);
+                if (s < total_steps) {
+                    const uint8_t* blk = my_stage + j * (BLOCKS * 2048);
+                    v8i xb[MB];
+#pragma unroll
+                    for (int mb = 0; mb < MB; ++mb)
+                        xb[mb] = join(*reinterpret_cast<const v4i*>(blk + (NT + mb) * 2048 + rd_lo),
+                                      *reinterpret_cast<const v4i*>(blk + (NT + mb) * 2048 + rd_hi));
+#pragma unroll
+                    for (int nt = 0; nt < NT; ++nt) {
+                        const v8i a = join(*reinterpret_cast<const v4i*>(blk + nt * 2048 + rd_lo),
+                                           *reinterpret_cast<const v4i*>(blk + nt * 2048 + rd_hi));
+#pragma unroll
+                        for (int mb = 0; mb < MB; ++mb)
+                            acc[nt][mb] = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(
+                                a, xb[mb], acc[nt][mb], 0, 0, 0, 0, 0, 0);
+                    }
+                }
             }
         }
+        // the partial sums below overwrite this wavefront's own staging: its reads must be done
+        asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
     }
 
     // ---- 3. add the eight wavefronts' partial sums, in wavefront order -------------------
 #pragma unroll
     for (int nt = 0; nt < NT; ++nt)
 #pragma unroll
-        for (int mb = 0; mb < MB; ++mb) red[wave][nt][mb][lane] = acc[nt][mb];
+        for (int mb = 0; mb < MB; ++mb) red(wave, nt, mb, lane) = acc[nt][mb];
     __syncthreads();
     if (!e_role) return;
-    v4f g = red[0][e_nt][e_mb][e_lane];
+    v4f g = red(0, e_nt, e_mb, e_lane);
 #pragma unroll
-    for (int w = 1; w < SK_WAVES; ++w) g += red[w][e_nt][e_mb][e_lane];
+    for (int w = 1; w < SK_WAVES; ++w) g += red(w, e_nt, e_mb, e_lane);
     v4f u = v4f{0.f, 0.f, 0.f, 0.f};
     if constexpr (GATED) {
-        u = red[0][e_nt][e_mb][e_lane + 32];
+        u = red(0, e_nt, e_mb, e_lane + 32);
 #pragma unroll
-        for (int w = 1; w < SK_WAVES; ++w) u += red[w][e_nt][e_mb][e_lane + 32];
+        for (int w = 1; w < SK_WAVES; ++w) u += red(w, e_nt, e_mb, e_lane + 32);
     }
 
     // ---- 4. epilogue ------------------------------------------------------------------------
@@ -270,13 +356,27 @@ SkinnyPlan skinny_plan(int M, int N, int K, int epilogue) {
     return pl;
 }
 
+// The staged form wherever its LDS fits (8 wavefronts x KPW steps x (NT + MB) blocks of 2 KB).
+template <int MB, int NT, int KPW, int EPI>
+static void sk_launch_one(const SkinnyArgs& a, const dim3& grid, hipStream_t st) {
+    constexpr bool fits = SK_WAVES * KPW * (NT + MB) * 2048 <= 128 * 1024;
+    static const bool want = []() { const char* e = getenv("PHYAI_FP8_SKINNY_STAGED"); return !(e && atoi(e) == 0); }();
+    if constexpr (fits) {
+        if (want && a.K * (int64_t)(a.N > a.M ? a.N : a.M) < ((int64_t)1 << 32)) {
+            hipLaunchKernelGGL((gemm_fp8_skinny_kernel<MB, NT, KPW, EPI, true>), grid, dim3(SK_THREADS), 0, st, a);
+            return;
+        }
+    }
+    hipLaunchKernelGGL((gemm_fp8_skinny_kernel<MB, NT, KPW, EPI, false>), grid, dim3(SK_THREADS), 0, st, a);
+}
+
 template <int MB, int NT, int EPI>
 static int sk_launch_kpw(const SkinnyArgs& a, const SkinnyPlan& pl, hipStream_t st) {
-    const dim3 grid(pl.tiles, pl.msplit), block(SK_THREADS);
+    const dim3 grid(pl.tiles, pl.msplit);
     switch (pl.kpw) {
-    case 1: hipLaunchKernelGGL((gemm_fp8_skinny_kernel<MB, NT, 1, EPI>), grid, block, 0, st, a); return 0;
-    case 2: hipLaunchKernelGGL((gemm_fp8_skinny_kernel<MB, NT, 2, EPI>), grid, block, 0, st, a); return 0;
-    case 4: hipLaunchKernelGGL((gemm_fp8_skinny_kernel<MB, NT, 4, EPI>), grid, block, 0, st, a); return 0;
+    case 1: sk_launch_one<MB, NT, 1, EPI>(a, grid, st); return 0;
+    case 2: sk_launch_one<MB, NT, 2, EPI>(a, grid, st); return 0;
+    case 4: sk_launch_one<MB, NT, 4, EPI>(a, grid, st); return 0;
     default: return -2;
     }
 }
