@@ -433,7 +433,7 @@ static int big_tiles(int M, int N, int epilogue, int bm, int bn) {
 // only about 45 GB/s from L2, so a mid-sized GEMM finishes sooner on more CUs even though the
 // partial sums then make a round trip through memory.
 BigPlan big_plan(int M, int N, int K, int epilogue) {
-    BigPlan pl = {0, 1};
+    BigPlan pl = {0, 1, 0};
     if (K % 128 != 0 || K < 512) return pl;   // slabs come in pairs and must fill the ring
     int forced = -1;
     if (const char* e = getenv("PHYAI_FP8_BIG")) forced = atoi(e);   // "0": never; "256"/"128": force
@@ -444,6 +444,7 @@ BigPlan big_plan(int M, int N, int K, int epilogue) {
     else if (big_tiles(M, N, epilogue, 128, 128) >= 32) pl.tile = 128;   // fewer: the weight-streaming kernel wins
     else return pl;
     const int tiles = big_tiles(M, N, epilogue, pl.tile, pl.tile);
+    pl.tiles = tiles;
     if (pl.tile == 128) {
         // Measured at M = 816: splitting pays for K = 16384 (67 -> 49 us with two splits) and
         // costs for K = 2048 (19 -> 25 us): the partial-sum round trip is worth about 6 us.

@@ -346,6 +346,9 @@ SkinnyPlan skinny_plan(int M, int N, int K, int epilogue) {
     const int steps = K / 128;
     const int per_wave = sk_ceil_div(steps, SK_WAVES);
     pl.kpw = per_wave >= 4 ? 4 : (per_wave >= 2 ? 2 : 1);
+    // staging of 8 wavefronts x kpw steps x (nt + mb) blocks of 2 KB must fit the 160 KB of LDS:
+    // more rounds of fewer steps beat the unstaged form (down 50..400 x 1024 x 4096: 12 -> 7 us)
+    while (pl.kpw > 1 && SK_WAVES * pl.kpw * (pl.nt + pl.mb) * 2048 > 160 * 1024) pl.kpw /= 2;
     pl.rounds = sk_ceil_div(per_wave, pl.kpw);
     if (const char* e = getenv("PHYAI_FP8_SKINNY_PLAN")) {  // "nt,mb" tuning override
         int nt = 0, mb = 0;
@@ -359,7 +362,7 @@ SkinnyPlan skinny_plan(int M, int N, int K, int epilogue) {
 // The staged form wherever its LDS fits (8 wavefronts x KPW steps x (NT + MB) blocks of 2 KB).
 template <int MB, int NT, int KPW, int EPI>
 static void sk_launch_one(const SkinnyArgs& a, const dim3& grid, hipStream_t st) {
-    constexpr bool fits = SK_WAVES * KPW * (NT + MB) * 2048 <= 128 * 1024;
+    constexpr bool fits = SK_WAVES * KPW * (NT + MB) * 2048 <= 160 * 1024;
     static const bool want = []() { const char* e = getenv("PHYAI_FP8_SKINNY_STAGED"); return !(e && atoi(e) == 0); }();
     if constexpr (fits) {
         if (want && a.K * (int64_t)(a.N > a.M ? a.N : a.M) < ((int64_t)1 << 32)) {

@@ -349,10 +349,12 @@ static int launch_epi(const TileArgs& a, const TileConfig& c, dim3 grid, hipStre
 
 int launch_gemm(const GemmProblem& g, hipStream_t st) {
     if (g.M == 0 || g.N == 0) return 0;
-    // Kernel choice (measured on the expert and prefill shapes):
+    // Kernel choice (measured on the expert and prefill shapes, M = 50 .. 13056):
     //   M <= 64                      weight-streaming kernel, nothing else comes close;
-    //   pipelined tile kernel        as soon as its grid has enough tiles (big_plan);
-    //   64 < M <= 512 otherwise      weight-streaming kernel again (few output columns);
+    //   pipelined tile kernel        256 x 256 tiles, or at least 64 tiles of 128 x 128;
+    //   64 < M <= 512 otherwise      weight-streaming kernel again (few output columns: at
+    //                                N = 1024 it wins up to M = 512, at N = 2560 up to M = 300);
+    //   32 .. 63 small tiles         pipelined tile kernel after all (M > 512);
     //   the rest                     generic LDS tile kernel (any K, any alignment).
     // The weight-streaming kernel reads scales / bias / output with 128- and 64-bit accesses.
     const bool vec_ok = (reinterpret_cast<uintptr_t>(g.w_scale) % 16 == 0) &&
@@ -362,7 +364,8 @@ int launch_gemm(const GemmProblem& g, hipStream_t st) {
     if (skinny_ok && g.M <= 64) return launch_gemm_skinny(g, skinny_plan(g.M, g.N, g.K, g.epilogue), st);
     if (!getenv("PHYAI_FP8_TILE")) {
         const BigPlan bp = big_plan(g.M, g.N, g.K, g.epilogue);
-        if (bp.tile) {
+        const bool few_small_tiles = bp.tile == 128 && bp.tiles < 64 && !getenv("PHYAI_FP8_BIG");
+        if (bp.tile && !(few_small_tiles && skinny_ok)) {
             const int rc = launch_gemm_big(g, bp, st);
             if (rc != -2) return rc;  // -2: output not 16-byte addressable, try the others
         }

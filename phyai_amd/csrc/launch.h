@@ -94,6 +94,7 @@ int launch_gemm_skinny(const GemmProblem& p, const SkinnyPlan& pl, hipStream_t s
 struct BigPlan {
     int tile;    // 256, 128, or 0 if the kernel does not apply
     int splits;
+    int tiles;   // output tiles of that size
 };
 BigPlan big_plan(int M, int N, int K, int epilogue);
 size_t big_partial_bytes(int M, int N, int epilogue, const BigPlan& pl);
