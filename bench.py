@@ -56,7 +56,7 @@ DIT_SET = [("qkv", 6144, 2048, None, 4800), ("out", 2048, 2048, None, 4800),
 # HBM bytes moved by one layer's four GEMM launches at M = 50 (20.87 MB fetched + 0.87 MB written),
 # measured with rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE on `bench.py --probe` and calibrated against
 # a 64 MiB copy (profiles/expert_m50_hbm_traffic.md has the counter values).
-EXPERT_LAYER_HBM_TRAFFIC = 21_740_000
+EXPERT_LAYER_HBM_TRAFFIC = 21_780_000
 
 
 def algorithmic_bytes(M: int, N: int, K: int, epilogue, bias: bool = False) -> int:
@@ -140,9 +140,9 @@ def torch_reference_times(dev, layers, shapes, denoise_steps, steps, warmup):
 def decoder_layer_times(dev, layers, M, denoise_steps, steps, warmup):
     """The expert layer's linear path WITH its neighbours (adaptive norms before qkv / gate_up, gated
     residuals after o / down; reference models/pi05/modeling_pi05.py:812-835), two ways on the same
-    tensors: `separate` = norm, quantizer, GEMM and addcmul as their own launches (12 per layer, the
+    tensors: `separate` = norm, quantizer, GEMM and addcmul as their own kernels (12 per layer, the
     reference's structure), `fused` = norm+quantizer in one kernel, addcmul in the GEMM epilogue
-    (6 per layer).  Attention and RoPE are not part of either."""
+    (8 per layer).  Attention and RoPE are not part of either."""
     from phyai_amd import ops
     from phyai_amd.runtime import HipGraph
 
@@ -329,6 +329,9 @@ def main() -> int:
     ap.add_argument("--warmup", type=int, default=20)
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--no-prefill", action="store_true")
+    ap.add_argument("--no-extras", action="store_true",
+                    help="skip the comparisons in `extra` (fused decoder-layer path, torch reference path): "
+                         "only this library's kernels run, for profiler sessions")
     ap.add_argument("--sweep", action="store_true",
                     help="also time the batched-serving sweep (B = 1..16, both linear sets, outlier channels)")
     ap.add_argument("--probe", action="store_true",
@@ -398,20 +401,21 @@ def main() -> int:
         pts, _ = time_replays(pg, 30, 3)
         p_layer_us = statistics.median(pts) * 1e3 / len(pl)
         flops = sum(2 * 816 * N * K for _, N, K, _ in PREFILL_SET)
-        tref = torch_reference_times(dev, pl, PREFILL_SET, 1, 10, 3)
+        tref = "skipped" if args.no_extras else torch_reference_times(dev, pl, PREFILL_SET, 1, 10, 3)
         extra["prefill_M816"] = {"torch_reference_path_us_per_layer": (round(tref / len(pl), 2) if not isinstance(tref, str) else tref),
                                  "us_per_layer": round(p_layer_us, 2),
                                  "TFLOP/s": round(flops / (p_layer_us * 1e-6) / 1e12, 1),
                                  "frac_fp8_peak": round(flops / (p_layer_us * 1e-6) / 1e12 / FP8_PEAK_TFLOPS, 4)}
         del pl, pg
-    dl = decoder_layer_times(dev, layers, M, denoise_steps, max(20, args.steps // 4), 5)
-    extra["expert_step_with_norms_and_residuals_us"] = {
-        **dl, "note": "per denoise step, 18 layers: adaptive norm -> qkv, o -> gated residual, adaptive norm -> "
-                      "gate_up+GeGLU, down -> gated residual; separate = 12 launches per layer, fused = 6"}
-    extra["torch_reference_path_us"] = {
-        "expert_step": torch_reference_times(dev, layers, EXPERT_SET, denoise_steps, max(10, args.steps // 10), 3),
-        "note": "same linears through the reference's own arithmetic on this GPU: torch-op quantizer + "
-                "torch._scaled_mm (+ torch GELU*up); compare with `value`"}
+    if not args.no_extras:
+        dl = decoder_layer_times(dev, layers, M, denoise_steps, max(20, args.steps // 4), 5)
+        extra["expert_step_with_norms_and_residuals_us"] = {
+            **dl, "note": "per denoise step, 18 layers: adaptive norm -> qkv, o -> gated residual, adaptive norm -> "
+                          "gate_up+GeGLU, down -> gated residual; separate = 12 kernels per layer, fused = 8"}
+        extra["torch_reference_path_us"] = {
+            "expert_step": torch_reference_times(dev, layers, EXPERT_SET, denoise_steps, max(10, args.steps // 10), 3),
+            "note": "same linears through the reference's own arithmetic on this GPU: torch-op quantizer + "
+                    "torch._scaled_mm (+ torch GELU*up); compare with `value`"}
     if args.sweep:
         extra["batched_sweep"] = sweep(dev)
 
