@@ -1,7 +1,9 @@
 // MFMA-bound fp8 GEMM for large M (prefix prefill, batched serving).
 // Workgroup = 4 wavefronts (2 x 2); a wavefront owns TM x TN blocks of 32 x 32, so the
-// workgroup tile is 64*TM x 64*TN: 256 x 256 (TM = TN = 4) when the grid still fills the chip,
-// 128 x 128 (TM = TN = 2, two workgroups per CU) for mid-sized problems.
+// workgroup tile is 64*TM x 64*TN: 256 x 256 (TM = TN = 4, one workgroup per CU) for long K,
+// 192 x 128 (TM = 3, TN = 2, two workgroups per CU) when there are plenty of tiles and K is short,
+// 128 x 128 (TM = TN = 2; ring of four stages, or of two with two workgroups per CU) for
+// mid-sized problems.
 //
 // Why 4 x 4 blocks per wavefront.  One v_mfma_f32_32x32x64_f8f6f4 takes 64 cycles and consumes
 // two 2 KB operand blocks.  A wavefront with TM x TN blocks reads (TM + TN) blocks from LDS per
@@ -59,6 +61,7 @@ struct BigArgs {
     float* __restrict__ partials;
     int* __restrict__ counters;
     int m_tiles, n_tiles;            // tile grid; the launch is 1-D over it (see big_tile_of)
+    int band;                        // tile rows per band of that order
     ResidualArgs res;
 };
 
@@ -70,14 +73,14 @@ struct BigArgs {
 // from HBM once per band - while the activation rows of the band stay in its L2.  Tile columns
 // are padded to a multiple of 8; ids that fall into the padding have no tile.
 struct BigTile { int m, n; };
-__device__ __forceinline__ BigTile big_tile_of(int id, int m_tiles, int n_tiles) {
+__device__ __forceinline__ BigTile big_tile_of(int id, int m_tiles, int n_tiles, int band_rows) {
     const int nt8 = (n_tiles + 7) & ~7;
-    const int band = id / (4 * nt8);
-    const int local = id - band * 4 * nt8;
-    const int bm = m_tiles - 4 * band < 4 ? m_tiles - 4 * band : 4;
+    const int band = id / (band_rows * nt8);
+    const int local = id - band * band_rows * nt8;
+    const int bm = m_tiles - band_rows * band < band_rows ? m_tiles - band_rows * band : band_rows;
     BigTile t;
     t.n = (local / (8 * bm)) * 8 + (local & 7);
-    t.m = 4 * band + (local >> 3) % bm;
+    t.m = band_rows * band + (local >> 3) % bm;
     return t;
 }
 
@@ -102,8 +105,12 @@ __device__ __forceinline__ v8i big_frag(const uint8_t* buf, int row, int h, int 
 }
 
 // DEPTH: stages of the LDS ring, each holding BIG_BK bytes of K for the whole tile.
+// Variants whose ring leaves room for two workgroups per CU are held to the register budget of
+// two wavefronts per SIMD: while one workgroup is in its prologue or epilogue the other one
+// keeps the MFMA pipe busy.
 template <int TM, int TN, int DEPTH, int EPI, bool SPLIT>
-__global__ __launch_bounds__(256) void gemm_fp8_big_kernel(const BigArgs p) {
+__global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu((DEPTH == 2 && TM < 4) ? 2 : 1)))
+void gemm_fp8_big_kernel(const BigArgs p) {
     constexpr bool GATED = epi_is_gated(EPI);
     constexpr int BM = 64 * TM, BN = 64 * TN;        // workgroup tile
     constexpr int WM = 32 * TM, WN = 32 * TN;        // wavefront tile
@@ -112,7 +119,7 @@ __global__ __launch_bounds__(256) void gemm_fp8_big_kernel(const BigArgs p) {
     constexpr int COPIES = CA + CB;
     constexpr int SLOTS_PER_STAGE = 2 * TM * TN;     // MFMAs of a wavefront per stage
     constexpr int CPS = (COPIES * 2 + SLOTS_PER_STAGE - 1) / SLOTS_PER_STAGE;   // copies per MFMA: done by mid-stage
-    static_assert(TM == TN && TM % 2 == 0, "square wavefront tile, even block count");
+    static_assert((TM == TN && TM % 2 == 0) || (TM == 3 && TN == 2), "supported wavefront tiles");
     static_assert(DEPTH == 2 || DEPTH == 4, "ring depth");
     __shared__ __attribute__((aligned(1024))) uint8_t lds[DEPTH * STAGE_BYTES];
 
@@ -120,7 +127,7 @@ __global__ __launch_bounds__(256) void gemm_fp8_big_kernel(const BigArgs p) {
     const int wm = wave >> 1, wn = wave & 1;
     const int l32 = lane & 31, h = lane >> 5;
     const int half_n = p.N / 2;
-    const BigTile tile_id = big_tile_of(blockIdx.x, p.m_tiles, p.n_tiles);
+    const BigTile tile_id = big_tile_of(blockIdx.x, p.m_tiles, p.n_tiles, p.band);
     if (tile_id.n >= p.n_tiles) return;              // padding of the tile order
     const int m0 = tile_id.m * BM;
     const int n0 = GATED ? tile_id.n * (BN / 2) : tile_id.n * BN;
@@ -432,64 +439,79 @@ static int big_tiles(int M, int N, int epilogue, int bm, int bn) {
 // tiles, and those are split along K when even the small tiles leave CUs idle: a CU can pull
 // only about 45 GB/s from L2, so a mid-sized GEMM finishes sooner on more CUs even though the
 // partial sums then make a round trip through memory.
+static int big_tile_cols(int tile) { return tile == 256 ? 256 : 128; }
+
 BigPlan big_plan(int M, int N, int K, int epilogue) {
-    BigPlan pl = {0, 1, 0};
+    BigPlan pl = {0, 1, 0, 0};
     if (K % 128 != 0 || K < 512) return pl;   // slabs come in pairs and must fill the ring
     int forced = -1;
-    if (const char* e = getenv("PHYAI_FP8_BIG")) forced = atoi(e);   // "0": never; "256"/"128": force
+    if (const char* e = getenv("PHYAI_FP8_BIG")) forced = atoi(e);   // "0": never; "256"/"192"/"128": force
     if (forced == 0) return pl;
-    if (forced == 256 || forced == 128) pl.tile = forced;
+    if (forced == 256 || forced == 192 || forced == 128) pl.tile = forced;
     else if (M < 128) return pl;
+    // 256 x 256 tiles need the fewest bytes from L2 per flop but run one workgroup per CU, so a
+    // tile's prologue and epilogue leave the MFMA pipe idle; 192 x 128 tiles fit twice and overlap
+    // them.  The small tile wins once there are enough of them and while K is short enough for
+    // prologue and epilogue to matter (measured: 4-18 % up to K = 8192), unless M pads worse.
+    else if (K <= 8192 && big_tiles(M, N, epilogue, 192, 128) >= 400 &&
+             big_ceil_div(M, 192) * 192 <= big_ceil_div(M, 256) * 256) pl.tile = 192;
     else if (big_tiles(M, N, epilogue, 256, 256) >= 200) pl.tile = 256;
     else if (big_tiles(M, N, epilogue, 128, 128) >= 32) pl.tile = 128;   // fewer: the weight-streaming kernel wins
     else return pl;
-    const int tiles = big_tiles(M, N, epilogue, pl.tile, pl.tile);
+    const int tiles = big_tiles(M, N, epilogue, pl.tile, big_tile_cols(pl.tile));
     pl.tiles = tiles;
+    pl.depth = pl.tile == 128 ? 4 : 2;
     if (pl.tile == 128) {
         // Measured at M = 816: splitting pays for K = 16384 (67 -> 49 us with two splits) and
         // costs for K = 2048 (19 -> 25 us): the partial-sum round trip is worth about 6 us.
         if (tiles < 200 && K >= 8192 && K % 256 == 0) pl.splits = 2;
+        // With well over one tile per CU a ring of two stages lets two workgroups share a CU
+        // (17.5 -> 14.4 us at 800 x 8192 x 1024); with fewer, the deeper ring hides more latency.
+        else if (tiles >= 400) pl.depth = 2;
     }
     if (const char* e = getenv("PHYAI_FP8_BIG_SPLITS")) {
         const int s = atoi(e);
-        if (s >= 1 && K % (s * 128) == 0 && K / s >= 512 && tiles * s <= 4096) pl.splits = s;
+        if (pl.tile != 192 && s >= 1 && K % (s * 128) == 0 && K / s >= 512 && tiles * s <= 4096) pl.splits = s;
+    }
+    if (const char* e = getenv("PHYAI_FP8_BIG_DEPTH")) {
+        const int d = atoi(e);
+        if (pl.tile == 128 && pl.splits == 1 && (d == 2 || d == 4)) pl.depth = d;
     }
     return pl;
 }
 
 size_t big_partial_bytes(int M, int N, int epilogue, const BigPlan& pl) {
     if (pl.splits <= 1) return 0;
-    return (size_t)big_tiles(M, N, epilogue, pl.tile, pl.tile) * pl.splits * pl.tile * pl.tile * sizeof(float);
+    const int bn = big_tile_cols(pl.tile);
+    return (size_t)big_tiles(M, N, epilogue, pl.tile, bn) * pl.splits * pl.tile * bn * sizeof(float);
 }
 
-#ifndef BIG_DEPTH_SMALL
-#define BIG_DEPTH_SMALL 4
-#endif
-template <int T, int EPI>
+template <int TM, int TN, int DEPTH, int EPI>
 static void big_launch(BigArgs a, const GemmProblem& g, int splits, hipStream_t st) {
     const bool gated = epi_is_gated(EPI);
-    const int bn_eff = gated ? 32 * T : 64 * T;
+    const int bn_eff = gated ? 32 * TN : 64 * TN;
     a.n_tiles = big_ceil_div(gated ? g.N / 2 : g.N, bn_eff);
-    a.m_tiles = big_ceil_div(g.M, 64 * T);
+    a.m_tiles = big_ceil_div(g.M, 64 * TM);
+    a.band = 4;
+    if (const char* e = getenv("PHYAI_FP8_BAND")) { const int b = atoi(e); if (b >= 1 && b <= 16) a.band = b; }
     const dim3 grid(a.m_tiles * ((a.n_tiles + 7) & ~7), 1, splits);
-    if constexpr (T == 2) {
-        if (splits > 1) hipLaunchKernelGGL((gemm_fp8_big_kernel<2, 2, BIG_DEPTH_SMALL, EPI, true>), grid, dim3(256), 0, st, a);
-        else hipLaunchKernelGGL((gemm_fp8_big_kernel<2, 2, BIG_DEPTH_SMALL, EPI, false>), grid, dim3(256), 0, st, a);
+    if (splits > 1) {
+        if constexpr (TM == TN && (TM == 4 || DEPTH == 4))
+            hipLaunchKernelGGL((gemm_fp8_big_kernel<TM, TN, DEPTH, EPI, true>), grid, dim3(256), 0, st, a);
     } else {
-        if (splits > 1) hipLaunchKernelGGL((gemm_fp8_big_kernel<4, 4, 2, EPI, true>), grid, dim3(256), 0, st, a);
-        else hipLaunchKernelGGL((gemm_fp8_big_kernel<4, 4, 2, EPI, false>), grid, dim3(256), 0, st, a);
+        hipLaunchKernelGGL((gemm_fp8_big_kernel<TM, TN, DEPTH, EPI, false>), grid, dim3(256), 0, st, a);
     }
 }
 
-template <int T>
+template <int TM, int TN, int DEPTH>
 static int big_launch_epi(const BigArgs& a, const GemmProblem& g, int splits, hipStream_t st) {
     switch (g.epilogue) {
-    case EPI_NONE: big_launch<T, EPI_NONE>(a, g, splits, st); return 0;
-    case EPI_GEGLU_TANH: big_launch<T, EPI_GEGLU_TANH>(a, g, splits, st); return 0;
-    case EPI_GEGLU_ERF: big_launch<T, EPI_GEGLU_ERF>(a, g, splits, st); return 0;
-    case EPI_SWIGLU: big_launch<T, EPI_SWIGLU>(a, g, splits, st); return 0;
-    case EPI_GELU_TANH: big_launch<T, EPI_GELU_TANH>(a, g, splits, st); return 0;
-    case EPI_GELU_ERF: big_launch<T, EPI_GELU_ERF>(a, g, splits, st); return 0;
+    case EPI_NONE: big_launch<TM, TN, DEPTH, EPI_NONE>(a, g, splits, st); return 0;
+    case EPI_GEGLU_TANH: big_launch<TM, TN, DEPTH, EPI_GEGLU_TANH>(a, g, splits, st); return 0;
+    case EPI_GEGLU_ERF: big_launch<TM, TN, DEPTH, EPI_GEGLU_ERF>(a, g, splits, st); return 0;
+    case EPI_SWIGLU: big_launch<TM, TN, DEPTH, EPI_SWIGLU>(a, g, splits, st); return 0;
+    case EPI_GELU_TANH: big_launch<TM, TN, DEPTH, EPI_GELU_TANH>(a, g, splits, st); return 0;
+    case EPI_GELU_ERF: big_launch<TM, TN, DEPTH, EPI_GELU_ERF>(a, g, splits, st); return 0;
     default: return -2;
     }
 }
@@ -508,8 +530,10 @@ int launch_gemm_big(const GemmProblem& g, const BigPlan& pl, hipStream_t st) {
     if (pl.splits > 1 && (g.workspace == nullptr ||
                           g.workspace_bytes < kGemmHeaderBytes + big_partial_bytes(g.M, g.N, g.epilogue, pl)))
         return -3;
-    if (pl.tile == 256) return big_launch_epi<4>(a, g, pl.splits, st);
-    if (pl.tile == 128) return big_launch_epi<2>(a, g, pl.splits, st);
+    if (pl.tile == 256) return big_launch_epi<4, 4, 2>(a, g, pl.splits, st);
+    if (pl.tile == 192 && pl.splits == 1) return big_launch_epi<3, 2, 2>(a, g, 1, st);
+    if (pl.tile == 128 && pl.depth == 4) return big_launch_epi<2, 2, 4>(a, g, pl.splits, st);
+    if (pl.tile == 128 && pl.splits == 1) return big_launch_epi<2, 2, 2>(a, g, 1, st);
     return -2;
 }
 

@@ -279,7 +279,7 @@ def test_linear_epilogues(dev, epi_name, epi, M, N, K):
 
 
 @pytest.mark.parametrize("epi_name,epi", [("gelu_tanh", 4), ("gelu", 5), ("geglu_tanh", 1), ("geglu_erf", 2), ("swiglu", 3)])
-@pytest.mark.parametrize("M,force_big", [(64, ""), (256, "256"), (256, "128")])
+@pytest.mark.parametrize("M,force_big", [(64, ""), (256, "256"), (256, "128"), (200, "192")])
 def test_epilogue_activation_values(dev, monkeypatch, epi_name, epi, M, force_big):
     """One-hot weights hand chosen values to the epilogue: every e4m3 value times a per-row power of
     two reaches the activation exactly, so the device activation is compared with torch's value by
@@ -365,17 +365,25 @@ def test_linear_repeatable_and_workspace_stays_clean(dev):
 
 
 # ---------------------------------------------------------------------------
-# 256 x 256 tile kernel (large M), forced on shapes small enough for the oracle
+# Pipelined tile kernel (large M), every variant forced on shapes small enough for the oracle
 # ---------------------------------------------------------------------------
+
+def _force_big(monkeypatch, spec):
+    """spec = "rows" or "rows/ring depth": 256 (x 256 columns), 192 (x 128), 128 (x 128, ring of 4 or 2)."""
+    tile, _, depth = spec.partition("/")
+    monkeypatch.setenv("PHYAI_FP8_BIG", tile)
+    if depth:
+        monkeypatch.setenv("PHYAI_FP8_BIG_DEPTH", depth)
+
 
 @pytest.mark.parametrize("M,N,K,epi_name,epi", [
     (256, 256, 1024, None, 0), (300, 512, 1280, None, 0), (816, 768, 1024, None, 0), (513, 400, 1536, "gelu", 5),
     (816, 1024, 1152, "geglu_tanh", 1), (260, 288, 1024, "swiglu", 3), (1000, 256, 2048, None, 0),
 ])
-@pytest.mark.parametrize("tile", ["256", "128"])
+@pytest.mark.parametrize("tile", ["256", "192", "128", "128/2"])
 def test_big_tile_kernel_forced(dev, monkeypatch, tile, M, N, K, epi_name, epi):
     ops = _ops()
-    monkeypatch.setenv("PHYAI_FP8_BIG", tile)
+    _force_big(monkeypatch, tile)
     x, wq, ws, b = _problem(M, N, K, seed=7 * M + N + K)
     got = ops.fp8_linear(x.to(dev), wq.to(dev), ws.to(dev), b.to(dev), epilogue=epi_name)
     torch.cuda.synchronize()
@@ -384,10 +392,10 @@ def test_big_tile_kernel_forced(dev, monkeypatch, tile, M, N, K, epi_name, epi):
     assert_close_to_ref(got, want, f"big kernel {M}x{N}x{K} epi={epi_name}")
 
 
-@pytest.mark.parametrize("tile", ["256", "128"])
+@pytest.mark.parametrize("tile", ["256", "192", "128", "128/2"])
 def test_big_tile_kernel_exact_integer(dev, monkeypatch, tile):
     ops = _ops()
-    monkeypatch.setenv("PHYAI_FP8_BIG", tile)
+    _force_big(monkeypatch, tile)
     g = torch.Generator().manual_seed(11)
     for (M, N, K) in [(256, 256, 1024), (700, 528, 1280), (257, 784, 1152)]:
         xi = torch.randint(-4, 5, (M, K), generator=g).float()
@@ -451,7 +459,8 @@ def test_quant_rowwise_exhaustive_all_values_all_scales(dev):
 
 @pytest.mark.parametrize("M,N,K,force,gate_rows", [
     (50, 1024, 2048, "", 1), (50, 1024, 4096, "", 50), (200, 1024, 4096, "", 4), (70, 192, 272, "", 70),
-    (816, 2048, 2048, "128", 816), (816, 2048, 2048, "256", 1), (300, 384, 4096, "128", 3), (9, 64, 128, "", 9)])
+    (816, 2048, 2048, "128", 816), (816, 2048, 2048, "256", 1), (300, 384, 4096, "128", 3), (9, 64, 128, "", 9),
+    (816, 2048, 2048, "192", 816), (500, 640, 1024, "192", 5)])
 def test_linear_gated_residual(dev, monkeypatch, M, N, K, force, gate_rows):
     """out = addcmul(residual, linear(x), gate) inside the GEMM epilogue, every kernel family; the result
     must equal torch.addcmul applied to the device's own plain linear output bit for bit."""
@@ -516,7 +525,7 @@ def test_quantizer_bit_exact_with_reference_expressions_on_device(dev, shape):
 
 @pytest.mark.parametrize("M,N,K,force", [(50, 2560, 1024, ""), (50, 1024, 4096, ""), (200, 1024, 2048, ""),
                                          (816, 2560, 2048, ""), (816, 2048, 16384, ""), (816, 4096, 2048, "256"),
-                                         (70, 192, 272, "")])
+                                         (816, 4096, 2048, "192"), (70, 192, 272, "")])
 def test_gemm_against_torch_scaled_mm(dev, monkeypatch, M, N, K, force):
     """torch._scaled_mm with row-wise scales is the GEMM the reference calls
     (layers/linear/backends/torch.py:166-175).  Same codes, same scales, same bias on this GPU: the
