@@ -427,6 +427,49 @@ def test_big_tile_kernel_split_k(dev, monkeypatch, tile):
         assert int(w[: ops.WORKSPACE_HEADER_BYTES].max().item()) == 0
 
 
+@pytest.mark.parametrize("M,N,K,epi_name", [
+    (50, 1024, 2048, None), (50, 1024, 4096, None), (16, 1024, 1024, None), (64, 512, 2048, None),
+    (33, 1024, 4096, "gelu_tanh"), (50, 2048, 2048, "geglu_tanh"), (7, 256, 1024, "swiglu"), (48, 768, 4096, None),
+])
+def test_linear_equals_quantizer_then_gemm_bit_for_bit(dev, M, N, K, epi_name):
+    """The linear entry point (bf16 in) against the GEMM entry point fed by the stand-alone quantizer
+    (whose codes and scales are pinned bit-exactly elsewhere): the outputs must be equal bit for
+    bit, whatever staging the library uses between its quantizer and its GEMM.  Rows with zeros
+    only, a signed zero, an outlier, tiny values, the largest finite bf16 and an Inf are
+    included, and the activations are also passed as a strided view."""
+    ops = _ops()
+    x, wq, ws, b = _problem(M, N, K, seed=3 * M + N + K)
+    x = x.clone()
+    x[0] = 0
+    x[1, ::2] = -0.0
+    x[2, 5] = 300.0
+    x[3] = x[3] * 1e-30
+    if M > 5:
+        x[4, 7] = torch.finfo(torch.bfloat16).max
+        x[5, 3] = float("inf")
+    wide = torch.zeros(M, K + 64, dtype=torch.bfloat16)
+    wide[:, :K] = x
+    xd = wide.to(dev)[:, :K]                                   # row stride K + 64
+    assert not xd.is_contiguous()
+    wd, sd, bd = wq.to(dev), ws.to(dev), b.to(dev)
+    xq, xs = ops.fp8_quant_rowwise(x.to(dev))
+    want = ops.fp8_gemm(xq, xs, wd, sd, bd, epilogue=epi_name)
+    for xin in (x.to(dev), xd):
+        got = ops.fp8_linear(xin, wd, sd, bd, epilogue=epi_name)
+        torch.cuda.synchronize()
+        assert torch.equal(_as_bits(got), _as_bits(want)), f"{(M, N, K, epi_name)}: {int((_as_bits(got) != _as_bits(want)).sum())} outputs differ"
+    if epi_name is None:
+        res = seeded((M, N), seed=8)
+        gate = seeded((1, N), seed=9, scale=0.5)
+        want = ops.fp8_gemm(xq, xs, wd, sd, bd, residual=res.to(dev), gate=gate.to(dev))
+        got = ops.fp8_linear(xd, wd, sd, bd, residual=res.to(dev), gate=gate.to(dev))
+        assert torch.equal(_as_bits(got), _as_bits(want))
+
+
+def _as_bits(t):
+    return t.contiguous().view(torch.int16)
+
+
 def test_quant_rowwise_exhaustive_all_values_all_scales(dev):
     """Every finite bf16 value against every possible row maximum (32 640 of them, hence every
     possible scale): 2.1e9 quotients.  The expected codes are the reference's own expression
