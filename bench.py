@@ -507,7 +507,10 @@ def main() -> int:
     }
 
     # ---- prefix prefill (M = 816): MFMA-bound regime -----------------------------
-    extra = {}
+    srt = sorted(ts_ms)
+    extra = {"denoise_step_us": {"p50": round(value_us, 2),
+                                 "p90": round(srt[min(len(srt) - 1, (9 * len(srt)) // 10)] * 1e3 / denoise_steps, 2),
+                                 "min": round(srt[0] * 1e3 / denoise_steps, 2), "replays": len(srt)}}
     if not args.no_prefill:
         pl = make_layers(dev, PREFILL_SET, 816, 4, seed0=10_000)
         pg = HipGraph()
