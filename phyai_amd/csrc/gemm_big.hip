@@ -492,7 +492,10 @@ static void big_launch(BigArgs a, const GemmProblem& g, int splits, hipStream_t 
     const int bn_eff = gated ? 32 * TN : 64 * TN;
     a.n_tiles = big_ceil_div(gated ? g.N / 2 : g.N, bn_eff);
     a.m_tiles = big_ceil_div(g.M, 64 * TM);
+    // bands of 4 tile rows; a grid of up to 8 tile rows whose activation rows still fit an XCD's
+    // L2 beside the weight stream is one band, so that the weights come from HBM once
     a.band = 4;
+    if (a.m_tiles <= 8 && (int64_t)a.m_tiles * (64 * TM) * (g.K < 4096 ? g.K : 4096) <= (5 << 19)) a.band = a.m_tiles;
     if (const char* e = getenv("PHYAI_FP8_BAND")) { const int b = atoi(e); if (b >= 1 && b <= 16) a.band = b; }
     const dim3 grid(a.m_tiles * ((a.n_tiles + 7) & ~7), 1, splits);
     if (splits > 1) {
