@@ -5,38 +5,43 @@
 // 128 x 128 (TM = TN = 2; ring of four stages, or of two with two workgroups per CU) for
 // mid-sized problems.
 //
-// Why 4 x 4 blocks per wavefront.  One v_mfma_f32_32x32x64_f8f6f4 takes 64 cycles and consumes
-// two 2 KB operand blocks.  A wavefront with TM x TN blocks reads (TM + TN) blocks from LDS per
-// TM*TN MFMAs; LDS delivers 128 bytes per clock to the whole CU, so four wavefronts with 4 x 4
-// blocks ask for 64 bytes per clock, 2 x 2 blocks for 128.  The same ratio governs the bytes
-// that must come from L2: (BM + BN) * K per tile, and on this chip L2 -> CU delivery
-// (measured: about 10-13 TB/s over all CUs) is what finally bounds the kernel, not the MFMA
-// pipe.  4 x 4 blocks of 16 accumulators are 256 registers: they live in AGPRs, one
-// wavefront per SIMD, and latency is hidden inside the wavefront:
+// Why 4 x 4 blocks per wavefront for the large tile.  One v_mfma_f32_32x32x64_f8f6f4 takes 64
+// cycles and consumes two 2 KB operand blocks.  A wavefront with TM x TN blocks reads (TM + TN)
+// blocks from LDS per TM*TN MFMAs; LDS delivers 128 bytes per clock to the whole CU, so four
+// wavefronts with 4 x 4 blocks ask for 64 bytes per clock, 2 x 2 blocks for 128.  The same ratio
+// governs the bytes that must come from L2: (BM + BN) * K per tile, and L2 -> CU delivery
+// (measured: 10-13 TB/s over all CUs inside these kernels) bounds the small tiles.  4 x 4 blocks
+// of 16 accumulators are 256 registers: they live in AGPRs, one wavefront per SIMD, and latency
+// is hidden inside the wavefront:
 //
 //  * global -> LDS copies bypass the register file (global_load_lds_dwordx4): lane i of a
 //    wavefront fetches one 16-byte chunk and the hardware deposits chunk i at LDS base + 16*i.
-//    The XOR swizzle that keeps the 128-bit operand reads conflict-free is therefore applied
-//    on the global side: lane i (row i/4 of a 16-row group, slot i%4 of the 64-byte row)
-//    fetches chunk (i%4) ^ swizzle(row) of its row.
-//  * K is consumed in 64-byte slabs through a ring of four LDS stages: the copies of slab s+3
-//    are requested while slabs s and s+1 are being multiplied, one copy instruction after every
-//    second MFMA, so the wavefront never waits on the memory pipeline's issue queue with its
-//    MFMA pipe empty.  One barrier per slab, placed in the MIDDLE of slab s: it publishes slab
-//    s+1 and tells everyone that the stage about to be refilled is no longer read.  All
-//    wavefronts reach it at about the same time, with MFMAs queued.
-//  * the operand blocks that open slab s+1 are read from LDS during the last row group of
-//    slab s into a second register set, and inside a slab the A block of the next row group is
-//    read before the current group's MFMAs are issued, so ds_read latency overlaps MFMA time.
+//    An LDS row is 128 bytes of K - one L2 line per row per request; the XOR swizzle that keeps
+//    the 128-bit operand reads conflict-free is therefore applied on the global side: lane i
+//    (row i/8 of an 8-row group, slot i%8 of the row) fetches chunk (i%8) ^ swizzle(row).
+//  * K is consumed in 128-byte stage-loads through a ring of DEPTH LDS stages: the copies of
+//    load d+DEPTH are requested while loads d and d+1 are being multiplied, one or two copy
+//    instructions per MFMA, so the wavefront never waits on the memory pipeline's issue queue
+//    with its MFMA pipe empty.  One barrier per stage-load, placed in its second K half: it
+//    publishes the next stage and tells everyone that the stage about to be refilled is no
+//    longer read.  All wavefronts reach it at about the same time, with MFMAs queued.
+//  * the operand blocks that open the next K half are read from LDS during the later row groups
+//    of the current one into a second register set, and inside a half the A blocks of the later
+//    row groups are read before the first group's MFMAs are issued, so ds_read latency overlaps
+//    MFMA time.
 //  * epilogue: the weight block is the MFMA's first operand, which gives a lane runs of four
 //    consecutive output columns of one token row; each wavefront stages its bf16 tile in its own
 //    slice of the (now idle) LDS and writes it out row-wise, 16 bytes per lane, whole row
 //    segments per instruction.
 //
+// The smaller tiles (192 x 128, and 128 x 128 with a ring of two) keep within the register and
+// LDS budget of two workgroups per CU, so that one workgroup's prologue and epilogue run under
+// the other's MFMAs.
+//
 // Gated epilogues: within a wavefront's 32*TN columns the first half are gate columns and the
 // second half the matching up columns, so the pair sits in the same lane of two accumulators.
-// Requires K % 128 == 0 and K >= 512 per split (slabs are never partial, come in pairs, and
-// must fill the ring).
+// Requires K % 128 == 0 and K >= 512 per split (stage-loads are never partial and must fill the
+// ring).
 #include "fp8_device.h"
 #include "launch.h"
 #include "splitk.h"

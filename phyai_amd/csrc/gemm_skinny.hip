@@ -15,11 +15,11 @@
 //    (grid.y): a workgroup then owns 16*NT columns x 16*MB token rows.  Workgroups that
 //    share a weight tile differ only in blockIdx.y, and with a multiple of 8 tiles they land
 //    on the same XCD, so the tile comes from HBM once and from that XCD's L2 afterwards.
-//  * Every lane requests all of its bytes first - weights and quantized
-//    activations, straight from global memory into VGPRs in MFMA operand layout -
-//    together with the scales and bias the epilogue will want, and only then
-//    starts to compute.  Nothing is staged through LDS before the MFMAs, so there
-//    is no barrier between the loads and the math.
+//  * Every wavefront requests all of its bytes first - weights and quantized activations,
+//    together with the scales and bias the epilogue will want - and only then starts to
+//    compute.  The operands go global -> LDS (the wavefront's own slice, see STAGED below) ->
+//    VGPRs in MFMA operand layout; nobody else reads that slice, so there is no barrier
+//    between the loads and the math.
 //  * v_mfma_f32_16x16x128_f8f6f4: lane l supplies operand row (l % 16) and 32 of
 //    the 128 K bytes of a step.  Which 32 is free as long as both operands agree;
 //    lane group q = l / 16 takes bytes [16q, 16q+16) and [64+16q, 64+16q+16), so

@@ -351,7 +351,8 @@ int launch_gemm(const GemmProblem& g, hipStream_t st) {
     if (g.M == 0 || g.N == 0) return 0;
     // Kernel choice (measured on the expert and prefill shapes, M = 50 .. 13056):
     //   M <= 64                      weight-streaming kernel, nothing else comes close;
-    //   pipelined tile kernel        256 x 256 tiles, or at least 64 tiles of 128 x 128;
+    //   pipelined tile kernel        when big_plan finds a tile shape that fills the chip, or at
+    //                                least 64 tiles of 128 x 128;
     //   64 < M <= 512 otherwise      weight-streaming kernel again (few output columns: at
     //                                N = 1024 it wins up to M = 512, at N = 2560 up to M = 300);
     //   32 .. 63 small tiles         pipelined tile kernel after all (M > 512);
