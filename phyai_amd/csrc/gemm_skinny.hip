@@ -284,9 +284,9 @@ __global__ __launch_bounds__(SK_THREADS) void gemm_fp8_skinny_kernel(const Skinn
     float vf[4];
 #pragma unroll
     for (int r = 0; r < 4; ++r) {
-        float v = g[r] * (sa * sw4[r]) + bwf[r];
+        float v = __builtin_fmaf(g[r], sa * sw4[r], bwf[r]);   // one rounding, like the tile kernels
         if constexpr (GATED) {
-            const float up = u[r] * (sa * su4[r]) + buf[r];
+            const float up = __builtin_fmaf(u[r], sa * su4[r], buf[r]);
             v = apply_act<EPI>(round_bf16(v)) * round_bf16(up);
         } else if constexpr (EPI != EPI_NONE) {
             v = apply_act<EPI>(round_bf16(v));

@@ -226,9 +226,9 @@ __global__ __launch_bounds__(256) void gemm_fp8_tile_kernel(const TileArgs p) {
 #pragma unroll
             for (int r = 0; r < 16; ++r) {
                 const int m = m0 + wm * WM + i * 32 + 8 * (r / 4) + 4 * h + (r % 4);
-                float v = acc[i][j][r] * (sa[i][r] * sg) + bg;
+                float v = __builtin_fmaf(acc[i][j][r], sa[i][r] * sg, bg);   // one rounding, like the other kernels
                 if constexpr (GATED) {
-                    const float u = acc[i][j + TN / 2][r] * (sa[i][r] * su) + bu;
+                    const float u = __builtin_fmaf(acc[i][j + TN / 2][r], sa[i][r] * su, bu);
                     v = apply_act<EPI>(round_bf16(v)) * round_bf16(u);
                 } else if constexpr (EPI != EPI_NONE) {
                     v = apply_act<EPI>(round_bf16(v));

@@ -406,6 +406,40 @@ def test_big_tile_kernel_exact_integer(dev, monkeypatch, tile):
         assert torch.equal(got.cpu(), want), f"{(M, N, K)}"
 
 
+def test_tile_variants_agree_bit_for_bit_on_random_shapes(dev, monkeypatch):
+    """Every variant of the pipelined tile kernel, and the generic tile kernel, walks K in the same
+    order with the same MFMA, so without split-K their outputs must be identical bit for bit
+    whatever the tile shape: 30 seeded shapes with ragged M, N off the tile grid, K down to the
+    smallest the ring accepts, all epilogues; one variant is also held to the oracle tolerance."""
+    ops = _ops()
+    rng = np.random.default_rng(20240607)
+    epis = [(None, 0), ("geglu_tanh", 1), ("geglu_erf", 2), ("swiglu", 3), ("gelu_tanh", 4), ("gelu", 5)]
+    for case in range(30):
+        M = int(rng.integers(65, 700))
+        N = 32 * int(rng.integers(1, 40))
+        K = 128 * int(rng.integers(4, 14))
+        epi_name, epi = epis[case % len(epis)]
+        x, wq, ws, b = _problem(M, N, K, seed=1000 + case)
+        xq, xs = ops.fp8_quant_rowwise(x.to(dev))
+        wd, sd, bd = wq.to(dev), ws.to(dev), b.to(dev)
+        outs = {}
+        for spec in ("256", "192", "128", "128/2", "generic"):
+            monkeypatch.delenv("PHYAI_FP8_BIG", raising=False)
+            monkeypatch.delenv("PHYAI_FP8_BIG_DEPTH", raising=False)
+            monkeypatch.delenv("PHYAI_FP8_TILE", raising=False)
+            if spec == "generic":
+                monkeypatch.setenv("PHYAI_FP8_TILE", "128,128,1")     # generic kernel, no split-K
+            else:
+                _force_big(monkeypatch, spec)
+            outs[spec] = ops.fp8_gemm(xq, xs, wd, sd, bd, epilogue=epi_name)
+        torch.cuda.synchronize()
+        for spec, o in outs.items():
+            assert torch.equal(_as_bits(o), _as_bits(outs["256"])), \
+                f"case {case} {(M, N, K, epi_name)}: {spec} differs from 256 in {int((_as_bits(o) != _as_bits(outs['256'])).sum())} outputs"
+        want = ref.epilogue(ref.gemm_f32(*ref.quant_rowwise(x), wq, ws, b), epi).float()
+        assert_close_to_ref(outs["192"], want, f"case {case} {(M, N, K, epi_name)}")
+
+
 @pytest.mark.parametrize("tile", ["128", "256"])
 def test_big_tile_kernel_split_k(dev, monkeypatch, tile):
     """Both tile sizes with the K range split over two and four workgroups (partials in the workspace)."""
