@@ -328,8 +328,10 @@ SkinnyPlan skinny_plan(int M, int N, int K, int epilogue) {
     const int per_tile = gated ? 8 : 16;
     SkinnyPlan pl;
     const int blocks = sk_ceil_div(M, 16);  // 16-row token blocks in all
-    // two weight tiles per workgroup once that still leaves a workgroup for every CU
-    pl.nt = sk_ceil_div(cols, 2 * per_tile) >= 256 ? 2 : 1;
+    // two weight tiles per workgroup once that still leaves a workgroup for every CU - except for a
+    // single token block, where the narrow tile's smaller staging lets two workgroups share a CU
+    // and overlap each other's phases (1 x 12288 x 2048: 8.6 -> 7.8 us)
+    pl.nt = (sk_ceil_div(cols, 2 * per_tile) >= 256 && blocks > 1) ? 2 : 1;
     pl.tiles = sk_ceil_div(cols, per_tile * pl.nt);
     if (blocks <= 4) {
         // split M while there are fewer workgroups than CUs
