@@ -453,6 +453,8 @@ def main() -> int:
                          "meant to run under `rocprofv3 --pmc FETCH_SIZE` / `--pmc WRITE_SIZE`")
     ap.add_argument("--probe-prefill", action="store_true",
                     help="the same for the prefill GEMM shapes (M = 816, 4 weight sets), for the MFMA / LDS counters")
+    ap.add_argument("--probe-m", type=int, default=816,
+                    help="token rows of --probe-prefill (816 x batch for the batched-serving shapes)")
     args = ap.parse_args()
     if args.gpus != 1 or int(os.environ.get("WORLD_SIZE", "1")) != 1:
         print("bench.py: this path is built and measured on ONE GPU (TP=1, no collectives); "
@@ -469,7 +471,7 @@ def main() -> int:
     M, n_layers, denoise_steps = 50, 18, 10
 
     if args.probe_prefill:
-        probe(dev, make_layers(dev, PREFILL_SET, 816, 4, seed0=10_000), 816, PREFILL_SET)
+        probe(dev, make_layers(dev, PREFILL_SET, args.probe_m, 4, seed0=10_000), args.probe_m, PREFILL_SET)
         return 0
 
     layers = make_layers(dev, EXPERT_SET, M, n_layers)
