@@ -446,6 +446,12 @@ static int big_tiles(int M, int N, int epilogue, int bm, int bn) {
 // partial sums then make a round trip through memory.
 static int big_tile_cols(int tile) { return tile == 256 ? 256 : 128; }
 
+// Fraction of the tile slots that hold a tile, over all rounds of `slots` concurrent tiles.
+static double big_fill(int tiles, int slots) {
+    const int rounds = big_ceil_div(tiles, slots);
+    return rounds > 0 ? (double)tiles / ((double)rounds * slots) : 1.0;
+}
+
 BigPlan big_plan(int M, int N, int K, int epilogue) {
     BigPlan pl = {0, 1, 0, 0};
     if (K % 128 != 0 || K < 512) return pl;   // slabs come in pairs and must fill the ring
@@ -457,9 +463,13 @@ BigPlan big_plan(int M, int N, int K, int epilogue) {
     // 256 x 256 tiles need the fewest bytes from L2 per flop but run one workgroup per CU, so a
     // tile's prologue and epilogue leave the MFMA pipe idle; 192 x 128 tiles fit twice and overlap
     // them.  The small tile wins once there are enough of them and while K is short enough for
-    // prologue and epilogue to matter (measured: 4-18 % up to K = 8192), unless M pads worse.
+    // prologue and epilogue to matter (measured: 4-18 % up to K = 8192), unless M pads worse or
+    // its last round of 512 tiles would be much emptier than the large tile's last round of 256
+    // (6528 x 2048 x 2048: 544 small tiles take 42 us, 208 large ones 37.5 us).
     else if (K <= 8192 && big_tiles(M, N, epilogue, 192, 128) >= 400 &&
-             big_ceil_div(M, 192) * 192 <= big_ceil_div(M, 256) * 256) pl.tile = 192;
+             big_ceil_div(M, 192) * 192 <= big_ceil_div(M, 256) * 256 &&
+             big_fill(big_tiles(M, N, epilogue, 192, 128), 512) >= big_fill(big_tiles(M, N, epilogue, 256, 256), 256) - 0.15)
+        pl.tile = 192;
     else if (big_tiles(M, N, epilogue, 256, 256) >= 200) pl.tile = 256;
     else if (big_tiles(M, N, epilogue, 128, 128) >= 32) pl.tile = 128;   // fewer: the weight-streaming kernel wins
     else return pl;
