@@ -67,6 +67,7 @@ struct BigArgs {
     int* __restrict__ counters;
     int m_tiles, n_tiles;            // tile grid; the launch is 1-D over it (see big_tile_of)
     int band;                        // tile rows per band of that order
+    int by_rows;                     // the order with the roles of tile rows and columns exchanged
     ResidualArgs res;
 };
 
@@ -132,8 +133,14 @@ void gemm_fp8_big_kernel(const BigArgs p) {
     const int wm = wave >> 1, wn = wave & 1;
     const int l32 = lane & 31, h = lane >> 5;
     const int half_n = p.N / 2;
-    const BigTile tile_id = big_tile_of(blockIdx.x, p.m_tiles, p.n_tiles, p.band);
-    if (tile_id.n >= p.n_tiles) return;              // padding of the tile order
+    BigTile tile_id;
+    if (p.by_rows) {   // an XCD takes tile rows: bands of tile columns, 8 neighbouring tile rows per 8 ids
+        const BigTile t = big_tile_of(blockIdx.x, p.n_tiles, p.m_tiles, p.band);
+        tile_id.m = t.n; tile_id.n = t.m;
+    } else {
+        tile_id = big_tile_of(blockIdx.x, p.m_tiles, p.n_tiles, p.band);
+    }
+    if (tile_id.n >= p.n_tiles || tile_id.m >= p.m_tiles) return;   // padding of the tile order
     const int m0 = tile_id.m * BM;
     const int n0 = GATED ? tile_id.n * (BN / 2) : tile_id.n * BN;
 
@@ -507,12 +514,27 @@ static void big_launch(BigArgs a, const GemmProblem& g, int splits, hipStream_t 
     const int bn_eff = gated ? 32 * TN : 64 * TN;
     a.n_tiles = big_ceil_div(gated ? g.N / 2 : g.N, bn_eff);
     a.m_tiles = big_ceil_div(g.M, 64 * TM);
+    // Which operand the XCDs share.  By default an XCD takes tile columns: its L2 then holds the
+    // weight rows of those columns once, but every XCD streams all activation rows it meets.
+    // With few tile columns and long rows of activations (816 x B tokens into a 16384 -> 2048
+    // projection) that is eight copies of the larger operand; then the roles are exchanged.
+    // Estimated bytes from HBM: the operand an XCD does not own is read once per XCD (up to 8
+    // times), the other once per band.
+    {
+        const double a_bytes = (double)g.M * g.K, b_bytes = (double)g.N * g.K;
+        const int band_c = 4, band_r = 4;
+        const double by_cols = a_bytes * (a.n_tiles < 8 ? a.n_tiles : 8) + b_bytes * big_ceil_div(a.m_tiles, band_c);
+        const double by_rows = b_bytes * (a.m_tiles < 8 ? a.m_tiles : 8) + a_bytes * big_ceil_div(a.n_tiles, band_r);
+        a.by_rows = by_rows < 0.8 * by_cols;
+        if (const char* e = getenv("PHYAI_FP8_BY_ROWS")) a.by_rows = atoi(e) != 0;
+    }
     // bands of 4 tile rows; a grid of up to 8 tile rows whose activation rows still fit an XCD's
     // L2 beside the weight stream is one band, so that the weights come from HBM once
     a.band = 4;
-    if (a.m_tiles <= 8 && (int64_t)a.m_tiles * (64 * TM) * (g.K < 4096 ? g.K : 4096) <= (5 << 19)) a.band = a.m_tiles;
+    if (!a.by_rows && a.m_tiles <= 8 && (int64_t)a.m_tiles * (64 * TM) * (g.K < 4096 ? g.K : 4096) <= (5 << 19)) a.band = a.m_tiles;
     if (const char* e = getenv("PHYAI_FP8_BAND")) { const int b = atoi(e); if (b >= 1 && b <= 16) a.band = b; }
-    const dim3 grid(a.m_tiles * ((a.n_tiles + 7) & ~7), 1, splits);
+    const int outer = a.by_rows ? a.n_tiles : a.m_tiles, inner = a.by_rows ? a.m_tiles : a.n_tiles;
+    const dim3 grid(outer * ((inner + 7) & ~7), 1, splits);
     if (splits > 1) {
         if constexpr (TM == TN && (TM == 4 || DEPTH == 4))
             hipLaunchKernelGGL((gemm_fp8_big_kernel<TM, TN, DEPTH, EPI, true>), grid, dim3(256), 0, st, a);

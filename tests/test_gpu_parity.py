@@ -423,16 +423,22 @@ def test_tile_variants_agree_bit_for_bit_on_random_shapes(dev, monkeypatch):
         xq, xs = ops.fp8_quant_rowwise(x.to(dev))
         wd, sd, bd = wq.to(dev), ws.to(dev), b.to(dev)
         outs = {}
-        for spec in ("256", "192", "128", "128/2", "generic"):
+        for spec in ("256", "192", "128", "128/2", "256/rows", "128/rows", "generic"):
             monkeypatch.delenv("PHYAI_FP8_BIG", raising=False)
             monkeypatch.delenv("PHYAI_FP8_BIG_DEPTH", raising=False)
             monkeypatch.delenv("PHYAI_FP8_TILE", raising=False)
+            monkeypatch.delenv("PHYAI_FP8_BY_ROWS", raising=False)
             if spec == "generic":
                 monkeypatch.setenv("PHYAI_FP8_TILE", "128,128,1")     # generic kernel, no split-K
+            elif spec.endswith("/rows"):                               # the tile order that gives an XCD tile rows
+                _force_big(monkeypatch, spec.split("/")[0])
+                monkeypatch.setenv("PHYAI_FP8_BY_ROWS", "1")
             else:
                 _force_big(monkeypatch, spec)
+                monkeypatch.setenv("PHYAI_FP8_BY_ROWS", "0")
             outs[spec] = ops.fp8_gemm(xq, xs, wd, sd, bd, epilogue=epi_name)
         torch.cuda.synchronize()
+        monkeypatch.delenv("PHYAI_FP8_BY_ROWS", raising=False)
         for spec, o in outs.items():
             assert torch.equal(_as_bits(o), _as_bits(outs["256"])), \
                 f"case {case} {(M, N, K, epi_name)}: {spec} differs from 256 in {int((_as_bits(o) != _as_bits(outs['256'])).sum())} outputs"
