@@ -312,12 +312,17 @@ void gemm_fp8_big_kernel(const BigArgs p) {
         // splitk_arrive opens with a barrier, after which nobody reads operands any more: a word
         // of the ring serves as its flag
         if (!splitk_arrive(p.counters, tile, S, reinterpret_cast<int*>(lds))) return;
+        // gather: as much of the fragment per round trip as the registers allow
+        constexpr int GCH = FRAG <= 64 ? FRAG : 32;
 #pragma unroll
-        for (int c = 0; c < TM * TN / 2; ++c) {
-            float frag[CHUNK];
-            splitk_gather_part<FRAG, 256, CHUNK>(p.partials, tile, S, c * CHUNK, frag);
+        for (int c = 0; c < FRAG / GCH; ++c) {
+            float frag[GCH];
+            splitk_gather_part<FRAG, 256, GCH>(p.partials, tile, S, c * GCH, frag);
 #pragma unroll
-            for (int r = 0; r < 32; ++r) acc[(2 * c) / TN][(2 * c) % TN + r / 16][r % 16] = frag[r];
+            for (int r = 0; r < GCH; ++r) {
+                const int blk = (c * GCH + r) / 16;
+                acc[blk / TN][blk % TN][r % 16] = frag[r];
+            }
         }
         splitk_reset(p.counters, tile);
     }

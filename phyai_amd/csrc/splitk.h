@@ -63,20 +63,30 @@ __device__ __forceinline__ bool splitk_arrive(int* counters, int tile, int S, in
     return *s_flag != 0;
 }
 
-// Sum of elements e0 .. e0+CHUNK-1 over the S partials of a tile, in split order.
+// Sum of elements e0 .. e0+CHUNK-1 over the S partials of a tile, in split order.  The loads of
+// two partials are in flight together: every batch of loads is a round trip to memory, and the
+// round trips, not the bytes, are what the gathering workgroup waits for.
 template <int FRAG, int THREADS, int CHUNK>
 __device__ __forceinline__ void splitk_gather_part(const float* partials, int tile, int S, int e0, float* frag) {
     const float* all = partials + (size_t)tile * S * (size_t)(FRAG * THREADS);
 #pragma unroll
     for (int e = 0; e < CHUNK; ++e) frag[e] = 0.f;
-    for (int z = 0; z < S; ++z) {
-        const float* pz = all + (size_t)z * (FRAG * THREADS);
-        float t[CHUNK];
+    for (int z = 0; z < S; z += 2) {
+        const bool pair = z + 1 < S;   // uniform over the workgroup
+        const float* p0 = all + (size_t)z * (FRAG * THREADS);
+        const float* p1 = p0 + (pair ? FRAG * THREADS : 0);
+        float t0[CHUNK], t1[CHUNK];
 #pragma unroll
-        for (int e = 0; e < CHUNK; e += 2)
-            coherent_load2(pz + (((e0 + e) / 2) * THREADS + threadIdx.x) * 2, t[e], t[e + 1]);
+        for (int e = 0; e < CHUNK; e += 2) {
+            coherent_load2(p0 + (((e0 + e) / 2) * THREADS + threadIdx.x) * 2, t0[e], t0[e + 1]);
+            coherent_load2(p1 + (((e0 + e) / 2) * THREADS + threadIdx.x) * 2, t1[e], t1[e + 1]);
+        }
 #pragma unroll
-        for (int e = 0; e < CHUNK; ++e) frag[e] += t[e];
+        for (int e = 0; e < CHUNK; ++e) frag[e] += t0[e];
+        if (pair) {
+#pragma unroll
+            for (int e = 0; e < CHUNK; ++e) frag[e] += t1[e];
+        }
     }
 }
 
