@@ -383,11 +383,37 @@ def sweep(dev):
         us = statistics.median(ts) * 1e3 / len(items)
         t_hbm = algorithmic_bytes(M, N, K, epi, with_bias) / (HBM_PEAK_GBS * 1e9) * 1e6
         t_mfma = 2.0 * M * N * K / (FP8_PEAK_TFLOPS * 1e12) * 1e6
-        rows.append({"set": set_name, "B": B, "M": M, "shape": name, "us": round(us, 2),
-                     "bound": "hbm" if t_hbm >= t_mfma else "mfma",
-                     "roofline_us": round(max(t_hbm, t_mfma), 3),
-                     "frac": round(max(t_hbm, t_mfma) / us, 4)})
-        del items, gr
+        row = {"set": set_name, "B": B, "M": M, "shape": name, "us": round(us, 2),
+               "bound": "hbm" if t_hbm >= t_mfma else "mfma",
+               "roofline_us": round(max(t_hbm, t_mfma), 3),
+               "frac": round(max(t_hbm, t_mfma) / us, 4)}
+        del gr
+        # the GEMM alone (codes ready, no activation) beside torch._scaled_mm - the call the
+        # reference makes (layers/linear/backends/torch.py:168-175), hipBLASLt underneath
+        pre = [(ops.fp8_quant_rowwise(x), wq, ws, b, torch.empty(M, N, dtype=torch.bfloat16, device=dev))
+               for x, wq, ws, b, _ in items]
+
+        def ours():
+            for (xq, xs), wq, ws, b, o in pre:
+                ops.fp8_gemm(xq, xs, wq, ws, b, out=o)
+
+        def blaslt():
+            for (xq, xs), wq, ws, b, o in pre:
+                torch._scaled_mm(xq, wq.t(), scale_a=xs, scale_b=ws.reshape(1, -1), bias=b, out_dtype=torch.bfloat16, out=o)
+
+        for key, f in (("gemm_us", ours), ("scaled_mm_us", blaslt)):
+            try:
+                f()
+                torch.cuda.synchronize()
+                gr = HipGraph()
+                gr.capture(f, {})
+                ts, _ = time_replays(gr, 10, 3)
+                row[key] = round(statistics.median(ts) * 1e3 / len(pre), 2)
+                del gr
+            except Exception as e:  # noqa: BLE001 - torch._scaled_mm may not run on every image
+                row[key] = f"unavailable: {str(e)[:80]}"
+        rows.append(row)
+        del items, pre
     return rows
 
 
