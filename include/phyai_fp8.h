@@ -31,7 +31,7 @@
 extern "C" {
 #endif
 
-#define PHYAI_FP8_ABI_VERSION 2
+#define PHYAI_FP8_ABI_VERSION 3
 
 enum {
     PHYAI_FP8_OK = 0,
@@ -168,6 +168,19 @@ int phyai_fp8_adarmsnorm_quant(const void *x, int64_t ldx, const void *modulatio
                                int64_t ld_mod, int64_t mod_rows, int64_t M, int64_t D,
                                float eps, void *out, int64_t ldo, void *gate_out,
                                int64_t ld_gate, void *xq, float *x_scale, void *stream);
+
+/*
+ * Which kernel phyai_fp8_gemm would launch for a problem with 16-byte aligned operands and a
+ * dense output (ldo = output width): a short text such as
+ *   "small-m nt=2 mb=4 kpw=1 rounds=1"      weight-streaming kernel
+ *   "tile 192x128 depth=2 splits=1 tiles=2304"   pipelined tile kernel
+ *   "generic 128x128 splits=2"               fallback tile kernel
+ * written to buf (at most n bytes, always terminated).  Host only: nothing is launched, no GPU is
+ * needed.  Returns the length of the text, or a negative status for bad arguments.  The
+ * reference has no counterpart (its dispatcher only picks between whole backends,
+ * layers/linear/dispatch.py:28-95); this is for logs and for tests of the selection rules.
+ */
+int phyai_fp8_describe_plan(int64_t M, int64_t N, int64_t K, int epilogue, char *buf, size_t n);
 
 /*
  * Test hook: run the device fp32 -> e4m3fn cast used by the quantizers over n

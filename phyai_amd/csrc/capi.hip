@@ -291,6 +291,19 @@ int phyai_fp8_adarmsnorm_quant(const void* x, int64_t ldx, const void* modulatio
     return check_launch("phyai_fp8_adarmsnorm_quant");
 }
 
+int phyai_fp8_describe_plan(int64_t M, int64_t N, int64_t K, int epilogue, char* buf, size_t n) {
+    if (!buf || n == 0) return fail(PHYAI_FP8_EINVAL, "phyai_fp8_describe_plan: no buffer");
+    buf[0] = 0;
+    if (M < 0 || N <= 0 || K <= 0 || M >= kMaxElems || N >= kMaxElems || K >= kMaxElems)
+        return fail(PHYAI_FP8_EINVAL, "phyai_fp8_describe_plan: bad shape M=%lld N=%lld K=%lld", (long long)M, (long long)N, (long long)K);
+    if (int rc = check_epilogue(epilogue, N)) return rc;
+    if (K % 16 != 0 || N % 16 != 0)
+        return fail(PHYAI_FP8_EUNSUPPORTED, "phyai_fp8_describe_plan: K=%lld and N=%lld must be multiples of 16", (long long)K, (long long)N);
+    const int len = phyai::describe_gemm_plan((int)M, (int)N, (int)K, epilogue, buf, n);
+    buf[n - 1] = 0;
+    return len;
+}
+
 int phyai_fp8_debug_cast_e4m3(const float* v, int64_t n, void* codes, void* stream) {
     if (n < 0 || (n > 0 && (!v || !codes))) return fail(PHYAI_FP8_EINVAL, "phyai_fp8_debug_cast_e4m3: bad arguments");
     phyai::launch_debug_cast(v, n, codes, static_cast<hipStream_t>(stream));

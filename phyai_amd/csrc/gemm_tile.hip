@@ -347,6 +347,27 @@ static int launch_epi(const TileArgs& a, const TileConfig& c, dim3 grid, hipStre
     }
 }
 
+int describe_gemm_plan(int M, int N, int K, int epilogue, char* buf, size_t n) {
+    // mirrors launch_gemm below for operands that satisfy every alignment requirement
+    const int64_t ldo = epi_is_gated(epilogue) ? N / 2 : N;
+    const bool skinny_ok = skinny_applicable(M, N, K, epilogue, ldo);
+    auto small = [&]() {
+        const SkinnyPlan pl = skinny_plan(M, N, K, epilogue);
+        return snprintf(buf, n, "small-m nt=%d mb=%d kpw=%d rounds=%d", pl.nt, pl.mb, pl.kpw, pl.rounds);
+    };
+    if (skinny_ok && M <= 64) return small();
+    if (!getenv("PHYAI_FP8_TILE")) {
+        const BigPlan bp = big_plan(M, N, K, epilogue);
+        const bool few_small_tiles = bp.tile == 128 && bp.tiles < 64 && !getenv("PHYAI_FP8_BIG");
+        if (bp.tile && ldo % 8 == 0 && !(few_small_tiles && skinny_ok))
+            return snprintf(buf, n, "tile %dx%d depth=%d splits=%d tiles=%d", bp.tile, bp.tile == 256 ? 256 : 128,
+                            bp.depth, bp.splits, bp.tiles);
+        if (skinny_ok) return small();
+    }
+    const TileConfig c = pick_config(M, N, K, epilogue);
+    return snprintf(buf, n, "generic %dx%d splits=%d", c.bm, c.bn, c.splits);
+}
+
 int launch_gemm(const GemmProblem& g, hipStream_t st) {
     if (g.M == 0 || g.N == 0) return 0;
     // Kernel choice (measured on the expert and prefill shapes, M = 50 .. 13056):

@@ -101,4 +101,7 @@ BigPlan big_plan(int M, int N, int K, int epilogue);
 size_t big_partial_bytes(int M, int N, int epilogue, const BigPlan& pl);
 int launch_gemm_big(const GemmProblem& p, const BigPlan& pl, hipStream_t st);
 
+// Text form of launch_gemm's choice for aligned operands and a dense output; returns its length.
+int describe_gemm_plan(int M, int N, int K, int epilogue, char* buf, size_t n);
+
 }  // namespace phyai

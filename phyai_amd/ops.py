@@ -76,6 +76,17 @@ def workspace_bytes(M: int, N: int, K: int, epilogue=EPI_NONE) -> int:
     return int(_lib.load().phyai_fp8_linear_workspace_bytes(M, N, K, _epi("workspace_bytes", epilogue)))
 
 
+def describe_plan(M: int, N: int, K: int, epilogue=EPI_NONE) -> str:
+    """Which kernel the GEMM entry point would launch for this problem (host only, no GPU needed)."""
+    import ctypes
+
+    buf = ctypes.create_string_buffer(128)
+    rc = _lib.load().phyai_fp8_describe_plan(M, N, K, _epi("describe_plan", epilogue), buf, len(buf))
+    if rc < 0:
+        raise _err("describe_plan", _lib.load().phyai_fp8_last_error().decode())
+    return buf.value.decode()
+
+
 def reserve_workspace(nbytes: int, device: torch.device | None = None) -> torch.Tensor:
     """Make sure the current stream's workspace on ``device`` holds ``nbytes``."""
     dev = torch.device("cuda", torch.cuda.current_device()) if device is None else torch.device(device)

@@ -57,6 +57,44 @@ def test_workspace_query_and_argument_validation_without_gpu():
     assert b"workspace" in lib.phyai_fp8_last_error()
 
 
+def test_kernel_selection_for_the_benchmark_shapes(monkeypatch):
+    """The dispatcher's choice, read back as text (host only).  The rules behind these cases were
+    measured on the GPU: weight streaming up to 64 token rows; 256 x 256 tiles when they fill the
+    chip and K is long or the last round of smaller tiles would be emptier; 192 x 128 tiles (two
+    workgroups per CU) for K <= 8192 with enough tiles; 128 x 128 tiles with a ring of two from 400
+    tiles up, split along K for K >= 8192 with few tiles; weight streaming again below 64 small
+    tiles up to 512 rows."""
+    from phyai_amd import ops
+
+    for var in ("PHYAI_FP8_BIG", "PHYAI_FP8_BIG_DEPTH", "PHYAI_FP8_BIG_SPLITS", "PHYAI_FP8_TILE",
+                "PHYAI_FP8_SKINNY_PLAN", "PHYAI_FP8_SKINNY_MAXM"):
+        monkeypatch.delenv(var, raising=False)
+    d = ops.describe_plan
+    # action expert, M = 50
+    assert d(50, 2560, 1024) == "small-m nt=1 mb=4 kpw=1 rounds=1"
+    assert d(50, 1024, 2048) == "small-m nt=1 mb=1 kpw=2 rounds=1"
+    assert d(50, 8192, 1024, "geglu_tanh") == "small-m nt=2 mb=4 kpw=1 rounds=1"
+    assert d(50, 1024, 4096) == "small-m nt=1 mb=1 kpw=4 rounds=1"
+    assert d(1, 12288, 2048).startswith("small-m nt=1 mb=1")
+    # prefix prefill, M = 816
+    assert d(816, 2560, 2048) == "tile 128x128 depth=4 splits=1 tiles=140"
+    assert d(816, 2048, 2048) == "tile 128x128 depth=4 splits=1 tiles=112"
+    assert d(816, 32768, 2048, "geglu_tanh") == "tile 256x256 depth=2 splits=1 tiles=512"
+    assert d(816, 2048, 16384) == "tile 128x128 depth=4 splits=2 tiles=112"
+    # batched serving and the DiT block
+    assert d(1632, 32768, 2048, "geglu_tanh") == "tile 192x128 depth=2 splits=1 tiles=2304"
+    assert d(4800, 8192, 2048, "gelu") == "tile 192x128 depth=2 splits=1 tiles=1600"
+    assert d(6528, 2048, 2048) == "tile 256x256 depth=2 splits=1 tiles=208"
+    assert d(6528, 2048, 16384) == "tile 256x256 depth=2 splits=1 tiles=208"
+    assert d(800, 8192, 1024, "geglu_tanh") == "tile 128x128 depth=2 splits=1 tiles=448"
+    assert d(200, 1024, 4096).startswith("small-m ")           # 16 small tiles: weight streaming wins
+    assert d(800, 1024, 4096) == "tile 128x128 depth=4 splits=1 tiles=56"
+    # what the fast kernels refuse goes to the generic one
+    assert d(300, 384, 272).startswith("generic ")
+    with pytest.raises(RuntimeError, match="multiples of 16"):
+        d(50, 1000, 1024)
+
+
 def test_missing_library_fails_loudly(monkeypatch, tmp_path):
     from phyai_amd import _lib
 
