@@ -178,6 +178,7 @@ def test_init_prefers_hip_kernel_for_fp8(monkeypatch):
     L.init()                                                            # validate passes on a CPU-only host
 
 
+@pytest.mark.skipif(torch.cuda.is_available(), reason="describes a machine without a GPU")
 def test_fp8_on_unsupported_device_raises_lazily():
     L.init()                                                            # sm == 0 here
     layer = L.ReplicatedLinear(32, 16, bias=False, params_dtype=torch.bfloat16,
