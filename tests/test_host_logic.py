@@ -294,6 +294,8 @@ def test_dense_mlp_bf16_paths_match_torch():
     L.init()
     torch.manual_seed(1)
     x = torch.randn(5, 32).bfloat16()
+    if torch.cuda.is_available():          # layers are created on the default device
+        x = x.cuda()
     for act, ref_act in (("gelu_tanh", lambda t: F.gelu(t, approximate="tanh")), ("silu", F.silu), ("gelu", F.gelu)):
         mlp = DenseMLP(32, 64, activation=act, params_dtype=torch.bfloat16)
         for p in mlp.parameters():

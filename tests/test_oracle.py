@@ -280,7 +280,18 @@ def test_golden_fixture_regenerates_identically(tmp_path):
     a, b = np.load(GOLDEN), np.load(mod.OUT)
     assert sorted(a.files) == sorted(b.files)
     for k in a.files:
-        np.testing.assert_array_equal(a[k], b[k], err_msg=k)
+        if "_out" in k:
+            # matmul outputs: the order of an fp32 sum is the CPU BLAS's business and differs
+            # between machines; inputs, codes and scales below are exact everywhere
+            x, y = a[k], b[k]
+            if x.dtype == np.uint16:                      # bf16 bit patterns
+                x = torch.from_numpy(x.copy()).view(torch.bfloat16).float().numpy()
+                y = torch.from_numpy(y.copy()).view(torch.bfloat16).float().numpy()
+                np.testing.assert_allclose(x, y, rtol=2.0 ** -7, atol=1e-6, err_msg=k)
+            else:
+                np.testing.assert_allclose(x, y, rtol=2e-5, atol=2e-6, err_msg=k)
+        else:
+            np.testing.assert_array_equal(a[k], b[k], err_msg=k)
 
 
 # ---- norm restatements (phyai-kernel triton/rms_norm.py, ada_rms_norm.py) -----------------------
