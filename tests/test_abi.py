@@ -95,6 +95,47 @@ def test_kernel_selection_for_the_benchmark_shapes(monkeypatch):
         d(50, 1000, 1024)
 
 
+C_CLIENT = r"""
+#include <stdio.h>
+#include <string.h>
+#include "phyai_fp8.h"
+int main(void) {
+    char buf[96];
+    if (phyai_fp8_abi_version() != PHYAI_FP8_ABI_VERSION) return 1;
+    if (phyai_fp8_linear_workspace_bytes(50, 1024, 4096, PHYAI_FP8_EPI_NONE) < PHYAI_FP8_WORKSPACE_HEADER_BYTES) return 2;
+    if (phyai_fp8_describe_plan(50, 8192, 1024, PHYAI_FP8_EPI_GEGLU_TANH, buf, sizeof buf) <= 0) return 3;
+    if (strncmp(buf, "small-m", 7) != 0) return 4;
+    if (phyai_fp8_gemm(NULL, NULL, 0, NULL, NULL, NULL, NULL, 64, 4, 64, 60, 0, NULL, 0, NULL) != PHYAI_FP8_EUNSUPPORTED) return 5;
+    if (strstr(phyai_fp8_last_error(), "multiples of 16") == NULL) return 6;
+    puts(buf);
+    return 0;
+}
+"""
+
+
+def test_header_and_library_serve_a_plain_c_client(tmp_path):
+    """The header compiles as C99 and a C program linked against the library can call it (host-side
+    entry points only: nothing here needs a GPU)."""
+    import shutil
+    import subprocess
+
+    from phyai_amd import _lib
+
+    _lib.load()
+    gcc = shutil.which("gcc")
+    if gcc is None:
+        pytest.skip("no C compiler")
+    src = tmp_path / "client.c"
+    src.write_text(C_CLIENT)
+    exe = tmp_path / "client"
+    libdir = os.path.dirname(_lib.LIB_PATH)
+    subprocess.check_call([gcc, "-std=c99", "-Wall", "-Werror", "-pedantic", "-I", os.path.join(ROOT, "include"),
+                           str(src), "-o", str(exe), "-L", libdir, "-lphyai_fp8", f"-Wl,-rpath,{libdir}"])
+    out = subprocess.run([str(exe)], capture_output=True, text=True, timeout=60)
+    assert out.returncode == 0, (out.returncode, out.stdout, out.stderr)
+    assert out.stdout.startswith("small-m nt=2 mb=4")
+
+
 def test_missing_library_fails_loudly(monkeypatch, tmp_path):
     from phyai_amd import _lib
 
