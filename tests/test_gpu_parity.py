@@ -510,6 +510,33 @@ def _as_bits(t):
     return t.contiguous().view(torch.int16)
 
 
+def test_two_streams_run_split_k_linears_concurrently(dev, monkeypatch):
+    """Each (device, stream) pair has its own workspace (split-K counters and partials, code
+    staging), so linears issued on two streams at once must give the serial results bit for bit."""
+    ops = _ops()
+    monkeypatch.setenv("PHYAI_FP8_BIG", "128")
+    monkeypatch.setenv("PHYAI_FP8_BIG_SPLITS", "4")
+    probs = []
+    for i in range(2):
+        x, wq, ws, b = _problem(300 + 20 * i, 384, 4096, seed=900 + i)
+        probs.append((x.to(dev), wq.to(dev), ws.to(dev), b.to(dev)))
+    serial = [ops.fp8_linear(*p) for p in probs]
+    torch.cuda.synchronize()
+    streams = [torch.cuda.Stream(), torch.cuda.Stream()]
+    outs = [[], []]
+    for rep in range(8):
+        for i, st in enumerate(streams):
+            st.wait_stream(torch.cuda.current_stream())
+            with torch.cuda.stream(st):
+                outs[i].append(ops.fp8_linear(*probs[i]))
+    torch.cuda.synchronize()
+    for i in range(2):
+        for o in outs[i]:
+            assert torch.equal(_as_bits(o), _as_bits(serial[i]))
+    keys = {k for k in ops._workspaces}
+    assert len({s.cuda_stream for s in streams} & {k[1] for k in keys}) == 2, "one workspace per stream"
+
+
 def test_quant_rowwise_exhaustive_all_values_all_scales(dev):
     """Every finite bf16 value against every possible row maximum (32 640 of them, hence every
     possible scale): 2.1e9 quotients.  The expected codes are the reference's own expression
