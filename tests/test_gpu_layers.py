@@ -223,3 +223,31 @@ def test_capture_without_warmup_on_a_fresh_stream(L, dev):
         graph.replay()
         torch.cuda.synchronize()
         assert torch.equal(out, eager)
+
+
+def test_graph_replays_of_the_split_k_tile_kernel(L, dev):
+    """The prefill down projection (816 x 2048 x 16384) runs the pipelined tile kernel with K split
+    in two; its arrival counters must be back at zero after every replay, so replays - with eager
+    calls of the same op in between - all equal the eager result."""
+    from phyai_amd import ops
+
+    assert ops.describe_plan(816, 2048, 16384) == "tile 128x128 depth=4 splits=2 tiles=112"
+    x = seeded((816, 16384), 50).to(dev)
+    wq, ws = ops.fp8_weight_quant(seeded((2048, 16384), 51, 0.02).to(dev))
+    eager = ops.fp8_linear(x, wq, ws)
+    torch.cuda.synchronize()
+    side = torch.cuda.Stream()
+    side.wait_stream(torch.cuda.current_stream())
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.stream(side):
+        ops.fp8_linear(x, wq, ws)                           # creates that stream's workspace
+        with torch.cuda.graph(graph, stream=side):
+            out = ops.fp8_linear(x, wq, ws)
+    for _ in range(4):
+        graph.replay()
+        torch.cuda.synchronize()
+        assert torch.equal(out, eager)
+        again = ops.fp8_linear(x, wq, ws)                   # eager work between the replays
+        torch.cuda.synchronize()
+        assert torch.equal(again, eager)
+
