@@ -73,8 +73,20 @@ __device__ __forceinline__ v8i join(v4i lo, v4i hi) {
 // phase of this kernel is bound by exactly that rate (every workgroup needs its weight tiles
 // AND all of the activation codes of its token rows).  Nobody but the wavefront itself reads
 // what it staged, so there is still no barrier before the math: copies, s_waitcnt, ds_read.
+//
+// Kernel arguments are plain scalars, ordered so that what the first instructions need (operand
+// pointers, sizes) sits in the first 16 dwords: the library is built with kernel-argument
+// preloading, which delivers those in SGPRs at wavefront start instead of through a scalar load
+// from memory at the head of every launch.  They are gathered into a SkinnyArgs right away.
 template <int MB, int NT, int KPW, int EPI, bool STAGED>
-__global__ __launch_bounds__(SK_THREADS) void gemm_fp8_skinny_kernel(const SkinnyArgs p) {
+__global__ __launch_bounds__(SK_THREADS) void gemm_fp8_skinny_kernel(
+    const uint8_t* __restrict__ a_w, const uint8_t* __restrict__ a_xq, int a_K, int a_M, int a_N, int a_rounds,
+    const float* __restrict__ a_x_scale, const float* __restrict__ a_w_scale, const uint16_t* __restrict__ a_bias,
+    uint16_t* __restrict__ a_out, int64_t a_ldo, int a_x_scale_scalar, const ResidualArgs a_res) {
+    SkinnyArgs p;
+    p.xq = a_xq; p.w = a_w; p.x_scale = a_x_scale; p.w_scale = a_w_scale; p.bias = a_bias; p.out = a_out;
+    p.ldo = a_ldo; p.M = a_M; p.N = a_N; p.K = a_K; p.x_scale_scalar = a_x_scale_scalar; p.rounds = a_rounds;
+    p.res = a_res;
     constexpr bool GATED = epi_is_gated(EPI);
     constexpr int COLS_PER_TILE = GATED ? 8 : 16;  // output columns per 16-row weight tile
     constexpr int BLOCKS = NT + MB;                // 16-row operand blocks (2 KB each) per K step
@@ -368,11 +380,15 @@ static void sk_launch_one(const SkinnyArgs& a, const dim3& grid, hipStream_t st)
     static const bool want = []() { const char* e = getenv("PHYAI_FP8_SKINNY_STAGED"); return !(e && atoi(e) == 0); }();
     if constexpr (fits) {
         if (want && a.K * (int64_t)(a.N > a.M ? a.N : a.M) < ((int64_t)1 << 32)) {
-            hipLaunchKernelGGL((gemm_fp8_skinny_kernel<MB, NT, KPW, EPI, true>), grid, dim3(SK_THREADS), 0, st, a);
+            hipLaunchKernelGGL((gemm_fp8_skinny_kernel<MB, NT, KPW, EPI, true>), grid, dim3(SK_THREADS), 0, st,
+                               a.w, a.xq, a.K, a.M, a.N, a.rounds, a.x_scale, a.w_scale, a.bias, a.out, a.ldo,
+                               a.x_scale_scalar, a.res);
             return;
         }
     }
-    hipLaunchKernelGGL((gemm_fp8_skinny_kernel<MB, NT, KPW, EPI, false>), grid, dim3(SK_THREADS), 0, st, a);
+    hipLaunchKernelGGL((gemm_fp8_skinny_kernel<MB, NT, KPW, EPI, false>), grid, dim3(SK_THREADS), 0, st,
+                       a.w, a.xq, a.K, a.M, a.N, a.rounds, a.x_scale, a.w_scale, a.bias, a.out, a.ldo,
+                       a.x_scale_scalar, a.res);
 }
 
 template <int MB, int NT, int EPI>
