@@ -116,7 +116,18 @@ __device__ __forceinline__ v8i big_frag(const uint8_t* buf, int row, int h, int 
 // keeps the MFMA pipe busy.
 template <int TM, int TN, int DEPTH, int EPI, bool SPLIT>
 __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu((DEPTH == 2 && TM < 4) ? 2 : 1)))
-void gemm_fp8_big_kernel(const BigArgs p) {
+void gemm_fp8_big_kernel(
+    const uint8_t* __restrict__ a_a, const uint8_t* __restrict__ a_b, int a_K, int a_M, int a_N, int a_m_tiles,
+    int a_n_tiles, int a_band, int a_by_rows, int a_k_per_split, const float* __restrict__ a_a_scale,
+    const float* __restrict__ a_b_scale, const uint16_t* __restrict__ a_bias, uint16_t* __restrict__ a_out,
+    int64_t a_ldo, int a_a_scale_scalar, float* __restrict__ a_partials, int* __restrict__ a_counters,
+    const ResidualArgs a_res) {
+    // scalar arguments, what the prologue needs first (the first 16 dwords are preloaded into SGPRs)
+    BigArgs p;
+    p.a = a_a; p.b = a_b; p.a_scale = a_a_scale; p.b_scale = a_b_scale; p.bias = a_bias; p.out = a_out;
+    p.ldo = a_ldo; p.M = a_M; p.N = a_N; p.K = a_K; p.a_scale_scalar = a_a_scale_scalar;
+    p.k_per_split = a_k_per_split; p.partials = a_partials; p.counters = a_counters;
+    p.m_tiles = a_m_tiles; p.n_tiles = a_n_tiles; p.band = a_band; p.by_rows = a_by_rows; p.res = a_res;
     constexpr bool GATED = epi_is_gated(EPI);
     constexpr int BM = 64 * TM, BN = 64 * TN;        // workgroup tile
     constexpr int WM = 32 * TM, WN = 32 * TN;        // wavefront tile
@@ -540,12 +551,15 @@ static void big_launch(BigArgs a, const GemmProblem& g, int splits, hipStream_t 
     if (const char* e = getenv("PHYAI_FP8_BAND")) { const int b = atoi(e); if (b >= 1 && b <= 16) a.band = b; }
     const int outer = a.by_rows ? a.n_tiles : a.m_tiles, inner = a.by_rows ? a.m_tiles : a.n_tiles;
     const dim3 grid(outer * ((inner + 7) & ~7), 1, splits);
+#define PHYAI_BIG_ARGS a.a, a.b, a.K, a.M, a.N, a.m_tiles, a.n_tiles, a.band, a.by_rows, a.k_per_split, a.a_scale, \
+                       a.b_scale, a.bias, a.out, a.ldo, a.a_scale_scalar, a.partials, a.counters, a.res
     if (splits > 1) {
         if constexpr (TM == TN && (TM == 4 || DEPTH == 4))
-            hipLaunchKernelGGL((gemm_fp8_big_kernel<TM, TN, DEPTH, EPI, true>), grid, dim3(256), 0, st, a);
+            hipLaunchKernelGGL((gemm_fp8_big_kernel<TM, TN, DEPTH, EPI, true>), grid, dim3(256), 0, st, PHYAI_BIG_ARGS);
     } else {
-        hipLaunchKernelGGL((gemm_fp8_big_kernel<TM, TN, DEPTH, EPI, false>), grid, dim3(256), 0, st, a);
+        hipLaunchKernelGGL((gemm_fp8_big_kernel<TM, TN, DEPTH, EPI, false>), grid, dim3(256), 0, st, PHYAI_BIG_ARGS);
     }
+#undef PHYAI_BIG_ARGS
 }
 
 template <int TM, int TN, int DEPTH>

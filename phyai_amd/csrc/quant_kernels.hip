@@ -254,7 +254,16 @@ __device__ __forceinline__ void unpack8(uint4 q, float* f) {
 // bf16 - the tensor the reference's norm kernel would have written - and, on those bf16 values,
 // the per-token quantizer (row absmax, scale, codes) of quant_rows_reg_kernel.
 template <int THREADS, int CHUNKS, bool ADAPTIVE>
-__global__ __launch_bounds__(THREADS) void norm_quant_kernel(const NormQuantArgs p) {
+__global__ __launch_bounds__(THREADS) void norm_quant_kernel(
+    const uint16_t* __restrict__ a_x, int64_t a_ldx, int a_D, int a_group, const uint16_t* __restrict__ a_mod,
+    int64_t a_ld_mod, const uint16_t* __restrict__ a_weight, float a_eps, int a_gemma, uint8_t* __restrict__ a_xq,
+    float* __restrict__ a_scale, uint16_t* __restrict__ a_out, int64_t a_ldo, uint16_t* __restrict__ a_gate,
+    int64_t a_ld_gate) {
+    // scalar arguments in the order the kernel needs them (the first 16 dwords are preloaded)
+    NormQuantArgs p;
+    p.x = a_x; p.ldx = a_ldx; p.D = a_D; p.eps = a_eps; p.weight = a_weight; p.gemma = a_gemma; p.mod = a_mod;
+    p.ld_mod = a_ld_mod; p.group = a_group; p.out = a_out; p.ldo = a_ldo; p.gate = a_gate; p.ld_gate = a_ld_gate;
+    p.xq = a_xq; p.scale = a_scale;
     __shared__ float ssum[THREADS / kWave];
     __shared__ uint32_t smax[THREADS / kWave];
     const int64_t row = blockIdx.x;
@@ -322,7 +331,16 @@ __global__ __launch_bounds__(THREADS) void norm_quant_kernel(const NormQuantArgs
 // Rows too long for registers (D > 8192, the reference's two-pass kernels): the row is read again
 // for every pass - sum of squares, then the bf16 result and its absmax, then the codes.
 template <bool ADAPTIVE>
-__global__ __launch_bounds__(256) void norm_quant_loop_kernel(const NormQuantArgs p) {
+__global__ __launch_bounds__(256) void norm_quant_loop_kernel(
+    const uint16_t* __restrict__ a_x, int64_t a_ldx, int a_D, int a_group, const uint16_t* __restrict__ a_mod,
+    int64_t a_ld_mod, const uint16_t* __restrict__ a_weight, float a_eps, int a_gemma, uint8_t* __restrict__ a_xq,
+    float* __restrict__ a_scale, uint16_t* __restrict__ a_out, int64_t a_ldo, uint16_t* __restrict__ a_gate,
+    int64_t a_ld_gate) {
+    // scalar arguments in the order the kernel needs them (the first 16 dwords are preloaded)
+    NormQuantArgs p;
+    p.x = a_x; p.ldx = a_ldx; p.D = a_D; p.eps = a_eps; p.weight = a_weight; p.gemma = a_gemma; p.mod = a_mod;
+    p.ld_mod = a_ld_mod; p.group = a_group; p.out = a_out; p.ldo = a_ldo; p.gate = a_gate; p.ld_gate = a_ld_gate;
+    p.xq = a_xq; p.scale = a_scale;
     __shared__ float ssum[256 / kWave];
     __shared__ uint32_t smax[256 / kWave];
     const int64_t row = blockIdx.x;
@@ -383,14 +401,16 @@ __global__ __launch_bounds__(256) void norm_quant_loop_kernel(const NormQuantArg
 template <bool ADAPTIVE>
 static int launch_norm_quant_t(const NormQuantArgs& a, int64_t M, hipStream_t st) {
     const dim3 grid((unsigned)M);
-#define PHYAI_NQ(T, C) hipLaunchKernelGGL((norm_quant_kernel<T, C, ADAPTIVE>), grid, dim3(T), 0, st, a)
+#define PHYAI_NQ_ARGS a.x, a.ldx, a.D, a.group, a.mod, a.ld_mod, a.weight, a.eps, a.gemma, a.xq, a.scale, a.out, a.ldo, a.gate, a.ld_gate
+#define PHYAI_NQ(T, C) hipLaunchKernelGGL((norm_quant_kernel<T, C, ADAPTIVE>), grid, dim3(T), 0, st, PHYAI_NQ_ARGS)
     if (a.D <= 512) PHYAI_NQ(64, 1);
     else if (a.D <= 1024) PHYAI_NQ(128, 1);
     else if (a.D <= 2048) PHYAI_NQ(256, 1);
     else if (a.D <= 4096) PHYAI_NQ(256, 2);
     else if (a.D <= 8192) PHYAI_NQ(256, 4);
-    else hipLaunchKernelGGL((norm_quant_loop_kernel<ADAPTIVE>), grid, dim3(256), 0, st, a);
+    else hipLaunchKernelGGL((norm_quant_loop_kernel<ADAPTIVE>), grid, dim3(256), 0, st, PHYAI_NQ_ARGS);
 #undef PHYAI_NQ
+#undef PHYAI_NQ_ARGS
     return 0;
 }
 
