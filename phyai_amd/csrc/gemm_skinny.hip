@@ -80,12 +80,15 @@ __device__ __forceinline__ v8i join(v4i lo, v4i hi) {
 // from memory at the head of every launch.  They are gathered into a SkinnyArgs right away.
 template <int MB, int NT, int KPW, int EPI, bool STAGED>
 __global__ __launch_bounds__(SK_THREADS) void gemm_fp8_skinny_kernel(
-    const uint8_t* __restrict__ a_w, const uint8_t* __restrict__ a_xq, int a_K, int a_M, int a_N, int a_rounds,
-    const float* __restrict__ a_x_scale, const float* __restrict__ a_w_scale, const uint16_t* __restrict__ a_bias,
-    uint16_t* __restrict__ a_out, int64_t a_ldo, int a_x_scale_scalar, const ResidualArgs a_res) {
+    const uint8_t* __restrict__ a_w, const uint8_t* __restrict__ a_xq, const float* __restrict__ a_x_scale,
+    const float* __restrict__ a_w_scale, const uint16_t* __restrict__ a_bias, int a_K, int a_N, int a_m_flags,
+    uint16_t* __restrict__ a_out, int64_t a_ldo, const ResidualArgs a_res) {
+    // 13 preloaded dwords: everything the operand requests and the early epilogue loads need.
+    // a_m_flags = M | x_scale_is_scalar << 30; the rounds follow from K.
     SkinnyArgs p;
     p.xq = a_xq; p.w = a_w; p.x_scale = a_x_scale; p.w_scale = a_w_scale; p.bias = a_bias; p.out = a_out;
-    p.ldo = a_ldo; p.M = a_M; p.N = a_N; p.K = a_K; p.x_scale_scalar = a_x_scale_scalar; p.rounds = a_rounds;
+    p.ldo = a_ldo; p.M = a_m_flags & 0x3FFFFFFF; p.N = a_N; p.K = a_K; p.x_scale_scalar = (a_m_flags >> 30) & 1;
+    p.rounds = (((a_K >> 7) + SK_WAVES - 1) / SK_WAVES + KPW - 1) / KPW;
     p.res = a_res;
     constexpr bool GATED = epi_is_gated(EPI);
     constexpr int COLS_PER_TILE = GATED ? 8 : 16;  // output columns per 16-row weight tile
@@ -130,13 +133,17 @@ __global__ __launch_bounds__(SK_THREADS) void gemm_fp8_skinny_kernel(
         if constexpr (GATED) bu2 = *reinterpret_cast<const uint2*>(p.bias + half_n + e_n_safe);
     }
     const float sa = p.x_scale[(p.x_scale_scalar || !e_live) ? 0 : e_m];
-    uint2 res2 = make_uint2(0, 0), gate2 = make_uint2(0, 0);   // gated residual, requested early too
-    if constexpr (EPI == EPI_NONE) {
-        if (p.res.residual != nullptr && e_live) {
-            res2 = *reinterpret_cast<const uint2*>(p.res.residual + (int64_t)e_m * p.res.ld_res + e_n);
-            gate2 = *reinterpret_cast<const uint2*>(p.res.gate + (int64_t)(e_m / p.res.gate_group) * p.res.ld_gate + e_n);
+    // gated residual: requested once the operand requests are out (its arguments are not among
+    // the preloaded ones, and nothing before the operand requests should wait for a scalar load)
+    uint2 res2 = make_uint2(0, 0), gate2 = make_uint2(0, 0);
+    auto request_residual = [&]() {
+        if constexpr (EPI == EPI_NONE) {
+            if (p.res.residual != nullptr && e_live) {
+                res2 = *reinterpret_cast<const uint2*>(p.res.residual + (int64_t)e_m * p.res.ld_res + e_n);
+                gate2 = *reinterpret_cast<const uint2*>(p.res.gate + (int64_t)(e_m / p.res.gate_group) * p.res.ld_gate + e_n);
+            }
         }
-    }
+    };
 
     // ---- operand rows ----------------------------------------------------------------------
     // weight row of operand row r16 (0..15) of tile nt, token row of operand row r16 of block mb
@@ -188,6 +195,7 @@ __global__ __launch_bounds__(SK_THREADS) void gemm_fp8_skinny_kernel(
                     xhi[j][mb] = *reinterpret_cast<const v4i*>(xrow[mb] + off + 64);
                 }
             }
+            if (rnd == 0) request_residual();
             // ---- 2. MFMA ---------------------------------------------------------------------
 #pragma unroll
             for (int j = 0; j < KPW; ++j) {
@@ -242,6 +250,7 @@ __global__ __launch_bounds__(SK_THREADS) void gemm_fp8_skinny_kernel(
                             copy16_to_lds(p.xq + ((size_t)s << 7), xoff[mb][hf], dst + ((NT + mb) * 2 + hf) * 1024);
                 }
             }
+            if (rnd == 0) request_residual();
             wait_copies<0>();   // everything this wavefront asked for (epilogue operands included)
             // ---- 2. MFMA ---------------------------------------------------------------------
 #pragma unroll
@@ -381,14 +390,14 @@ static void sk_launch_one(const SkinnyArgs& a, const dim3& grid, hipStream_t st)
     if constexpr (fits) {
         if (want && a.K * (int64_t)(a.N > a.M ? a.N : a.M) < ((int64_t)1 << 32)) {
             hipLaunchKernelGGL((gemm_fp8_skinny_kernel<MB, NT, KPW, EPI, true>), grid, dim3(SK_THREADS), 0, st,
-                               a.w, a.xq, a.K, a.M, a.N, a.rounds, a.x_scale, a.w_scale, a.bias, a.out, a.ldo,
-                               a.x_scale_scalar, a.res);
+                               a.w, a.xq, a.x_scale, a.w_scale, a.bias, a.K, a.N, a.M | (a.x_scale_scalar ? 1 << 30 : 0),
+                               a.out, a.ldo, a.res);
             return;
         }
     }
     hipLaunchKernelGGL((gemm_fp8_skinny_kernel<MB, NT, KPW, EPI, false>), grid, dim3(SK_THREADS), 0, st,
-                       a.w, a.xq, a.K, a.M, a.N, a.rounds, a.x_scale, a.w_scale, a.bias, a.out, a.ldo,
-                       a.x_scale_scalar, a.res);
+                       a.w, a.xq, a.x_scale, a.w_scale, a.bias, a.K, a.N, a.M | (a.x_scale_scalar ? 1 << 30 : 0),
+                       a.out, a.ldo, a.res);
 }
 
 template <int MB, int NT, int EPI>
