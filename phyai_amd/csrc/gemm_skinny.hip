@@ -221,9 +221,11 @@ __global__ __launch_bounds__(SK_THREADS) void gemm_fp8_skinny_kernel(
             const int r16 = hf * 8 + c_row;
             const uint32_t chunk = (uint32_t)((c_slot ^ ((r16 >> 1) & 7)) << 4);
 #pragma unroll
-            for (int nt = 0; nt < NT; ++nt) woff[nt][hf] = (uint32_t)w_row(nt, r16) * (uint32_t)p.K + chunk;
+            // rows and K are below 2^24 and their product below 2^32 (checked by the launcher): the
+            // 24-bit multiply is a full-rate instruction, the general one is not
+            for (int nt = 0; nt < NT; ++nt) woff[nt][hf] = __umul24((uint32_t)w_row(nt, r16), (uint32_t)p.K) + chunk;
 #pragma unroll
-            for (int mb = 0; mb < MB; ++mb) xoff[mb][hf] = (uint32_t)x_row(mb, r16) * (uint32_t)p.K + chunk;
+            for (int mb = 0; mb < MB; ++mb) xoff[mb][hf] = __umul24((uint32_t)x_row(mb, r16), (uint32_t)p.K) + chunk;
         }
         const uint32_t lds_wave = __builtin_amdgcn_readfirstlane((uint32_t)(uintptr_t)smem + wave * PER_WAVE);
         const uint8_t* my_stage = smem + wave * PER_WAVE;
@@ -388,7 +390,7 @@ static void sk_launch_one(const SkinnyArgs& a, const dim3& grid, hipStream_t st)
     constexpr bool fits = SK_WAVES * KPW * (NT + MB) * 2048 <= 160 * 1024;
     static const bool want = []() { const char* e = getenv("PHYAI_FP8_SKINNY_STAGED"); return !(e && atoi(e) == 0); }();
     if constexpr (fits) {
-        if (want && a.K * (int64_t)(a.N > a.M ? a.N : a.M) < ((int64_t)1 << 32)) {
+        if (want && a.K * (int64_t)(a.N > a.M ? a.N : a.M) < ((int64_t)1 << 32) && a.K < (1 << 24) && a.N < (1 << 24)) {
             hipLaunchKernelGGL((gemm_fp8_skinny_kernel<MB, NT, KPW, EPI, true>), grid, dim3(SK_THREADS), 0, st,
                                a.w, a.xq, a.x_scale, a.w_scale, a.bias, a.K, a.N, a.M | (a.x_scale_scalar ? 1 << 30 : 0),
                                a.out, a.ldo, a.res);
