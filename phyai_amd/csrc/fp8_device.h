@@ -45,13 +45,41 @@ __device__ __forceinline__ uint32_t e4m3_pack2(float a, float b) {
     return w & 0xFFFFu;
 }
 
+// Cross-lane data movement inside a row of 16 lanes (DPP: a modifier of the VALU instruction
+// itself, a few cycles) instead of a trip through the LDS crossbar (ds_bpermute: ~100 cycles each,
+// six of them in a row for a 64-lane butterfly).  CTRL: 0xB1 = quad_perm [1,0,3,2], 0x4E =
+// quad_perm [2,3,0,1], 0x141 = row_half_mirror, 0x140 = row_mirror; every lane has a source.
+template <int CTRL>
+__device__ __forceinline__ uint32_t dpp_move_u32(uint32_t v) {
+    return (uint32_t)__builtin_amdgcn_update_dpp(0, (int)v, CTRL, 0xF, 0xF, true);
+}
+
+// Maximum over the wavefront, the same value in every lane: four DPP steps leave each row of 16
+// lanes with its maximum, the four rows meet through scalar registers.
 __device__ __forceinline__ uint32_t wave_max_u32(uint32_t v) {
-#pragma unroll
-    for (int off = 32; off >= 1; off >>= 1) {
-        uint32_t o = (uint32_t)__shfl_xor((int)v, off, kWave);
-        v = o > v ? o : v;
-    }
-    return v;
+    uint32_t o;
+    o = dpp_move_u32<0xB1>(v);  v = o > v ? o : v;
+    o = dpp_move_u32<0x4E>(v);  v = o > v ? o : v;
+    o = dpp_move_u32<0x141>(v); v = o > v ? o : v;
+    o = dpp_move_u32<0x140>(v); v = o > v ? o : v;
+    const uint32_t r0 = (uint32_t)__builtin_amdgcn_readlane((int)v, 0), r1 = (uint32_t)__builtin_amdgcn_readlane((int)v, 16);
+    const uint32_t r2 = (uint32_t)__builtin_amdgcn_readlane((int)v, 32), r3 = (uint32_t)__builtin_amdgcn_readlane((int)v, 48);
+    const uint32_t a = r0 > r1 ? r0 : r1, b = r2 > r3 ? r2 : r3;
+    return a > b ? a : b;
+}
+
+// Sum over the wavefront, the same value in every lane, in a fixed order (pairs, quads, halves of
+// a row, rows of 16, then the four rows): reproducible from run to run.
+__device__ __forceinline__ float wave_sum_f32(float v) {
+    v += __uint_as_float(dpp_move_u32<0xB1>(__float_as_uint(v)));
+    v += __uint_as_float(dpp_move_u32<0x4E>(__float_as_uint(v)));
+    v += __uint_as_float(dpp_move_u32<0x141>(__float_as_uint(v)));
+    v += __uint_as_float(dpp_move_u32<0x140>(__float_as_uint(v)));
+    const float r0 = __uint_as_float((uint32_t)__builtin_amdgcn_readlane((int)__float_as_uint(v), 0));
+    const float r1 = __uint_as_float((uint32_t)__builtin_amdgcn_readlane((int)__float_as_uint(v), 16));
+    const float r2 = __uint_as_float((uint32_t)__builtin_amdgcn_readlane((int)__float_as_uint(v), 32));
+    const float r3 = __uint_as_float((uint32_t)__builtin_amdgcn_readlane((int)__float_as_uint(v), 48));
+    return (r0 + r1) + (r2 + r3);
 }
 
 // One 16-byte chunk per lane from global memory straight into LDS: lane i's chunk lands at

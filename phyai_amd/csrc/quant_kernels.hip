@@ -226,8 +226,7 @@ int launch_weight_quant(const void* w, int64_t N, int64_t K, int64_t ldw, void* 
 // ---- RMSNorm / adaptive RMSNorm + quantizer ----------------------------------------------
 template <int THREADS>
 __device__ __forceinline__ float block_sum_f32(float v, float* smem) {
-#pragma unroll
-    for (int off = 32; off >= 1; off >>= 1) v += __shfl_xor(v, off, kWave);
+    v = wave_sum_f32(v);
     if constexpr (THREADS > kWave) {
         constexpr int NW = THREADS / kWave;
         const int wave = threadIdx.x / kWave, lane = threadIdx.x % kWave;
