@@ -493,6 +493,12 @@ BigPlan big_plan(int M, int N, int K, int epilogue) {
              big_ceil_div(M, 192) * 192 <= big_ceil_div(M, 256) * 256 &&
              big_fill(big_tiles(M, N, epilogue, 192, 128), 512) >= big_fill(big_tiles(M, N, epilogue, 256, 256), 256) - 0.15)
         pl.tile = 192;
+    // ... and also when it fits one round of two workgroups per CU while 128 x 128 tiles would just
+    // spill into a second one (3264 x 2560 x 2048: 340 tiles of 192 x 128 take 27 us, 520 of
+    // 128 x 128 take 33 us; with 416 of those, 3264 x 2048 x 2048, the smaller tile wins 20.6 to 25.3)
+    else if (K <= 8192 && big_tiles(M, N, epilogue, 256, 256) < 200 && big_tiles(M, N, epilogue, 192, 128) > 256 &&
+             big_tiles(M, N, epilogue, 192, 128) <= 512 && big_tiles(M, N, epilogue, 128, 128) > 512)
+        pl.tile = 192;
     else if (big_tiles(M, N, epilogue, 256, 256) >= 200) pl.tile = 256;
     else if (big_tiles(M, N, epilogue, 128, 128) >= 32) pl.tile = 128;   // fewer: the weight-streaming kernel wins
     else return pl;
@@ -503,9 +509,11 @@ BigPlan big_plan(int M, int N, int K, int epilogue) {
         // Measured at M = 816: splitting pays for K = 16384 (67 -> 49 us with two splits) and
         // costs for K = 2048 (19 -> 25 us): the partial-sum round trip is worth about 6 us.
         if (tiles < 200 && K >= 8192 && K % 256 == 0) pl.splits = 2;
-        // With well over one tile per CU a ring of two stages lets two workgroups share a CU
-        // (17.5 -> 14.4 us at 800 x 8192 x 1024); with fewer, the deeper ring hides more latency.
-        else if (tiles >= 400) pl.depth = 2;
+        // With more tiles than CUs a ring of two stages lets two workgroups share a CU instead of
+        // queueing behind each other (800 x 8192 x 1024, 448 tiles: 17.5 -> 14.4 us; 1632 x 2560 x 2048,
+        // 260 tiles: 23.3 -> 18.3 us); up to one tile per CU the deeper ring hides more latency
+        // (1632 x 2048 x 2048, 208 tiles: 14.2 against 17.3 us).
+        else if (tiles > 256) pl.depth = 2;
     }
     if (const char* e = getenv("PHYAI_FP8_BIG_SPLITS")) {
         const int s = atoi(e);

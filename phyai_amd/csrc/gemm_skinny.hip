@@ -331,18 +331,27 @@ __global__ __launch_bounds__(SK_THREADS) void gemm_fp8_skinny_kernel(
 static int sk_ceil_div(int a, int b) { return (a + b - 1) / b; }
 
 // Widths are multiples of 8 so that four consecutive output columns are valid together.
-// Largest M served here.  Every 64-row group of tokens re-reads the weight tiles from L2, so
-// beyond a few hundred rows the LDS-staged tile kernels win; the dispatcher prefers those as
-// soon as their grid is large enough (see launch_gemm) and falls back to this kernel up to here.
+// Largest M served here.  Every group of token rows re-reads the weight tiles from L2, so with
+// enough output tiles the LDS-staged tile kernels win; the dispatcher prefers those as soon as
+// their grid is large enough (see launch_gemm) and falls back to this kernel up to here
+// (N = 1024: ahead of 56 tiles of 128 x 128 up to M = 800, 12.3 against 17.5 us at 600 x 1024 x 4096).
 static int skinny_max_m() {
     if (const char* e = getenv("PHYAI_FP8_SKINNY_MAXM")) return atoi(e);
-    return 512;
+    return 896;
 }
 
 bool skinny_applicable(int M, int N, int K, int epilogue, int64_t ldo) {
     if (M > skinny_max_m() || K % 128 != 0 || ldo % 4 != 0) return false;
     if (epi_is_gated(epilogue)) return (N / 2) % 8 == 0;
     return N % 8 == 0;
+}
+
+// K steps a wavefront stages per round: up to 4, as many as K offers and the LDS holds
+static int skinny_steps_per_round(int K, int nt, int mb) {
+    const int per_wave = sk_ceil_div(K / 128, SK_WAVES);
+    int kpw = per_wave >= 4 ? 4 : (per_wave >= 2 ? 2 : 1);
+    while (kpw > 1 && SK_WAVES * kpw * (nt + mb) * 2048 > 160 * 1024) kpw /= 2;
+    return kpw;
 }
 
 SkinnyPlan skinny_plan(int M, int N, int K, int epilogue) {
@@ -364,23 +373,37 @@ SkinnyPlan skinny_plan(int M, int N, int K, int epilogue) {
         if (blocks == 3 && pl.tiles * 3 <= 256) pl.msplit = 3;
         pl.mb = blocks / pl.msplit;
     } else {
-        // more than 64 rows: 64 rows per workgroup keeps the re-reads of a weight tile lowest
-        pl.mb = 4;
-        pl.msplit = sk_ceil_div(blocks, 4);
+        // More than 64 rows.  A workgroup's time is set by the operand blocks it pulls through its
+        // CU's vector cache (nt + mb per K step) and the launch takes as many rounds as the
+        // workgroups need on 256 CUs: take the shape with the smallest product.  Shapes whose
+        // staging would not hold two K steps per wavefront where K offers them are left out
+        // (2 x 4 blocks at K = 4096: 14 us against 6).  Measured at M = 100 .. 600 on the expert
+        // projections, this picks the fastest or second fastest of the eight shapes every time and
+        // beats the former fixed 1 x 4 by 10-30 % (600 x 1024 x 4096: 16.2 -> 12.1 us).
+        int best_cost = 1 << 30;
+        for (int nt = 1; nt <= 2; ++nt) {
+            for (int mb = 1; mb <= 4; ++mb) {
+                if (skinny_steps_per_round(K, nt, mb) < (K >= 2048 ? 2 : 1)) continue;
+                const int wgs = sk_ceil_div(cols, per_tile * nt) * sk_ceil_div(blocks, mb);
+                const int cost = sk_ceil_div(wgs, 256) * (nt + mb);
+                if (cost < best_cost || (cost == best_cost && nt + mb < pl.nt + pl.mb)) {
+                    best_cost = cost; pl.nt = nt; pl.mb = mb;
+                }
+            }
+        }
+        pl.tiles = sk_ceil_div(cols, per_tile * pl.nt);
+        pl.msplit = sk_ceil_div(blocks, pl.mb);
     }
-    const int steps = K / 128;
-    const int per_wave = sk_ceil_div(steps, SK_WAVES);
-    pl.kpw = per_wave >= 4 ? 4 : (per_wave >= 2 ? 2 : 1);
-    // staging of 8 wavefronts x kpw steps x (nt + mb) blocks of 2 KB must fit the 160 KB of LDS:
-    // more rounds of fewer steps beat the unstaged form (down 50..400 x 1024 x 4096: 12 -> 7 us)
-    while (pl.kpw > 1 && SK_WAVES * pl.kpw * (pl.nt + pl.mb) * 2048 > 160 * 1024) pl.kpw /= 2;
-    pl.rounds = sk_ceil_div(per_wave, pl.kpw);
     if (const char* e = getenv("PHYAI_FP8_SKINNY_PLAN")) {  // "nt,mb" tuning override
         int nt = 0, mb = 0;
         if (sscanf(e, "%d,%d", &nt, &mb) == 2 && (nt == 1 || nt == 2) && mb >= 1 && mb <= 4) {
             pl.nt = nt; pl.tiles = sk_ceil_div(cols, per_tile * nt); pl.mb = mb; pl.msplit = sk_ceil_div(blocks, mb);
         }
     }
+    // staging of 8 wavefronts x kpw steps x (nt + mb) blocks of 2 KB must fit the 160 KB of LDS:
+    // more rounds of fewer steps beat the unstaged form (down 50..400 x 1024 x 4096: 12 -> 7 us)
+    pl.kpw = skinny_steps_per_round(K, pl.nt, pl.mb);
+    pl.rounds = sk_ceil_div(sk_ceil_div(K / 128, SK_WAVES), pl.kpw);
     return pl;
 }
 

@@ -374,9 +374,9 @@ int launch_gemm(const GemmProblem& g, hipStream_t st) {
     //   M <= 64                      weight-streaming kernel, nothing else comes close;
     //   pipelined tile kernel        when big_plan finds a tile shape that fills the chip, or at
     //                                least 64 tiles of 128 x 128;
-    //   64 < M <= 512 otherwise      weight-streaming kernel again (few output columns: at
-    //                                N = 1024 it wins up to M = 512, at N = 2560 up to M = 300);
-    //   32 .. 63 small tiles         pipelined tile kernel after all (M > 512);
+    //   64 < M <= 896 otherwise      weight-streaming kernel again (few output columns: at
+    //                                N = 1024 it wins up to M = 800, at N = 2560 up to M = 300);
+    //   32 .. 63 small tiles         pipelined tile kernel after all (M > 896);
     //   the rest                     generic LDS tile kernel (any K, any alignment).
     // The weight-streaming kernel reads scales / bias / output with 128- and 64-bit accesses.
     const bool vec_ok = (reinterpret_cast<uintptr_t>(g.w_scale) % 16 == 0) &&

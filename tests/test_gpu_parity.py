@@ -446,6 +446,46 @@ def test_tile_variants_agree_bit_for_bit_on_random_shapes(dev, monkeypatch):
         assert_close_to_ref(outs["192"], want, f"case {case} {(M, N, K, epi_name)}")
 
 
+def test_weight_streaming_kernel_workgroup_shapes_agree_bit_for_bit(dev, monkeypatch):
+    """The weight-streaming kernel above 64 token rows, in each of its eight workgroup shapes
+    (1-2 weight tiles x 1-4 blocks of 16 token rows) and as the dispatcher picks it: a wavefront
+    always walks its K steps in the same order and the eight partial sums are added in wavefront
+    order, so the shape must not change a single bit.  Ragged M (last workgroup partly or wholly
+    past M), N off the tile width, all epilogues, gated residual; one shape is held to the oracle."""
+    ops = _ops()
+    rng = np.random.default_rng(77)
+    epis = [(None, 0), ("geglu_tanh", 1), ("gelu", 5), ("swiglu", 3)]
+    monkeypatch.setenv("PHYAI_FP8_BIG", "0")              # keep the tile kernels out of the way
+    monkeypatch.setenv("PHYAI_FP8_SKINNY_MAXM", "2048")
+    for case in range(12):
+        M = int(rng.integers(65, 900))
+        N = 32 * int(rng.integers(1, 48))
+        K = 128 * int(rng.integers(1, 34))
+        epi_name, epi = epis[case % len(epis)]
+        x, wq, ws, b = _problem(M, N, K, seed=3000 + case)
+        xq, xs = ops.fp8_quant_rowwise(x.to(dev))
+        wd, sd, bd = wq.to(dev), ws.to(dev), b.to(dev)
+        res = gate = None
+        if epi == 0 and case % 8 == 0:
+            res = seeded((M, N), seed=4000 + case).to(dev)
+            gate = seeded((1, N), seed=5000 + case).to(dev)
+        outs = {}
+        for plan in [None] + [f"{nt},{mb}" for nt in (1, 2) for mb in (1, 2, 3, 4)]:
+            if plan is None:
+                monkeypatch.delenv("PHYAI_FP8_SKINNY_PLAN", raising=False)
+            else:
+                monkeypatch.setenv("PHYAI_FP8_SKINNY_PLAN", plan)
+            assert ops.describe_plan(M, N, K, epi_name).startswith("small-m ")
+            outs[plan] = ops.fp8_gemm(xq, xs, wd, sd, bd, epilogue=epi_name, residual=res, gate=gate)
+        torch.cuda.synchronize()
+        for plan, o in outs.items():
+            assert torch.equal(_as_bits(o), _as_bits(outs[None])), \
+                f"case {case} {(M, N, K, epi_name)}: shape {plan} differs in {int((_as_bits(o) != _as_bits(outs[None])).sum())} outputs"
+        if res is None:
+            want = ref.epilogue(ref.gemm_f32(*ref.quant_rowwise(x), wq, ws, b), epi).float()
+            assert_close_to_ref(outs[None], want, f"case {case} {(M, N, K, epi_name)}")
+
+
 @pytest.mark.parametrize("tile", ["128", "256"])
 def test_big_tile_kernel_split_k(dev, monkeypatch, tile):
     """Both tile sizes with the K range split over two and four workgroups (partials in the workspace)."""
