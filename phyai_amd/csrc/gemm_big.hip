@@ -76,18 +76,49 @@ struct BigArgs {
 // grid is cut into bands of 4 tile rows; inside a band, 8 consecutive ids are 8 neighbouring
 // tile columns (one per XCD), and the next 8 ids the same columns one tile row further down.  An
 // XCD thus works on all (up to 4) tile rows of one tile column together - the weight rows come
-// from HBM once per band - while the activation rows of the band stay in its L2.  Tile columns
-// are padded to a multiple of 8; ids that fall into the padding have no tile.
+// from HBM once per band - while the activation rows of the band stay in its L2.
+// Tile columns beyond the last multiple of 8 would leave some XCDs a whole column more than
+// others (20 columns: three for XCDs 0-3, two for the rest, and the launch lasts as long as the
+// busiest XCD).  The tiles of those last columns are therefore taken in column-major order and
+// cut into 8 runs of equal length (within one), one per XCD: still whole or half columns per
+// XCD, and every XCD gets the same number of tiles.  Ids past an XCD's run have no tile.
 struct BigTile { int m, n; };
 __device__ __forceinline__ BigTile big_tile_of(int id, int m_tiles, int n_tiles, int band_rows) {
-    const int nt8 = (n_tiles + 7) & ~7;
-    const int band = id / (band_rows * nt8);
-    const int local = id - band * band_rows * nt8;
+    const int full = n_tiles >> 3, rest = n_tiles & 7;   // whole groups of 8 tile columns; columns after them
+    const int per_band = 8 * (band_rows * full + ((rest * band_rows + 7) >> 3));
+    const int band = id / per_band;
+    const int local = id - band * per_band;
     const int bm = m_tiles - band_rows * band < band_rows ? m_tiles - band_rows * band : band_rows;
     BigTile t;
-    t.n = (local / (8 * bm)) * 8 + (local & 7);
-    t.m = band_rows * band + (local >> 3) % bm;
+    if (local < 8 * bm * full) {
+        t.n = (local / (8 * bm)) * 8 + (local & 7);
+        t.m = band_rows * band + (local >> 3) % bm;
+    } else {
+        const int j = local - 8 * bm * full, x = j & 7, total = rest * bm;
+        const int e = ((x * total) >> 3) + (j >> 3);                  // (j / 8)-th tile of XCD x's run
+        t.n = e < (((x + 1) * total) >> 3) ? 8 * full + e / bm : n_tiles;   // n_tiles: no tile
+        t.m = band_rows * band + e % bm;
+    }
     return t;
+}
+// Tiles of the busiest XCD under that order (host side; the same arithmetic, band by band).
+static int big_max_tiles_per_xcd(int m_tiles, int n_tiles, int band_rows) {
+    const int full = n_tiles >> 3, rest = n_tiles & 7;
+    int per_xcd[8] = {0, 0, 0, 0, 0, 0, 0, 0};
+    for (int m = 0; m < m_tiles; m += band_rows) {
+        const int bm = m_tiles - m < band_rows ? m_tiles - m : band_rows;
+        for (int x = 0; x < 8; ++x) per_xcd[x] += bm * full + ((((x + 1) * rest * bm) >> 3) - ((x * rest * bm) >> 3));
+    }
+    int mx = 0;
+    for (int x = 0; x < 8; ++x) mx = per_xcd[x] > mx ? per_xcd[x] : mx;
+    return mx;
+}
+// Ids that order needs (host side).
+static int big_grid_ids(int m_tiles, int n_tiles, int band_rows) {
+    const int full = n_tiles >> 3, rest = n_tiles & 7;
+    const int bands = m_tiles / band_rows, last = m_tiles % band_rows;
+    return bands * 8 * (band_rows * full + ((rest * band_rows + 7) >> 3)) +
+           (last ? 8 * (last * full + ((rest * last + 7) >> 3)) : 0);
 }
 
 // Swizzle of the eight 16-byte chunks of a 128-byte row.  LDS has 64 banks of 4 bytes, so one
@@ -487,11 +518,13 @@ BigPlan big_plan(int M, int N, int K, int epilogue) {
     // tile's prologue and epilogue leave the MFMA pipe idle; 192 x 128 tiles fit twice and overlap
     // them.  The small tile wins once there are enough of them and while K is short enough for
     // prologue and epilogue to matter (measured: 4-18 % up to K = 8192), unless M pads worse or
-    // its last round of 512 tiles would be much emptier than the large tile's last round of 256
-    // (6528 x 2048 x 2048: 544 small tiles take 42 us, 208 large ones 37.5 us).
+    // its last round of 512 tiles would be emptier than the large tile's last round of 256
+    // (6528 x 2048 x 2048: 544 small tiles take 42 us, 208 large ones 37.5 us; with operands that
+    // come from HBM, 13056 x 2560 x 2048: 1360 small tiles 80 us, 510 large ones 75.5 us, and
+    // 4800 x 6144 x 2048: 73.4 against 68.7 us).
     else if (K <= 8192 && big_tiles(M, N, epilogue, 192, 128) >= 400 &&
              big_ceil_div(M, 192) * 192 <= big_ceil_div(M, 256) * 256 &&
-             big_fill(big_tiles(M, N, epilogue, 192, 128), 512) >= big_fill(big_tiles(M, N, epilogue, 256, 256), 256) - 0.15)
+             big_fill(big_tiles(M, N, epilogue, 192, 128), 512) >= big_fill(big_tiles(M, N, epilogue, 256, 256), 256) - 0.05)
         pl.tile = 192;
     // ... and also when it fits one round of two workgroups per CU while 128 x 128 tiles would just
     // spill into a second one (3264 x 2560 x 2048: 340 tiles of 192 x 128 take 27 us, 520 of
@@ -550,6 +583,13 @@ static void big_launch(BigArgs a, const GemmProblem& g, int splits, hipStream_t 
         const double by_cols = a_bytes * (a.n_tiles < 8 ? a.n_tiles : 8) + b_bytes * big_ceil_div(a.m_tiles, band_c);
         const double by_rows = b_bytes * (a.m_tiles < 8 ? a.m_tiles : 8) + a_bytes * big_ceil_div(a.n_tiles, band_r);
         a.by_rows = by_rows < 0.8 * by_cols;
+        // ... unless the busiest XCD then needs one more round of tiles than in the other order
+        // (13056 x 2560 x 2048 in 256 x 256 tiles: 510 tiles are 64 per XCD by tile columns, two
+        // rounds on 32 CUs, but 65 on some XCDs by tile rows: 92 against 75.5 us)
+        const int slots = 32 * ((DEPTH == 2 && TM < 4) ? 2 : 1);
+        const int rounds_c = big_ceil_div(big_max_tiles_per_xcd(a.m_tiles, a.n_tiles, 4), slots);
+        const int rounds_r = big_ceil_div(big_max_tiles_per_xcd(a.n_tiles, a.m_tiles, 4), slots);
+        if (rounds_c != rounds_r) a.by_rows = rounds_r < rounds_c;
         if (const char* e = getenv("PHYAI_FP8_BY_ROWS")) a.by_rows = atoi(e) != 0;
     }
     // bands of 4 tile rows; a grid of up to 8 tile rows whose activation rows still fit an XCD's
@@ -558,7 +598,7 @@ static void big_launch(BigArgs a, const GemmProblem& g, int splits, hipStream_t 
     if (!a.by_rows && a.m_tiles <= 8 && (int64_t)a.m_tiles * (64 * TM) * (g.K < 4096 ? g.K : 4096) <= (5 << 19)) a.band = a.m_tiles;
     if (const char* e = getenv("PHYAI_FP8_BAND")) { const int b = atoi(e); if (b >= 1 && b <= 16) a.band = b; }
     const int outer = a.by_rows ? a.n_tiles : a.m_tiles, inner = a.by_rows ? a.m_tiles : a.n_tiles;
-    const dim3 grid(outer * ((inner + 7) & ~7), 1, splits);
+    const dim3 grid(big_grid_ids(outer, inner, a.band), 1, splits);
 #define PHYAI_BIG_ARGS a.a, a.b, a.K, a.M, a.N, a.m_tiles, a.n_tiles, a.band, a.by_rows, a.k_per_split, a.a_scale, \
                        a.b_scale, a.bias, a.out, a.ldo, a.a_scale_scalar, a.partials, a.counters, a.res
     if (splits > 1) {
