@@ -112,35 +112,52 @@ __global__ __launch_bounds__(SK_THREADS) void gemm_fp8_skinny_kernel(
     const int total_steps = p.K >> 7;
     const int m_base = blockIdx.y * (MB * 16);
 
-    // ---- epilogue role of this thread and its operands (requested first) ---------
-    // thread -> (tile e_nt, token block e_mb, lane position e_lane); it finishes token
-    // m = 16*e_mb + e_lane%16 and output columns e_n .. e_n+3.
+    // ---- epilogue roles of this thread and their operands (requested first) --------------------
+    // A role is (tile e_nt, token block e_mb): the thread finishes token m = 16*e_mb + lane%16
+    // and output columns e_n .. e_n+3 of it.  The eight wavefronts cover eight roles at a time;
+    // workgroup shapes with more blocks than that (NT * MB > 8) go round twice.
+    constexpr int ROLE_ROUNDS = (NT * MB + SK_WAVES - 1) / SK_WAVES;
     const int e_lane = tid & 63;
-    const int e_mb = (tid >> 6) % MB;
-    const int e_nt = (tid >> 6) / MB;
     const int e_q = e_lane >> 4;
-    const bool e_role = (e_nt < NT) && (!GATED || e_q < 2);
-    const int e_m = m_base + e_mb * 16 + (e_lane & 15);
-    const int e_n = col0 + (e_nt < NT ? e_nt : 0) * COLS_PER_TILE + 4 * e_q;
-    const bool e_live = e_role && e_m < p.M && e_n < n_out_total;
-    const int e_n_safe = e_live ? e_n : 0;
-    const v4f sw4 = *reinterpret_cast<const v4f*>(p.w_scale + e_n_safe);
-    v4f su4 = v4f{0.f, 0.f, 0.f, 0.f};
-    if constexpr (GATED) su4 = *reinterpret_cast<const v4f*>(p.w_scale + half_n + e_n_safe);
-    uint2 bw2 = make_uint2(0, 0), bu2 = make_uint2(0, 0);
-    if (p.bias) {
-        bw2 = *reinterpret_cast<const uint2*>(p.bias + e_n_safe);
-        if constexpr (GATED) bu2 = *reinterpret_cast<const uint2*>(p.bias + half_n + e_n_safe);
+    int e_mb[ROLE_ROUNDS], e_nt[ROLE_ROUNDS], e_m[ROLE_ROUNDS], e_n[ROLE_ROUNDS];
+    bool e_role[ROLE_ROUNDS], e_live[ROLE_ROUNDS];
+    v4f sw4[ROLE_ROUNDS], su4[ROLE_ROUNDS];
+    uint2 bw2[ROLE_ROUNDS], bu2[ROLE_ROUNDS];
+    float sa[ROLE_ROUNDS];
+#pragma unroll
+    for (int rr = 0; rr < ROLE_ROUNDS; ++rr) {
+        const int role = rr * SK_WAVES + (tid >> 6);
+        e_mb[rr] = role % MB;
+        e_nt[rr] = role / MB;
+        e_role[rr] = (e_nt[rr] < NT) && (!GATED || e_q < 2);
+        e_m[rr] = m_base + e_mb[rr] * 16 + (e_lane & 15);
+        e_n[rr] = col0 + (e_nt[rr] < NT ? e_nt[rr] : 0) * COLS_PER_TILE + 4 * e_q;
+        e_live[rr] = e_role[rr] && e_m[rr] < p.M && e_n[rr] < n_out_total;
+        const int e_n_safe = e_live[rr] ? e_n[rr] : 0;
+        sw4[rr] = *reinterpret_cast<const v4f*>(p.w_scale + e_n_safe);
+        su4[rr] = v4f{0.f, 0.f, 0.f, 0.f};
+        if constexpr (GATED) su4[rr] = *reinterpret_cast<const v4f*>(p.w_scale + half_n + e_n_safe);
+        bw2[rr] = make_uint2(0, 0); bu2[rr] = make_uint2(0, 0);
+        if (p.bias) {
+            bw2[rr] = *reinterpret_cast<const uint2*>(p.bias + e_n_safe);
+            if constexpr (GATED) bu2[rr] = *reinterpret_cast<const uint2*>(p.bias + half_n + e_n_safe);
+        }
+        sa[rr] = p.x_scale[(p.x_scale_scalar || !e_live[rr]) ? 0 : e_m[rr]];
     }
-    const float sa = p.x_scale[(p.x_scale_scalar || !e_live) ? 0 : e_m];
     // gated residual: requested once the operand requests are out (its arguments are not among
     // the preloaded ones, and nothing before the operand requests should wait for a scalar load)
-    uint2 res2 = make_uint2(0, 0), gate2 = make_uint2(0, 0);
+    uint2 res2[ROLE_ROUNDS], gate2[ROLE_ROUNDS];
+#pragma unroll
+    for (int rr = 0; rr < ROLE_ROUNDS; ++rr) { res2[rr] = make_uint2(0, 0); gate2[rr] = make_uint2(0, 0); }
     auto request_residual = [&]() {
         if constexpr (EPI == EPI_NONE) {
-            if (p.res.residual != nullptr && e_live) {
-                res2 = *reinterpret_cast<const uint2*>(p.res.residual + (int64_t)e_m * p.res.ld_res + e_n);
-                gate2 = *reinterpret_cast<const uint2*>(p.res.gate + (int64_t)(e_m / p.res.gate_group) * p.res.ld_gate + e_n);
+#pragma unroll
+            for (int rr = 0; rr < ROLE_ROUNDS; ++rr) {
+                if (p.res.residual != nullptr && e_live[rr]) {
+                    res2[rr] = *reinterpret_cast<const uint2*>(p.res.residual + (int64_t)e_m[rr] * p.res.ld_res + e_n[rr]);
+                    gate2[rr] = *reinterpret_cast<const uint2*>(
+                        p.res.gate + (int64_t)(e_m[rr] / p.res.gate_group) * p.res.ld_gate + e_n[rr]);
+                }
             }
         }
     };
@@ -287,43 +304,46 @@ __global__ __launch_bounds__(SK_THREADS) void gemm_fp8_skinny_kernel(
 #pragma unroll
         for (int mb = 0; mb < MB; ++mb) red(wave, nt, mb, lane) = acc[nt][mb];
     __syncthreads();
-    if (!e_role) return;
-    v4f g = red(0, e_nt, e_mb, e_lane);
 #pragma unroll
-    for (int w = 1; w < SK_WAVES; ++w) g += red(w, e_nt, e_mb, e_lane);
-    v4f u = v4f{0.f, 0.f, 0.f, 0.f};
-    if constexpr (GATED) {
-        u = red(0, e_nt, e_mb, e_lane + 32);
+    for (int rr = 0; rr < ROLE_ROUNDS; ++rr) {
+        if (!e_role[rr]) continue;
+        v4f g = red(0, e_nt[rr], e_mb[rr], e_lane);
 #pragma unroll
-        for (int w = 1; w < SK_WAVES; ++w) u += red(w, e_nt, e_mb, e_lane + 32);
-    }
-
-    // ---- 4. epilogue ------------------------------------------------------------------------
-    const float bwf[4] = {bf16_bits_to_f32(bw2.x & 0xFFFFu), bf16_bits_to_f32(bw2.x >> 16),
-                          bf16_bits_to_f32(bw2.y & 0xFFFFu), bf16_bits_to_f32(bw2.y >> 16)};
-    const float buf[4] = {bf16_bits_to_f32(bu2.x & 0xFFFFu), bf16_bits_to_f32(bu2.x >> 16),
-                          bf16_bits_to_f32(bu2.y & 0xFFFFu), bf16_bits_to_f32(bu2.y >> 16)};
-    uint32_t o[4];
-    float vf[4];
-#pragma unroll
-    for (int r = 0; r < 4; ++r) {
-        float v = __builtin_fmaf(g[r], sa * sw4[r], bwf[r]);   // one rounding, like the tile kernels
+        for (int w = 1; w < SK_WAVES; ++w) g += red(w, e_nt[rr], e_mb[rr], e_lane);
+        v4f u = v4f{0.f, 0.f, 0.f, 0.f};
         if constexpr (GATED) {
-            const float up = __builtin_fmaf(u[r], sa * su4[r], buf[r]);
-            v = apply_act<EPI>(round_bf16(v)) * round_bf16(up);
-        } else if constexpr (EPI != EPI_NONE) {
-            v = apply_act<EPI>(round_bf16(v));
-        }
-        vf[r] = v;
-    }
-    if constexpr (EPI == EPI_NONE) {
-        if (p.res.residual != nullptr) addcmul4(vf, res2, gate2);
-    }
+            u = red(0, e_nt[rr], e_mb[rr], e_lane + 32);
 #pragma unroll
-    for (int r = 0; r < 4; ++r) o[r] = f32_to_bf16_bits(vf[r]);
-    if (e_live)
-        *reinterpret_cast<uint2*>(p.out + (int64_t)e_m * p.ldo + e_n) =
-            make_uint2(o[0] | (o[1] << 16), o[2] | (o[3] << 16));
+            for (int w = 1; w < SK_WAVES; ++w) u += red(w, e_nt[rr], e_mb[rr], e_lane + 32);
+        }
+
+        // ---- 4. epilogue --------------------------------------------------------------------
+        const float bwf[4] = {bf16_bits_to_f32(bw2[rr].x & 0xFFFFu), bf16_bits_to_f32(bw2[rr].x >> 16),
+                              bf16_bits_to_f32(bw2[rr].y & 0xFFFFu), bf16_bits_to_f32(bw2[rr].y >> 16)};
+        const float buf[4] = {bf16_bits_to_f32(bu2[rr].x & 0xFFFFu), bf16_bits_to_f32(bu2[rr].x >> 16),
+                              bf16_bits_to_f32(bu2[rr].y & 0xFFFFu), bf16_bits_to_f32(bu2[rr].y >> 16)};
+        uint32_t o[4];
+        float vf[4];
+#pragma unroll
+        for (int r = 0; r < 4; ++r) {
+            float v = __builtin_fmaf(g[r], sa[rr] * sw4[rr][r], bwf[r]);   // one rounding, like the tile kernels
+            if constexpr (GATED) {
+                const float up = __builtin_fmaf(u[r], sa[rr] * su4[rr][r], buf[r]);
+                v = apply_act<EPI>(round_bf16(v)) * round_bf16(up);
+            } else if constexpr (EPI != EPI_NONE) {
+                v = apply_act<EPI>(round_bf16(v));
+            }
+            vf[r] = v;
+        }
+        if constexpr (EPI == EPI_NONE) {
+            if (p.res.residual != nullptr) addcmul4(vf, res2[rr], gate2[rr]);
+        }
+#pragma unroll
+        for (int r = 0; r < 4; ++r) o[r] = f32_to_bf16_bits(vf[r]);
+        if (e_live[rr])
+            *reinterpret_cast<uint2*>(p.out + (int64_t)e_m[rr] * p.ldo + e_n[rr]) =
+                make_uint2(o[0] | (o[1] << 16), o[2] | (o[3] << 16));
+    }
 }
 
 // ---- host side -------------------------------------------------------------------------
@@ -334,10 +354,10 @@ static int sk_ceil_div(int a, int b) { return (a + b - 1) / b; }
 // Largest M served here.  Every group of token rows re-reads the weight tiles from L2, so with
 // enough output tiles the LDS-staged tile kernels win; the dispatcher prefers those as soon as
 // their grid is large enough (see launch_gemm) and falls back to this kernel up to here
-// (N = 1024: ahead of 56 tiles of 128 x 128 up to M = 800, 12.3 against 17.5 us at 600 x 1024 x 4096).
+// (N = 1024: ahead of the 128 x 128 tile kernel up to M = 1000, 11.0 against 17.5 us at 800 x 1024 x 4096).
 static int skinny_max_m() {
     if (const char* e = getenv("PHYAI_FP8_SKINNY_MAXM")) return atoi(e);
-    return 896;
+    return 1024;
 }
 
 bool skinny_applicable(int M, int N, int K, int epilogue, int64_t ldo) {
@@ -375,20 +395,19 @@ SkinnyPlan skinny_plan(int M, int N, int K, int epilogue) {
     } else {
         // More than 64 rows.  A workgroup's time is set by the operand blocks it pulls through its
         // CU's vector cache (nt + mb per K step) and the launch takes as many rounds as the
-        // workgroups need on 256 CUs: take the shape with the smallest product.  Shapes whose
-        // staging would not hold two K steps per wavefront where K offers them are left out
-        // (2 x 4 blocks at K = 4096: 14 us against 6).  Measured at M = 100 .. 600 on the expert
-        // projections, this picks the fastest or second fastest of the eight shapes every time and
-        // beats the former fixed 1 x 4 by 10-30 % (600 x 1024 x 4096: 16.2 -> 12.1 us).
+        // workgroups need on 256 CUs: take the shape with the smallest product.  Measured at
+        // M = 100 .. 1000 on the 1024-wide expert projections, the product orders the shapes as
+        // the clock does (800 x 1024 x 4096: 4x4 11.0 us, 2x4 13.6, 4x3 15.8, 2x3 16.4, 2x2 17.9
+        // for products 8, 12, 14, 15, 16) and the winner beats the former fixed 1 x 4 by 10-40 %
+        // (and the 128 x 128 tile kernel there: 17.5 us).
         int best_cost = 1 << 30;
-        for (int nt = 1; nt <= 2; ++nt) {
-            for (int mb = 1; mb <= 4; ++mb) {
-                if (skinny_steps_per_round(K, nt, mb) < (K >= 2048 ? 2 : 1)) continue;
-                const int wgs = sk_ceil_div(cols, per_tile * nt) * sk_ceil_div(blocks, mb);
-                const int cost = sk_ceil_div(wgs, 256) * (nt + mb);
-                if (cost < best_cost || (cost == best_cost && nt + mb < pl.nt + pl.mb)) {
-                    best_cost = cost; pl.nt = nt; pl.mb = mb;
-                }
+        static const int shapes[][2] = {{1, 1}, {1, 2}, {1, 3}, {1, 4}, {2, 1}, {2, 2}, {2, 3}, {2, 4}, {4, 3}, {4, 4}};
+        for (const auto& sh : shapes) {
+            const int nt = sh[0], mb = sh[1];
+            const int wgs = sk_ceil_div(cols, per_tile * nt) * sk_ceil_div(blocks, mb);
+            const int cost = sk_ceil_div(wgs, 256) * (nt + mb);
+            if (cost < best_cost || (cost == best_cost && nt + mb < pl.nt + pl.mb)) {
+                best_cost = cost; pl.nt = nt; pl.mb = mb;
             }
         }
         pl.tiles = sk_ceil_div(cols, per_tile * pl.nt);
@@ -396,7 +415,7 @@ SkinnyPlan skinny_plan(int M, int N, int K, int epilogue) {
     }
     if (const char* e = getenv("PHYAI_FP8_SKINNY_PLAN")) {  // "nt,mb" tuning override
         int nt = 0, mb = 0;
-        if (sscanf(e, "%d,%d", &nt, &mb) == 2 && (nt == 1 || nt == 2) && mb >= 1 && mb <= 4) {
+        if (sscanf(e, "%d,%d", &nt, &mb) == 2 && (nt == 1 || nt == 2 || (nt == 4 && mb >= 3)) && mb >= 1 && mb <= 4) {
             pl.nt = nt; pl.tiles = sk_ceil_div(cols, per_tile * nt); pl.mb = mb; pl.msplit = sk_ceil_div(blocks, mb);
         }
     }
@@ -438,6 +457,13 @@ static int sk_launch_kpw(const SkinnyArgs& a, const SkinnyPlan& pl, hipStream_t 
 
 template <int EPI>
 static int sk_launch_epi(const SkinnyArgs& a, const SkinnyPlan& pl, hipStream_t st) {
+    if (pl.nt == 4) {   // four weight tiles: 3 or 4 token blocks, one K step per wavefront per round
+        if (pl.kpw != 1) return -2;
+        const dim3 grid(pl.tiles, pl.msplit);
+        if (pl.mb == 3) { sk_launch_one<3, 4, 1, EPI>(a, grid, st); return 0; }
+        if (pl.mb == 4) { sk_launch_one<4, 4, 1, EPI>(a, grid, st); return 0; }
+        return -2;
+    }
     switch (pl.mb * 2 + (pl.nt - 1)) {
     case 2: return sk_launch_kpw<1, 1, EPI>(a, pl, st);
     case 3: return sk_launch_kpw<1, 2, EPI>(a, pl, st);

@@ -358,7 +358,7 @@ int describe_gemm_plan(int M, int N, int K, int epilogue, char* buf, size_t n) {
     if (skinny_ok && M <= 64) return small();
     if (!getenv("PHYAI_FP8_TILE")) {
         const BigPlan bp = big_plan(M, N, K, epilogue);
-        const bool few_small_tiles = bp.tile == 128 && bp.tiles < 64 && !getenv("PHYAI_FP8_BIG");
+        const bool few_small_tiles = bp.tile == 128 && bp.tiles <= 64 && !getenv("PHYAI_FP8_BIG");
         if (bp.tile && ldo % 8 == 0 && !(few_small_tiles && skinny_ok))
             return snprintf(buf, n, "tile %dx%d depth=%d splits=%d tiles=%d", bp.tile, bp.tile == 256 ? 256 : 128,
                             bp.depth, bp.splits, bp.tiles);
@@ -372,11 +372,11 @@ int launch_gemm(const GemmProblem& g, hipStream_t st) {
     if (g.M == 0 || g.N == 0) return 0;
     // Kernel choice (measured on the expert and prefill shapes, M = 50 .. 13056):
     //   M <= 64                      weight-streaming kernel, nothing else comes close;
-    //   pipelined tile kernel        when big_plan finds a tile shape that fills the chip, or at
-    //                                least 64 tiles of 128 x 128;
-    //   64 < M <= 896 otherwise      weight-streaming kernel again (few output columns: at
-    //                                N = 1024 it wins up to M = 800, at N = 2560 up to M = 300);
-    //   32 .. 63 small tiles         pipelined tile kernel after all (M > 896);
+    //   pipelined tile kernel        when big_plan finds a tile shape that fills the chip, or more
+    //                                than 64 tiles of 128 x 128;
+    //   64 < M <= 1024 otherwise     weight-streaming kernel again (few output columns: at
+    //                                N = 1024 it wins up to M = 1000, at N = 2560 up to M = 300);
+    //   32 .. 64 small tiles         pipelined tile kernel after all (M > 1024);
     //   the rest                     generic LDS tile kernel (any K, any alignment).
     // The weight-streaming kernel reads scales / bias / output with 128- and 64-bit accesses.
     const bool vec_ok = (reinterpret_cast<uintptr_t>(g.w_scale) % 16 == 0) &&
@@ -386,7 +386,7 @@ int launch_gemm(const GemmProblem& g, hipStream_t st) {
     if (skinny_ok && g.M <= 64) return launch_gemm_skinny(g, skinny_plan(g.M, g.N, g.K, g.epilogue), st);
     if (!getenv("PHYAI_FP8_TILE")) {
         const BigPlan bp = big_plan(g.M, g.N, g.K, g.epilogue);
-        const bool few_small_tiles = bp.tile == 128 && bp.tiles < 64 && !getenv("PHYAI_FP8_BIG");
+        const bool few_small_tiles = bp.tile == 128 && bp.tiles <= 64 && !getenv("PHYAI_FP8_BIG");
         if (bp.tile && !(few_small_tiles && skinny_ok)) {
             const int rc = launch_gemm_big(g, bp, st);
             if (rc != -2) return rc;  // -2: output not 16-byte addressable, try the others

@@ -63,7 +63,7 @@ def test_kernel_selection_for_the_benchmark_shapes(monkeypatch):
     chip and K is long or the last round of smaller tiles would be emptier; 192 x 128 tiles (two
     workgroups per CU) for K <= 8192 with enough tiles, or when they fit one round and 128 x 128 tiles
     would not; 128 x 128 tiles with a ring of two once there are more tiles than CUs, split along K
-    for K >= 8192 with few tiles; weight streaming again below 64 small tiles up to 896 rows, its
+    for K >= 8192 with few tiles; weight streaming again up to 64 small tiles and 1024 rows, its
     workgroup shape chosen by (rounds of workgroups) x (operand blocks per workgroup)."""
     from phyai_amd import ops
 
@@ -95,10 +95,12 @@ def test_kernel_selection_for_the_benchmark_shapes(monkeypatch):
     assert d(3264, 2560, 2048) == "tile 192x128 depth=2 splits=1 tiles=340"   # 520 small tiles would spill
     assert d(3264, 2048, 2048) == "tile 128x128 depth=2 splits=1 tiles=416"   # 416 do not
     assert d(200, 1024, 4096).startswith("small-m ")           # 16 small tiles: weight streaming wins
-    assert d(800, 1024, 4096) == "small-m nt=2 mb=3 kpw=2 rounds=2"  # 56 small tiles: still weight streaming
-    assert d(400, 1024, 2048) == "small-m nt=2 mb=2 kpw=2 rounds=1"  # fewest cache-bound rounds: 416 workgroups x 4 blocks
-    assert d(100, 2560, 1024) == "small-m nt=2 mb=3 kpw=1 rounds=1"
-    assert d(1000, 1024, 4096) == "tile 128x128 depth=4 splits=1 tiles=64"
+    assert d(800, 1024, 4096) == "small-m nt=4 mb=4 kpw=1 rounds=4"  # 56 small tiles: still weight streaming, 208 workgroups x 8 blocks
+    assert d(400, 1024, 2048) == "small-m nt=2 mb=4 kpw=1 rounds=2"  # 224 workgroups x 6 blocks
+    assert d(100, 2560, 1024) == "small-m nt=2 mb=3 kpw=1 rounds=1"  # 240 workgroups x 5 blocks
+    assert d(100, 8192, 1024, "geglu_tanh") == "small-m nt=4 mb=4 kpw=1 rounds=1"
+    assert d(1000, 1024, 4096) == "small-m nt=4 mb=4 kpw=1 rounds=4"
+    assert d(1100, 1024, 4096) == "tile 128x128 depth=4 splits=1 tiles=72"
     # what the fast kernels refuse goes to the generic one
     assert d(300, 384, 272).startswith("generic ")
     with pytest.raises(RuntimeError, match="multiples of 16"):

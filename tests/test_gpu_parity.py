@@ -447,8 +447,8 @@ def test_tile_variants_agree_bit_for_bit_on_random_shapes(dev, monkeypatch):
 
 
 def test_weight_streaming_kernel_workgroup_shapes_agree_bit_for_bit(dev, monkeypatch):
-    """The weight-streaming kernel above 64 token rows, in each of its eight workgroup shapes
-    (1-2 weight tiles x 1-4 blocks of 16 token rows) and as the dispatcher picks it: a wavefront
+    """The weight-streaming kernel above 64 token rows, in each of its workgroup shapes
+    (1-2 weight tiles x 1-4 blocks of 16 token rows, 4 tiles x 3-4 blocks) and as the dispatcher picks it: a wavefront
     always walks its K steps in the same order and the eight partial sums are added in wavefront
     order, so the shape must not change a single bit.  Ragged M (last workgroup partly or wholly
     past M), N off the tile width, all epilogues, gated residual; one shape is held to the oracle."""
@@ -470,7 +470,7 @@ def test_weight_streaming_kernel_workgroup_shapes_agree_bit_for_bit(dev, monkeyp
             res = seeded((M, N), seed=4000 + case).to(dev)
             gate = seeded((1, N), seed=5000 + case).to(dev)
         outs = {}
-        for plan in [None] + [f"{nt},{mb}" for nt in (1, 2) for mb in (1, 2, 3, 4)]:
+        for plan in [None] + [f"{nt},{mb}" for nt in (1, 2) for mb in (1, 2, 3, 4)] + ["4,3", "4,4"]:
             if plan is None:
                 monkeypatch.delenv("PHYAI_FP8_SKINNY_PLAN", raising=False)
             else:
