@@ -56,7 +56,7 @@ DIT_SET = [("qkv", 6144, 2048, None, 4800), ("out", 2048, 2048, None, 4800),
 # HBM bytes moved by one layer's four GEMM launches at M = 50 (20.87 MB fetched + 0.87 MB written),
 # measured with rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE on `bench.py --probe` and calibrated against
 # a 64 MiB copy (profiles/expert_m50_hbm_traffic.md has the counter values).
-EXPERT_LAYER_HBM_TRAFFIC = 21_780_000
+EXPERT_LAYER_HBM_TRAFFIC = 21_790_000
 
 
 def algorithmic_bytes(M: int, N: int, K: int, epilogue, bias: bool = False) -> int:

@@ -380,30 +380,22 @@ SkinnyPlan skinny_plan(int M, int N, int K, int epilogue) {
     const int per_tile = gated ? 8 : 16;
     SkinnyPlan pl;
     const int blocks = sk_ceil_div(M, 16);  // 16-row token blocks in all
-    // two weight tiles per workgroup once that still leaves a workgroup for every CU - except for a
-    // single token block, where the narrow tile's smaller staging lets two workgroups share a CU
-    // and overlap each other's phases (1 x 12288 x 2048: 8.6 -> 7.8 us)
-    pl.nt = (sk_ceil_div(cols, 2 * per_tile) >= 256 && blocks > 1) ? 2 : 1;
-    pl.tiles = sk_ceil_div(cols, per_tile * pl.nt);
-    if (blocks <= 4) {
-        // split M while there are fewer workgroups than CUs
-        pl.msplit = 1;
-        if (blocks % 2 == 0 && pl.tiles * 2 <= 256) pl.msplit = 2;
-        if (blocks % 4 == 0 && pl.tiles * 4 <= 256) pl.msplit = 4;
-        if (blocks == 3 && pl.tiles * 3 <= 256) pl.msplit = 3;
-        pl.mb = blocks / pl.msplit;
-    } else {
-        // More than 64 rows.  A workgroup's time is set by the operand blocks it pulls through its
-        // CU's vector cache (nt + mb per K step) and the launch takes as many rounds as the
-        // workgroups need on 256 CUs: take the shape with the smallest product.  Measured at
-        // M = 100 .. 1000 on the 1024-wide expert projections, the product orders the shapes as
-        // the clock does (800 x 1024 x 4096: 4x4 11.0 us, 2x4 13.6, 4x3 15.8, 2x3 16.4, 2x2 17.9
-        // for products 8, 12, 14, 15, 16) and the winner beats the former fixed 1 x 4 by 10-40 %
-        // (and the 128 x 128 tile kernel there: 17.5 us).
+    // Workgroup shape: nt weight tiles x mb token blocks.  A workgroup's time is set by the operand
+    // blocks it pulls through its CU's vector cache (nt + mb per K step) and the launch takes as
+    // many rounds as the workgroups need on 256 CUs: take the shape with the smallest product
+    // (ties: the smaller workgroup).  The product orders the shapes as the clock does - at M = 50
+    // (2560 columns: 2x2 3.49 us, 1x1 3.66, 1x4 3.73, 2x4 4.04 for products 4, 4, 5, 6; 1024
+    // columns: 1x1 with four workgroups along M; gate_up: 2x4) as at M = 100 .. 1000
+    // (800 x 1024 x 4096: 4x4 11.0 us, 2x4 13.6, 4x3 15.8, 2x3 16.4, 2x2 17.9 for products 8, 12,
+    // 14, 15, 16), where the winner beats a fixed 1 x 4 by 10-50 % and, on the 1024-wide
+    // projections, the 128 x 128 tile kernel (17.5 us).
+    {
         int best_cost = 1 << 30;
+        pl.nt = 1; pl.mb = 1;
         static const int shapes[][2] = {{1, 1}, {1, 2}, {1, 3}, {1, 4}, {2, 1}, {2, 2}, {2, 3}, {2, 4}, {4, 3}, {4, 4}};
         for (const auto& sh : shapes) {
             const int nt = sh[0], mb = sh[1];
+            if (mb > blocks && mb > 1) continue;   // token blocks that do not exist
             const int wgs = sk_ceil_div(cols, per_tile * nt) * sk_ceil_div(blocks, mb);
             const int cost = sk_ceil_div(wgs, 256) * (nt + mb);
             if (cost < best_cost || (cost == best_cost && nt + mb < pl.nt + pl.mb)) {

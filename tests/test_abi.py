@@ -72,7 +72,7 @@ def test_kernel_selection_for_the_benchmark_shapes(monkeypatch):
         monkeypatch.delenv(var, raising=False)
     d = ops.describe_plan
     # action expert, M = 50
-    assert d(50, 2560, 1024) == "small-m nt=1 mb=4 kpw=1 rounds=1"
+    assert d(50, 2560, 1024) == "small-m nt=2 mb=2 kpw=1 rounds=1"    # 160 workgroups x 4 operand blocks
     assert d(50, 1024, 2048) == "small-m nt=1 mb=1 kpw=2 rounds=1"
     assert d(50, 8192, 1024, "geglu_tanh") == "small-m nt=2 mb=4 kpw=1 rounds=1"
     assert d(50, 1024, 4096) == "small-m nt=1 mb=1 kpw=4 rounds=1"
