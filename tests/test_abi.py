@@ -86,7 +86,7 @@ def test_kernel_selection_for_the_benchmark_shapes(monkeypatch):
     assert d(1632, 32768, 2048, "geglu_tanh") == "tile 192x128 depth=2 splits=1 tiles=2304"
     assert d(4800, 8192, 2048, "gelu") == "tile 192x128 depth=2 splits=1 tiles=1600"
     assert d(6528, 2048, 2048) == "tile 256x256 depth=2 splits=1 tiles=208"
-    assert d(13056, 2560, 2048) == "tile 256x256 depth=2 splits=1 tiles=510"   # two full rounds of large tiles
+    assert d(13056, 2560, 2048) == "tile 192x128 depth=2 splits=1 tiles=1360"
     assert d(6528, 2560, 2048) == "tile 192x128 depth=2 splits=1 tiles=680"    # 260 large tiles: a nearly empty round
     assert d(6528, 2048, 16384) == "tile 256x256 depth=2 splits=1 tiles=208"
     assert d(800, 8192, 1024, "geglu_tanh") == "tile 128x128 depth=2 splits=1 tiles=448"
