@@ -110,18 +110,14 @@ __device__ __forceinline__ float scale_from_amax_bits(uint32_t amax_bits) {
     }
 }
 
-// Streams that are touched once: loads and stores that do not keep their lines in L2.  The codes
-// are always stored that way (816 x 16384: 12.1 -> 9.2 us, never slower); the rows are loaded that
-// way only when the tensor is far larger than the caches (from 100 MB: 13056 x 16384 119.9 ->
-// 106.3 us, 6.0 TB/s; at 6528 x 2048 it costs 10 %).  Same box, alternating builds.
-typedef unsigned int v2u __attribute__((ext_vector_type(2)));
+// A tensor that is far larger than the caches and read once is loaded without keeping its lines
+// in L2 (from 100 MB, long rows only: 13056 x 16384 119.9 -> 111.9 us; at 6528 x 2048 it would
+// cost 10 %).  The codes are stored normally: streaming them out as well makes this kernel
+// faster (816 x 16384: 12.0 -> 9.2 us) but the GEMM that reads them next slower by more.
+// Same box, alternating builds.
 __device__ __forceinline__ uint4 nt_load16(const uint16_t* p) {
     const v4i v = __builtin_nontemporal_load(reinterpret_cast<const v4i*>(p));
     return make_uint4((uint32_t)v[0], (uint32_t)v[1], (uint32_t)v[2], (uint32_t)v[3]);
-}
-__device__ __forceinline__ void nt_store8(uint8_t* p, uint2 v) {
-    const v2u w = {v.x, v.y};
-    __builtin_nontemporal_store(w, reinterpret_cast<v2u*>(p));
 }
 
 template <int THREADS, int CHUNKS, int MODE, bool STREAM_IN>
@@ -148,7 +144,7 @@ __global__ __launch_bounds__(THREADS) void quant_rows_reg_kernel(
 #pragma unroll
     for (int c = 0; c < CHUNKS; ++c) {
         const int k = (c * THREADS + threadIdx.x) * 8;
-        if (k < K) nt_store8(qr + k, encode8<MODE>(v[c], d));
+        if (k < K) *reinterpret_cast<uint2*>(qr + k) = encode8<MODE>(v[c], d);
     }
 }
 
