@@ -95,7 +95,8 @@ def run_layers(layers, shapes):
     for layer in layers:
         for name, _, _, _ in shapes:
             t = layer[name]
-            ops.fp8_linear(t["x"], t["w"], t["ws"], None, epilogue=t["epi"], out=t["out"])
+            ops.fp8_linear(t["x"], t["w"], t["ws"], None, epilogue=t["epi"], out=t["out"],
+                           stream_weights=t.get("stream", False))
 
 
 def torch_reference_times(dev, layers, shapes, denoise_steps, steps, warmup):
@@ -163,7 +164,8 @@ def decoder_layer_times(dev, layers, M, denoise_steps, steps, warmup):
                 y = ops.fp8_linear(attn, o["w"], o["ws"], None, out=o["out"])
                 torch.addcmul(h, y, gate, out=h1)
                 m, gate2 = ops.adarmsnorm(h1, mods[1], 1e-6)
-                a = ops.fp8_linear(m, gu["w"], gu["ws"], None, epilogue="geglu_tanh", out=gu["out"])
+                a = ops.fp8_linear(m, gu["w"], gu["ws"], None, epilogue="geglu_tanh", out=gu["out"],
+                                   stream_weights=gu.get("stream", False))
                 y2 = ops.fp8_linear(a, dn["w"], dn["ws"], None, out=dn["out"])
                 torch.addcmul(h1, y2, gate2, out=h2)
 
@@ -175,7 +177,8 @@ def decoder_layer_times(dev, layers, M, denoise_steps, steps, warmup):
                 ops.fp8_gemm(nq, ns, q["w"], q["ws"], None, out=q["out"])
                 ops.fp8_linear(attn, o["w"], o["ws"], None, residual=h, gate=gate, out=h1)
                 mq, ms, gate2 = ops.adarmsnorm_fp8(h1, mods[1], 1e-6)
-                a = ops.fp8_gemm(mq, ms, gu["w"], gu["ws"], None, epilogue="geglu_tanh", out=gu["out"])
+                a = ops.fp8_gemm(mq, ms, gu["w"], gu["ws"], None, epilogue="geglu_tanh", out=gu["out"],
+                                 stream_weights=gu.get("stream", False))
                 ops.fp8_linear(a, dn["w"], dn["ws"], None, residual=h1, gate=gate2, out=h2)
 
     res = {}
@@ -257,7 +260,8 @@ def whole_step_times(dev, layers, M, prefix_len, denoise_steps, steps, warmup):
         fused = ops.fp8_gemm(nq, ns, layer["qkv"]["w"], layer["qkv"]["ws"], None)
         h = ops.fp8_linear(attention(fused, li), layer["o"]["w"], layer["o"]["ws"], None, residual=h, gate=gate)
         mq, ms, gate2 = ops.adarmsnorm_fp8(h, mod[1], 1e-6)
-        a = ops.fp8_gemm(mq, ms, layer["gate_up"]["w"], layer["gate_up"]["ws"], None, epilogue="geglu_tanh")
+        a = ops.fp8_gemm(mq, ms, layer["gate_up"]["w"], layer["gate_up"]["ws"], None, epilogue="geglu_tanh",
+                         stream_weights=layer["gate_up"].get("stream", False))
         return ops.fp8_linear(a, layer["down"]["w"], layer["down"]["ws"], None, residual=h, gate=gate2)
 
     def layer_torch(h, layer, li, mod):
@@ -379,7 +383,8 @@ def gemm_only_times(dev, layers, shapes, M, reps=8, iters=30):
         def fn():
             for _ in range(reps):
                 for xq, xs, t in pre:
-                    ops.fp8_gemm(xq, xs, t["w"], t["ws"], None, epilogue=t["epi"], out=t["out"])
+                    ops.fp8_gemm(xq, xs, t["w"], t["ws"], None, epilogue=t["epi"], out=t["out"],
+                                 stream_weights=t.get("stream", False))
 
         g = HipGraph()
         g.capture(fn, {})
@@ -471,7 +476,8 @@ def probe(dev, layers, M, shapes=EXPERT_SET):
         pre = [(ops.fp8_quant_rowwise(layer[name]["x"]), layer[name]) for layer in layers]
         torch.cuda.synchronize()
         for (xq, xs), t in pre:
-            ops.fp8_gemm(xq, xs, t["w"], t["ws"], None, epilogue=t["epi"], out=t["out"])
+            ops.fp8_gemm(xq, xs, t["w"], t["ws"], None, epilogue=t["epi"], out=t["out"],
+                         stream_weights=t.get("stream", False))
         torch.cuda.synchronize()
     src = torch.empty(64 << 20, dtype=torch.uint8, device=dev).fill_(1)
     dst = torch.empty_like(src)
@@ -513,6 +519,8 @@ def main() -> int:
     ap.add_argument("--warmup", type=int, default=20)
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--no-prefill", action="store_true")
+    ap.add_argument("--no-cache-plan", action="store_true",
+                    help="read every weight matrix with ordinary loads (no matrix is streamed past the Infinity Cache)")
     ap.add_argument("--no-extras", action="store_true",
                     help="skip the comparisons in `extra` (fused decoder-layer path, torch reference path): "
                          "only this library's kernels run, for profiler sessions")
@@ -545,6 +553,16 @@ def main() -> int:
         return 0
 
     layers = make_layers(dev, EXPERT_SET, M, n_layers)
+    # What a runner does once per model: the weights of one denoise step (311 MB) exceed the 256 MB
+    # Infinity Cache, so the largest matrices are read past it and the others stay resident from
+    # step to step (phyai_amd/cache_plan.py).
+    from phyai_amd.cache_plan import choose_streamed
+    entries = [layer[name] for layer in layers for name, _, _, _ in EXPERT_SET]
+    frac = float(os.environ.get("PHYAI_BENCH_RESIDENT_FRACTION", "0.7"))
+    for t, streamed in zip(entries, choose_streamed([t["N"] * t["K"] for t in entries], resident_fraction=frac)):
+        t["stream"] = streamed and not args.no_cache_plan
+    streamed_mb = sum(t["N"] * t["K"] for t in entries if t["stream"]) / 1e6
+    resident_mb = sum(t["N"] * t["K"] for t in entries if not t["stream"]) / 1e6
 
     if args.probe:
         probe(dev, layers, M)
@@ -635,7 +653,10 @@ def main() -> int:
                                "gate_up 1024->8192 + GeGLU, down 4096->1024}, M=50, distinct weights per layer",
                    "step": "one hipGraph replay = 10 denoise steps = 720 quantized linears",
                    "denoise_steps_per_replay": denoise_steps, "cache_policy":
-                   "311 MB of weights per denoise step cycle through HBM; nothing is pinned in cache"},
+                   (f"311 MB of weights per denoise step against a 256 MB Infinity Cache: {streamed_mb:.0f} MB (the largest "
+                    f"matrices) are read with non-temporal loads, the other {resident_mb:.0f} MB may stay cached from "
+                    "step to step; nothing is pinned" if streamed_mb else
+                    "311 MB of weights per denoise step cycle through HBM; every matrix is read with ordinary loads")},
         "roofline": roofline, "cpu_baseline": cpu, "extra": extra,
     }
     print(json.dumps(line))

@@ -31,7 +31,7 @@
 extern "C" {
 #endif
 
-#define PHYAI_FP8_ABI_VERSION 3
+#define PHYAI_FP8_ABI_VERSION 4
 
 enum {
     PHYAI_FP8_OK = 0,
@@ -51,6 +51,21 @@ enum {
     PHYAI_FP8_EPI_GELU_TANH = 4,  /* plain fc1 -> gelu_tanh -> [M, N]              */
     PHYAI_FP8_EPI_GELU_ERF = 5    /* plain fc1 -> gelu (erf) -> [M, N]             */
 };
+
+/*
+ * Flags, OR-ed into the `epilogue` argument of phyai_fp8_gemm / phyai_fp8_linear (the epilogue
+ * code is `epilogue & PHYAI_FP8_EPILOGUE_MASK`).
+ *
+ * STREAM_WEIGHTS: read this call's weight matrix with non-temporal loads, so that it does not
+ * displace other data from the 256 MB Infinity Cache.  A model whose weights exceed that cache and
+ * are re-read every step (the action expert: 311 MB per denoise step, ten steps per inference)
+ * gets no cache hits at all when everything is cached alike; marking the largest matrices lets
+ * the rest stay resident (phyai_amd/cache_plan.py picks them).  Honoured by the small-M kernel
+ * (M <= 64, K % 128 == 0), ignored elsewhere; results are bit-identical with and without it.  The
+ * reference has no counterpart (its GEMM is a library call, linear/backends/torch.py:168-175).
+ */
+#define PHYAI_FP8_EPILOGUE_MASK 0xFF
+#define PHYAI_FP8_FLAG_STREAM_WEIGHTS 0x100
 
 int phyai_fp8_abi_version(void);
 const char *phyai_fp8_last_error(void);

@@ -106,7 +106,7 @@ int phyai_fp8_weight_quant_rowwise(const void* w, int64_t N, int64_t K, int64_t 
 }
 
 size_t phyai_fp8_linear_workspace_bytes(int64_t M, int64_t N, int64_t K, int epilogue) {
-    return carve(M, N, K, epilogue).total;
+    return carve(M, N, K, epilogue & PHYAI_FP8_EPILOGUE_MASK).total;
 }
 
 namespace {
@@ -135,6 +135,9 @@ int run_gemm(const char* fn, const void* xq, const float* x_scale, int x_scale_i
              int64_t N, int64_t K, int epilogue, void* workspace, size_t workspace_bytes, void* stream) {
     if (M < 0 || N <= 0 || K <= 0)
         return fail(PHYAI_FP8_EINVAL, "%s: bad shape M=%lld N=%lld K=%lld", fn, (long long)M, (long long)N, (long long)K);
+    const int flags = epilogue & ~PHYAI_FP8_EPILOGUE_MASK;
+    epilogue &= PHYAI_FP8_EPILOGUE_MASK;
+    if (flags & ~PHYAI_FP8_FLAG_STREAM_WEIGHTS) return fail(PHYAI_FP8_EINVAL, "%s: unknown flag bits 0x%x", fn, flags);
     if (int rc = check_epilogue(epilogue, N)) return rc;
     if (K % 16 != 0 || N % 16 != 0)
         return fail(PHYAI_FP8_EUNSUPPORTED, "%s: K=%lld and N=%lld must be multiples of 16", fn, (long long)K, (long long)N);
@@ -159,6 +162,7 @@ int run_gemm(const char* fn, const void* xq, const float* x_scale, int x_scale_i
     g.ldo = ldo;
     g.M = (int)M; g.N = (int)N; g.K = (int)K;
     g.epilogue = epilogue;
+    g.stream_weights = (flags & PHYAI_FP8_FLAG_STREAM_WEIGHTS) ? 1 : 0;
     g.workspace = workspace;
     g.workspace_bytes = workspace_bytes;
     g.gate_group = 1;
@@ -183,7 +187,7 @@ int run_linear(const char* fn, const void* x, int64_t ldx, const void* w, const 
     if (M < 0 || N <= 0 || K <= 0)
         return fail(PHYAI_FP8_EINVAL, "%s: bad shape M=%lld N=%lld K=%lld", fn, (long long)M, (long long)N, (long long)K);
     if (M == 0) return PHYAI_FP8_OK;
-    const LinearCarve c = carve(M, N, K, epilogue);
+    const LinearCarve c = carve(M, N, K, epilogue & PHYAI_FP8_EPILOGUE_MASK);
     if (!workspace || workspace_bytes < c.total)
         return fail(PHYAI_FP8_EWORKSPACE, "%s: workspace of %zu bytes is too small, need %zu", fn,
                     workspace ? workspace_bytes : (size_t)0, c.total);
@@ -296,6 +300,7 @@ int phyai_fp8_describe_plan(int64_t M, int64_t N, int64_t K, int epilogue, char*
     buf[0] = 0;
     if (M < 0 || N <= 0 || K <= 0 || M >= kMaxElems || N >= kMaxElems || K >= kMaxElems)
         return fail(PHYAI_FP8_EINVAL, "phyai_fp8_describe_plan: bad shape M=%lld N=%lld K=%lld", (long long)M, (long long)N, (long long)K);
+    epilogue &= PHYAI_FP8_EPILOGUE_MASK;   // flags do not change the choice of kernel
     if (int rc = check_epilogue(epilogue, N)) return rc;
     if (K % 16 != 0 || N % 16 != 0)
         return fail(PHYAI_FP8_EUNSUPPORTED, "phyai_fp8_describe_plan: K=%lld and N=%lld must be multiples of 16", (long long)K, (long long)N);

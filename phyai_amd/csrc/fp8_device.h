@@ -90,6 +90,13 @@ __device__ __forceinline__ void copy16_to_lds(const uint8_t* base, uint32_t lane
                  :: "v"(lane_offset), "s"(base), "s"(lds_wave_base) : "memory", "m0");
 }
 
+// The same copy for data that should not stay in the caches behind it (read once per pass over a
+// working set that is larger than they are).
+__device__ __forceinline__ void copy16_to_lds_nt(const uint8_t* base, uint32_t lane_offset, uint32_t lds_wave_base) {
+    asm volatile("s_mov_b32 m0, %2\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, %1 nt"
+                 :: "v"(lane_offset), "s"(base), "s"(lds_wave_base) : "memory", "m0");
+}
+
 // s_waitcnt vmcnt(N) with a compile-time N: at most N of this wavefront's copies still in flight.
 template <int N>
 __device__ __forceinline__ void wait_copies() {

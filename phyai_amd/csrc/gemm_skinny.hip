@@ -50,6 +50,7 @@ struct SkinnyArgs {
     int M, N, K;
     int x_scale_scalar;
     int rounds;  // K steps are consumed in rounds of SK_WAVES * KPW
+    int stream_w;  // weights with non-temporal loads
     ResidualArgs res;
 };
 
@@ -84,10 +85,14 @@ __global__ __launch_bounds__(SK_THREADS) void gemm_fp8_skinny_kernel(
     const float* __restrict__ a_w_scale, const uint16_t* __restrict__ a_bias, int a_K, int a_N, int a_m_flags,
     uint16_t* __restrict__ a_out, int64_t a_ldo, const ResidualArgs a_res) {
     // 13 preloaded dwords: everything the operand requests and the early epilogue loads need.
-    // a_m_flags = M | x_scale_is_scalar << 30; the rounds follow from K.
+    // a_m_flags = M | stream_weights << 29 | x_scale_is_scalar << 30; the rounds follow from K.
     SkinnyArgs p;
     p.xq = a_xq; p.w = a_w; p.x_scale = a_x_scale; p.w_scale = a_w_scale; p.bias = a_bias; p.out = a_out;
-    p.ldo = a_ldo; p.M = a_m_flags & 0x3FFFFFFF; p.N = a_N; p.K = a_K; p.x_scale_scalar = (a_m_flags >> 30) & 1;
+    p.ldo = a_ldo; p.M = a_m_flags & 0x0FFFFFFF; p.N = a_N; p.K = a_K; p.x_scale_scalar = (a_m_flags >> 30) & 1;
+    // weights read with non-temporal loads: a matrix that the caller does not want to displace
+    // others from the Infinity Cache (STAGED form only; the hint is ignored otherwise)
+    const bool stream_w = __builtin_amdgcn_readfirstlane((a_m_flags >> 29) & 1) != 0;
+    (void)stream_w;
     p.rounds = (((a_K >> 7) + SK_WAVES - 1) / SK_WAVES + KPW - 1) / KPW;
     p.res = a_res;
     constexpr bool GATED = epi_is_gated(EPI);
@@ -257,11 +262,20 @@ __global__ __launch_bounds__(SK_THREADS) void gemm_fp8_skinny_kernel(
                 const int s = __builtin_amdgcn_readfirstlane((rnd * KPW + j) * SK_WAVES + wave);
                 if (s < total_steps) {
                     const uint32_t dst = lds_wave + j * (BLOCKS * 2048);
+                    // one branch per K step: the weights of this call either pass the caches by or not
+                    if (stream_w) {
 #pragma unroll
-                    for (int nt = 0; nt < NT; ++nt)
+                        for (int nt = 0; nt < NT; ++nt)
 #pragma unroll
-                        for (int hf = 0; hf < 2; ++hf)
-                            copy16_to_lds(p.w + ((size_t)s << 7), woff[nt][hf], dst + (nt * 2 + hf) * 1024);
+                            for (int hf = 0; hf < 2; ++hf)
+                                copy16_to_lds_nt(p.w + ((size_t)s << 7), woff[nt][hf], dst + (nt * 2 + hf) * 1024);
+                    } else {
+#pragma unroll
+                        for (int nt = 0; nt < NT; ++nt)
+#pragma unroll
+                            for (int hf = 0; hf < 2; ++hf)
+                                copy16_to_lds(p.w + ((size_t)s << 7), woff[nt][hf], dst + (nt * 2 + hf) * 1024);
+                    }
 #pragma unroll
                     for (int mb = 0; mb < MB; ++mb)
 #pragma unroll
@@ -426,13 +440,13 @@ static void sk_launch_one(const SkinnyArgs& a, const dim3& grid, hipStream_t st)
     if constexpr (fits) {
         if (want && a.K * (int64_t)(a.N > a.M ? a.N : a.M) < ((int64_t)1 << 32) && a.K < (1 << 24) && a.N < (1 << 24)) {
             hipLaunchKernelGGL((gemm_fp8_skinny_kernel<MB, NT, KPW, EPI, true>), grid, dim3(SK_THREADS), 0, st,
-                               a.w, a.xq, a.x_scale, a.w_scale, a.bias, a.K, a.N, a.M | (a.x_scale_scalar ? 1 << 30 : 0),
+                               a.w, a.xq, a.x_scale, a.w_scale, a.bias, a.K, a.N, a.M | (a.x_scale_scalar ? 1 << 30 : 0) | (a.stream_w ? 1 << 29 : 0),
                                a.out, a.ldo, a.res);
             return;
         }
     }
     hipLaunchKernelGGL((gemm_fp8_skinny_kernel<MB, NT, KPW, EPI, false>), grid, dim3(SK_THREADS), 0, st,
-                       a.w, a.xq, a.x_scale, a.w_scale, a.bias, a.K, a.N, a.M | (a.x_scale_scalar ? 1 << 30 : 0),
+                       a.w, a.xq, a.x_scale, a.w_scale, a.bias, a.K, a.N, a.M | (a.x_scale_scalar ? 1 << 30 : 0) | (a.stream_w ? 1 << 29 : 0),
                        a.out, a.ldo, a.res);
 }
 
@@ -475,6 +489,7 @@ int launch_gemm_skinny(const GemmProblem& g, const SkinnyPlan& pl, hipStream_t s
     a.out = g.out; a.ldo = g.ldo; a.M = g.M; a.N = g.N; a.K = g.K;
     a.x_scale_scalar = g.x_scale_is_scalar;
     a.rounds = pl.rounds;
+    a.stream_w = g.stream_weights;
     a.res = residual_of(g);
     switch (g.epilogue) {
     case EPI_NONE: return sk_launch_epi<EPI_NONE>(a, pl, st);

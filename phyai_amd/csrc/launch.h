@@ -55,6 +55,8 @@ struct GemmProblem {
     const uint16_t* gate;      // [M / gate_group, N] bf16
     int64_t ld_gate;
     int gate_group;
+    // Hint: read the weights with non-temporal loads (honoured by the weight-streaming kernel).
+    int stream_weights;
 };
 
 // What the kernels need of the above, by value.

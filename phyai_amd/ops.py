@@ -30,6 +30,7 @@ EPILOGUES = {
 }
 
 WORKSPACE_HEADER_BYTES = 16384
+FLAG_STREAM_WEIGHTS = 0x100   # OR-ed into the epilogue argument of the C entry points
 
 
 def _err(op: str, msg: str) -> RuntimeError:
@@ -355,8 +356,12 @@ def _check_addcmul(op: str, residual, gate, lead: tuple[int, ...], M: int, N: in
 
 def fp8_gemm(xq: torch.Tensor, x_scale: torch.Tensor, weight: torch.Tensor, weight_scale: torch.Tensor,
              bias: torch.Tensor | None = None, *, epilogue=None, out: torch.Tensor | None = None,
-             residual: torch.Tensor | None = None, gate: torch.Tensor | None = None) -> torch.Tensor:
+             residual: torch.Tensor | None = None, gate: torch.Tensor | None = None,
+             stream_weights: bool = False) -> torch.Tensor:
     """``bf16(act((xq @ weight.T) * x_scale * weight_scale + bias))`` on quantized inputs.
+
+    ``stream_weights``: read the weights past the caches (see :mod:`phyai_amd.cache_plan`);
+    same result, honoured at small M without a gated residual.
 
     With ``residual`` and ``gate`` the result is ``torch.addcmul(residual, y, gate)`` of that
     linear output ``y`` (reference ``models/pi05/modeling_pi05.py:826,835``), in the same kernel;
@@ -395,7 +400,8 @@ def fp8_gemm(xq: torch.Tensor, x_scale: torch.Tensor, weight: torch.Tensor, weig
             g2.shape[0], out.data_ptr(), n_out, M, N, K, ws.data_ptr(), ws.numel(), _stream_ptr())
     else:
         rc = _lib.load().phyai_fp8_gemm(x2.data_ptr(), xs.data_ptr(), scalar, weight.data_ptr(),
-                                         weight_scale.data_ptr(), bias_ptr, out.data_ptr(), n_out, M, N, K, epi,
+                                         weight_scale.data_ptr(), bias_ptr, out.data_ptr(), n_out, M, N, K,
+                                         epi | (FLAG_STREAM_WEIGHTS if stream_weights else 0),
                                          ws.data_ptr(), ws.numel(), _stream_ptr())
     _lib.check(rc, op)
     return out
@@ -403,9 +409,12 @@ def fp8_gemm(xq: torch.Tensor, x_scale: torch.Tensor, weight: torch.Tensor, weig
 
 def fp8_linear(x: torch.Tensor, weight: torch.Tensor, weight_scale: torch.Tensor,
                bias: torch.Tensor | None = None, *, epilogue=None, out: torch.Tensor | None = None,
-               residual: torch.Tensor | None = None, gate: torch.Tensor | None = None) -> torch.Tensor:
+               residual: torch.Tensor | None = None, gate: torch.Tensor | None = None,
+               stream_weights: bool = False) -> torch.Tensor:
     """The whole W8A8 linear on bf16 ``x[..., K]``: per-token quantization, fp8 MFMA
     GEMM, per-channel dequantization, bias and optional activation, bf16 out.
+
+    ``stream_weights``: as for :func:`fp8_gemm`.
 
     Replaces ``TorchKernel._fp8_per_channel`` (reference
     ``layers/linear/backends/torch.py:155-176``) and, with a gated ``epilogue``,
@@ -433,7 +442,8 @@ def fp8_linear(x: torch.Tensor, weight: torch.Tensor, weight_scale: torch.Tensor
             g2.shape[0], out.data_ptr(), n_out, M, N, K, ws.data_ptr(), ws.numel(), _stream_ptr())
     else:
         rc = _lib.load().phyai_fp8_linear(x2.data_ptr(), x2.stride(0) if M > 1 else K, weight.data_ptr(),
-                                           weight_scale.data_ptr(), bias_ptr, out.data_ptr(), n_out, M, N, K, epi,
+                                           weight_scale.data_ptr(), bias_ptr, out.data_ptr(), n_out, M, N, K,
+                                           epi | (FLAG_STREAM_WEIGHTS if stream_weights else 0),
                                            ws.data_ptr(), ws.numel(), _stream_ptr())
     _lib.check(rc, op)
     return out

@@ -52,6 +52,11 @@ def test_workspace_query_and_argument_validation_without_gpu():
     assert b"multiples of 16" in lib.phyai_fp8_last_error()
     assert lib.phyai_fp8_gemm(None, None, 0, None, None, None, None, 64, 4, 64, 64, 9, None, 0, None) == -1
     assert lib.phyai_fp8_gemm(None, None, 0, None, None, None, None, 64, 0, 64, 64, 0, None, 0, None) == 0
+    # flag bits ride in the epilogue argument: the known one is accepted, others are not
+    assert lib.phyai_fp8_gemm(None, None, 0, None, None, None, None, 64, 0, 64, 64, 0x100 | 1, None, 0, None) == 0
+    assert lib.phyai_fp8_gemm(None, None, 0, None, None, None, None, 64, 4, 64, 64, 0x200, None, 0, None) == -1
+    assert b"flag" in lib.phyai_fp8_last_error()
+    assert lib.phyai_fp8_linear_workspace_bytes(50, 1024, 4096, 0x100) == lib.phyai_fp8_linear_workspace_bytes(50, 1024, 4096, 0)
     buf = (ctypes.c_char * 64)()
     assert lib.phyai_fp8_linear(ctypes.addressof(buf), 64, None, None, None, None, 64, 4, 64, 64, 0, None, 0, None) == -3
     assert b"workspace" in lib.phyai_fp8_last_error()

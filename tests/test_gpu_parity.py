@@ -446,6 +446,26 @@ def test_tile_variants_agree_bit_for_bit_on_random_shapes(dev, monkeypatch):
         assert_close_to_ref(outs["192"], want, f"case {case} {(M, N, K, epi_name)}")
 
 
+@pytest.mark.parametrize("M,N,K,epi_name", [
+    (50, 2560, 1024, None), (50, 8192, 1024, "geglu_tanh"), (50, 1024, 4096, None), (1, 12288, 2048, None),
+    (64, 4096, 1024, "gelu_tanh"), (33, 1024, 16384, None), (200, 1024, 4096, None), (816, 2048, 2048, None),
+])
+def test_streamed_weights_give_the_same_bits(dev, M, N, K, epi_name):
+    """Weights read with non-temporal loads (the flag that keeps a matrix out of the Infinity
+    Cache) change where the bytes are cached, never the result - in the kernel that honours the
+    flag (small M, also over several rounds of K steps) and in those that ignore it."""
+    ops = _ops()
+    x, wq, ws, b = _problem(M, N, K, seed=11 * M + N + K)
+    xd, wd, sd, bd = x.to(dev), wq.to(dev), ws.to(dev), b.to(dev)
+    xq, xs = ops.fp8_quant_rowwise(xd)
+    plain = ops.fp8_linear(xd, wd, sd, bd, epilogue=epi_name)
+    streamed = ops.fp8_linear(xd, wd, sd, bd, epilogue=epi_name, stream_weights=True)
+    streamed_gemm = ops.fp8_gemm(xq, xs, wd, sd, bd, epilogue=epi_name, stream_weights=True)
+    torch.cuda.synchronize()
+    assert torch.equal(_as_bits(streamed), _as_bits(plain))
+    assert torch.equal(_as_bits(streamed_gemm), _as_bits(plain))
+
+
 def test_weight_streaming_kernel_workgroup_shapes_agree_bit_for_bit(dev, monkeypatch):
     """The weight-streaming kernel above 64 token rows, in each of its workgroup shapes
     (1-2 weight tiles x 1-4 blocks of 16 token rows, 4 tiles x 3-4 blocks) and as the dispatcher picks it: a wavefront

@@ -360,3 +360,33 @@ def test_ops_reject_bad_arguments_before_touching_the_gpu():
     with pytest.raises(RuntimeError, match="unknown epilogue"):
         ops.fp8_linear(x, None, None, epilogue="relu")
     assert ops.workspace_bytes(50, 2560, 1024) >= 16384 + 50 * 1024
+
+
+def test_cache_plan_streams_the_largest_matrices_until_the_rest_fits():
+    """phyai_amd.cache_plan: the action expert's 72 matrices (311 MB against a 256 MB cache): only
+    gate_up matrices are streamed, as few as leave the rest within the resident share; a model
+    that fits streams nothing; the module form marks the layers."""
+    from phyai_amd.cache_plan import choose_streamed, plan_weight_streaming
+
+    per_layer = [2560 * 1024, 1024 * 2048, 8192 * 1024, 1024 * 4096]
+    sizes = per_layer * 18
+    flags = choose_streamed(sizes)
+    assert all(not f for s, f in zip(sizes, flags) if s != 8192 * 1024)        # only the largest kind
+    resident = sum(s for s, f in zip(sizes, flags) if not f)
+    assert resident <= 0.7 * (256 << 20) < resident + 8192 * 1024               # no more than needed
+    assert sum(flags) == 15
+    assert choose_streamed([10 << 20] * 10) == [False] * 10                     # 100 MB: fits
+    assert choose_streamed([]) == []
+    assert choose_streamed([300 << 20]) == [True]                               # one matrix larger than the cache
+
+    class Lin(torch.nn.Module):
+        def __init__(self, n, k):
+            super().__init__()
+            self.weight = torch.nn.Parameter(torch.empty(n, k, dtype=torch.uint8), requires_grad=False)
+
+    mods = [Lin(n, k) for n, k in [(2560, 1024), (1024, 2048), (8192, 1024), (1024, 4096)] * 18] + [torch.nn.ReLU()]
+    left = plan_weight_streaming(mods)
+    assert left == resident
+    assert [m.stream_weights for m in mods[:4]] == [False, False, True, False]
+    assert not hasattr(mods[-1], "stream_weights")
+
