@@ -95,6 +95,26 @@ def test_layers_run_the_hip_kernel(L, dev):
     assert_close_to_ref(y2, ref.gemm_f32(xq, xs, wq2, ws2), "skip_bias_add leaves the bias out")
 
 
+def test_cache_plan_marks_layers_and_the_marked_layers_give_the_same_bits(L, dev):
+    """plan_weight_streaming on a small stack of fp8 layers (cache size scaled down so that it has
+    to choose): the largest layer is marked, HipFp8Kernel passes the hint on, outputs are equal."""
+    from phyai_amd.cache_plan import plan_weight_streaming
+    from phyai_amd.quant import Fp8Spec
+
+    small = L.ReplicatedLinear(1024, 512, bias=False, params_dtype=torch.bfloat16, spec=Fp8Spec())
+    large = L.MergedColumnParallelLinear(1024, [2048, 2048], bias=False, params_dtype=torch.bfloat16, spec=Fp8Spec())
+    _load_fp8(small, seeded((512, 1024), 11, 0.02).to(dev))
+    _load_fp8(large, seeded((4096, 1024), 12, 0.02).to(dev))
+    x = seeded((50, 1024), 13).to(dev)
+    before = [small(x)[0].clone(), large(x)[0].clone()]
+    left = plan_weight_streaming([small, large], cache_bytes=2 << 20, resident_fraction=0.5)
+    assert (small.stream_weights, large.stream_weights) == (False, True) and left == 512 * 1024
+    after = [small(x)[0], large(x)[0]]
+    torch.cuda.synchronize()
+    for a, b in zip(before, after):
+        assert torch.equal(a.view(torch.int16), b.view(torch.int16))
+
+
 def test_per_tensor_layer(L, dev):
     from phyai_amd.quant import Fp8Spec, Granularity
 
