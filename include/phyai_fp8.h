@@ -60,8 +60,9 @@ enum {
  * displace other data from the 256 MB Infinity Cache.  A model whose weights exceed that cache and
  * are re-read every step (the action expert: 311 MB per denoise step, ten steps per inference)
  * gets no cache hits at all when everything is cached alike; marking the largest matrices lets
- * the rest stay resident (phyai_amd/cache_plan.py picks them).  Honoured by the small-M kernel
- * (M <= 64, K % 128 == 0), ignored elsewhere; results are bit-identical with and without it.  The
+ * the rest stay resident (phyai_amd/cache_plan.py picks them).  Honoured by the weight-streaming
+ * kernel (what phyai_fp8_describe_plan reports as "small-m"), ignored by the tile kernels, whose
+ * workgroups share weight rows through L2; results are bit-identical with and without it.  The
  * reference has no counterpart (its GEMM is a library call, linear/backends/torch.py:168-175).
  */
 #define PHYAI_FP8_EPILOGUE_MASK 0xFF

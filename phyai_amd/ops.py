@@ -361,7 +361,7 @@ def fp8_gemm(xq: torch.Tensor, x_scale: torch.Tensor, weight: torch.Tensor, weig
     """``bf16(act((xq @ weight.T) * x_scale * weight_scale + bias))`` on quantized inputs.
 
     ``stream_weights``: read the weights past the caches (see :mod:`phyai_amd.cache_plan`);
-    same result, honoured at small M without a gated residual.
+    same result, honoured by the weight-streaming kernel (small M) without a gated residual.
 
     With ``residual`` and ``gate`` the result is ``torch.addcmul(residual, y, gate)`` of that
     linear output ``y`` (reference ``models/pi05/modeling_pi05.py:826,835``), in the same kernel;
