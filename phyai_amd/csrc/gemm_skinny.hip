@@ -320,16 +320,21 @@ __global__ __launch_bounds__(SK_THREADS) void gemm_fp8_skinny_kernel(
     __syncthreads();
 #pragma unroll
     for (int rr = 0; rr < ROLE_ROUNDS; ++rr) {
-        if (!e_role[rr]) continue;
+        if (e_nt[rr] >= NT) continue;   // wavefront-uniform: this wavefront has no block in this round
         v4f g = red(0, e_nt[rr], e_mb[rr], e_lane);
 #pragma unroll
         for (int w = 1; w < SK_WAVES; ++w) g += red(w, e_nt[rr], e_mb[rr], e_lane);
         v4f u = v4f{0.f, 0.f, 0.f, 0.f};
         if constexpr (GATED) {
-            u = red(0, e_nt[rr], e_mb[rr], e_lane + 32);
+            // The up half of a gated tile sits 32 lanes further on.  Every lane has just added up its
+            // own slot, so the upper half of the wavefront hands its sums down instead of the lower
+            // half reading eight more partials each.
+            const int from = ((e_lane + 32) & 63) << 2;
 #pragma unroll
-            for (int w = 1; w < SK_WAVES; ++w) u += red(w, e_nt[rr], e_mb[rr], e_lane + 32);
+            for (int r = 0; r < 4; ++r)
+                u[r] = __uint_as_float((uint32_t)__builtin_amdgcn_ds_bpermute(from, (int)__float_as_uint(g[r])));
         }
+        if (!e_role[rr]) continue;
 
         // ---- 4. epilogue --------------------------------------------------------------------
         const float bwf[4] = {bf16_bits_to_f32(bw2[rr].x & 0xFFFFu), bf16_bits_to_f32(bw2[rr].x >> 16),
