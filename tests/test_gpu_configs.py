@@ -99,13 +99,25 @@ def test_config3_prefill_m816(dev, name, N, K, epi):
     check_case(dev, 816, N, K, epi, seed=300 + N + K)
 
 
+# q, k and v as the benchmark definition lists them: three projections instead of the reference's
+# fused qkv (layers/linear/layers.py:447-449).  k / v have a single KV head: N = 256.
+@pytest.mark.parametrize("name,N", [("q", 2048), ("k", 256), ("v", 256)])
+def test_config2_expert_separate_qkv_m50(dev, name, N):
+    check_case(dev, 50, N, 1024, None, seed=250 + N + ord(name))
+
+
+@pytest.mark.parametrize("name,N", [("q", 2048), ("k", 256), ("v", 256)])
+def test_config3_prefill_separate_qkv_m816(dev, name, N):
+    check_case(dev, 816, N, 2048, None, seed=350 + N + ord(name))
+
+
 @pytest.mark.parametrize("B", [2, 4, 8, 16])
 @pytest.mark.parametrize("name,N,K,epi", EXPERT)
 def test_config4_expert_batched(dev, B, name, N, K, epi):
     check_case(dev, 50 * B, N, K, epi, seed=400 + B + N, outliers=True)
 
 
-@pytest.mark.parametrize("B", [2, 16])
+@pytest.mark.parametrize("B", [2, 4, 8, 16])
 @pytest.mark.parametrize("name,N,K,epi", PREFILL)
 def test_config4_prefill_batched(dev, B, name, N, K, epi):
     check_case(dev, 816 * B, N, K, epi, seed=500 + B + N, outliers=True, nrows=128, ncols=64)
