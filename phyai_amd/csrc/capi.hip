@@ -130,18 +130,24 @@ int check_residual(const char* fn, const ResidualSpec& r, int64_t M, int64_t N, 
     return 0;
 }
 
-int run_gemm(const char* fn, const void* xq, const float* x_scale, int x_scale_is_scalar, const void* w,
-             const float* w_scale, const void* bias, const ResidualSpec& res, void* out, int64_t ldo, int64_t M,
-             int64_t N, int64_t K, int epilogue, void* workspace, size_t workspace_bytes, void* stream) {
+// Validates a GEMM call and fills in the problem; nothing is launched.  `flagged_epilogue` may carry
+// PHYAI_FP8_FLAG_* bits.  Returns 0, or a status after fail().
+int prepare_gemm(const char* fn, const void* xq, const float* x_scale, int x_scale_is_scalar, const void* w,
+                 const float* w_scale, const void* bias, const ResidualSpec& res, void* out, int64_t ldo, int64_t M,
+                 int64_t N, int64_t K, int flagged_epilogue, void* workspace, size_t workspace_bytes,
+                 phyai::GemmProblem* problem) {
     if (M < 0 || N <= 0 || K <= 0)
         return fail(PHYAI_FP8_EINVAL, "%s: bad shape M=%lld N=%lld K=%lld", fn, (long long)M, (long long)N, (long long)K);
-    const int flags = epilogue & ~PHYAI_FP8_EPILOGUE_MASK;
-    epilogue &= PHYAI_FP8_EPILOGUE_MASK;
+    const int flags = flagged_epilogue & ~PHYAI_FP8_EPILOGUE_MASK;
+    const int epilogue = flagged_epilogue & PHYAI_FP8_EPILOGUE_MASK;
     if (flags & ~PHYAI_FP8_FLAG_STREAM_WEIGHTS) return fail(PHYAI_FP8_EINVAL, "%s: unknown flag bits 0x%x", fn, flags);
     if (int rc = check_epilogue(epilogue, N)) return rc;
     if (K % 16 != 0 || N % 16 != 0)
         return fail(PHYAI_FP8_EUNSUPPORTED, "%s: K=%lld and N=%lld must be multiples of 16", fn, (long long)K, (long long)N);
     if (int rc = check_residual(fn, res, M, N, epilogue)) return rc;
+    phyai::GemmProblem g = {};
+    g.M = (int)M; g.N = (int)N; g.K = (int)K;
+    *problem = g;
     if (M == 0) return PHYAI_FP8_OK;
     if (!xq || !x_scale || !w || !w_scale || !out) return fail(PHYAI_FP8_EINVAL, "%s: null pointer", fn);
     if (!aligned(xq, 16) || !aligned(w, 16)) return fail(PHYAI_FP8_EINVAL, "%s: xq and w must be 16-byte aligned", fn);
@@ -151,7 +157,6 @@ int run_gemm(const char* fn, const void* xq, const float* x_scale, int x_scale_i
         return fail(PHYAI_FP8_EUNSUPPORTED, "%s: operand larger than 2^31 elements", fn);
     if (workspace && !aligned(workspace, 256)) return fail(PHYAI_FP8_EINVAL, "%s: workspace must be 256-byte aligned", fn);
 
-    phyai::GemmProblem g = {};
     g.xq = static_cast<const uint8_t*>(xq);
     g.x_scale = x_scale;
     g.x_scale_is_scalar = x_scale_is_scalar ? 1 : 0;
@@ -160,7 +165,6 @@ int run_gemm(const char* fn, const void* xq, const float* x_scale, int x_scale_i
     g.bias = static_cast<const uint16_t*>(bias);
     g.out = static_cast<uint16_t*>(out);
     g.ldo = ldo;
-    g.M = (int)M; g.N = (int)N; g.K = (int)K;
     g.epilogue = epilogue;
     g.stream_weights = (flags & PHYAI_FP8_FLAG_STREAM_WEIGHTS) ? 1 : 0;
     g.workspace = workspace;
@@ -173,12 +177,45 @@ int run_gemm(const char* fn, const void* xq, const float* x_scale, int x_scale_i
         g.ld_gate = res.ld_gate;
         g.gate_group = (int)(M / res.gate_rows);
     }
-    const int rc = phyai::launch_gemm(g, static_cast<hipStream_t>(stream));
-    if (rc == -3)
+    const size_t need = phyai::gemm_scratch_need(g);
+    if (need > 0 && (workspace == nullptr || workspace_bytes < need))
         return fail(PHYAI_FP8_EWORKSPACE, "%s: workspace of %zu bytes is too small, need %zu", fn,
-                    workspace ? workspace_bytes : (size_t)0, phyai::gemm_workspace_bytes(M, N, K, epilogue, ldo));
+                    workspace ? workspace_bytes : (size_t)0, need);
+    *problem = g;
+    return PHYAI_FP8_OK;
+}
+
+int launch_prepared(const char* fn, const phyai::GemmProblem& g, void* stream) {
+    if (g.M == 0) return PHYAI_FP8_OK;
+    const int rc = phyai::launch_gemm(g, static_cast<hipStream_t>(stream));
+    if (rc == -3) return fail(PHYAI_FP8_EWORKSPACE, "%s: workspace too small for the chosen kernel", fn);
     if (rc != 0) return fail(PHYAI_FP8_EUNSUPPORTED, "%s: no kernel for this problem (rc=%d)", fn, rc);
     return check_launch(fn);
+}
+
+int run_gemm(const char* fn, const void* xq, const float* x_scale, int x_scale_is_scalar, const void* w,
+             const float* w_scale, const void* bias, const ResidualSpec& res, void* out, int64_t ldo, int64_t M,
+             int64_t N, int64_t K, int epilogue, void* workspace, size_t workspace_bytes, void* stream) {
+    phyai::GemmProblem g;
+    if (int rc = prepare_gemm(fn, xq, x_scale, x_scale_is_scalar, w, w_scale, bias, res, out, ldo, M, N, K, epilogue,
+                              workspace, workspace_bytes, &g))
+        return rc;
+    return launch_prepared(fn, g, stream);
+}
+
+// Quantizer + GEMM with the codes and scales staged at xq / xs and the GEMM's own scratch at
+// gemm_ws.  Every argument of both launches is checked before the first one is enqueued.
+int run_linear_at(const char* fn, const void* x, int64_t ldx, const void* w, const float* w_scale, const void* bias,
+                  const ResidualSpec& res, void* out, int64_t ldo, int64_t M, int64_t N, int64_t K, int epilogue,
+                  void* xq, float* xs, void* gemm_ws, size_t gemm_ws_bytes, void* stream) {
+    if (int rc = check_quant_args(fn, x, M, K, ldx, xq)) return rc;
+    phyai::GemmProblem g;
+    if (int rc = prepare_gemm(fn, xq, xs, 0, w, w_scale, bias, res, out, ldo, M, N, K, epilogue, gemm_ws,
+                              gemm_ws_bytes, &g))
+        return rc;
+    phyai::launch_quant_rowwise(x, M, K, ldx, xq, xs, static_cast<hipStream_t>(stream));
+    if (int rc = check_launch(fn)) return rc;
+    return launch_prepared(fn, g, stream);
 }
 
 int run_linear(const char* fn, const void* x, int64_t ldx, const void* w, const float* w_scale, const void* bias,
@@ -193,10 +230,8 @@ int run_linear(const char* fn, const void* x, int64_t ldx, const void* w, const 
                     workspace ? workspace_bytes : (size_t)0, c.total);
     if (!aligned(workspace, 256)) return fail(PHYAI_FP8_EINVAL, "%s: workspace must be 256-byte aligned", fn);
     uint8_t* ws = static_cast<uint8_t*>(workspace);
-    void* xq = ws + c.xq_off;
-    float* xs = reinterpret_cast<float*>(ws + c.xs_off);
-    if (int rc = phyai_fp8_quant_rowwise(x, M, K, ldx, xq, xs, stream)) return rc;
-    return run_gemm(fn, xq, xs, 0, w, w_scale, bias, res, out, ldo, M, N, K, epilogue, workspace, c.gemm_bytes, stream);
+    return run_linear_at(fn, x, ldx, w, w_scale, bias, res, out, ldo, M, N, K, epilogue, ws + c.xq_off,
+                         reinterpret_cast<float*>(ws + c.xs_off), workspace, c.gemm_bytes, stream);
 }
 }  // namespace
 

@@ -44,6 +44,7 @@
 // ring).
 #include "fp8_device.h"
 #include "launch.h"
+#include "tuning.h"
 #include "splitk.h"
 #include <stdlib.h>
 
@@ -513,7 +514,7 @@ BigPlan big_plan(int M, int N, int K, int epilogue) {
     BigPlan pl = {0, 1, 0, 0};
     if (K % 128 != 0 || K < 512) return pl;   // slabs come in pairs and must fill the ring
     int forced = -1;
-    if (const char* e = getenv("PHYAI_FP8_BIG")) forced = atoi(e);   // "0": never; "256"/"192"/"128": force
+    if (const char* e = tuning_env("PHYAI_FP8_BIG")) forced = atoi(e);   // "0": never; "256"/"192"/"128": force
     if (forced == 0) return pl;
     if (forced == 256 || forced == 192 || forced == 128) pl.tile = forced;
     else if (M < 128) return pl;
@@ -549,11 +550,11 @@ BigPlan big_plan(int M, int N, int K, int epilogue) {
         // (1632 x 2048 x 2048, 208 tiles: 14.2 against 17.3 us).
         else if (tiles > 256) pl.depth = 2;
     }
-    if (const char* e = getenv("PHYAI_FP8_BIG_SPLITS")) {
+    if (const char* e = tuning_env("PHYAI_FP8_BIG_SPLITS")) {
         const int s = atoi(e);
         if (pl.tile != 192 && s >= 1 && K % (s * 128) == 0 && K / s >= 512 && tiles * s <= 4096) pl.splits = s;
     }
-    if (const char* e = getenv("PHYAI_FP8_BIG_DEPTH")) {
+    if (const char* e = tuning_env("PHYAI_FP8_BIG_DEPTH")) {
         const int d = atoi(e);
         if (pl.tile == 128 && pl.splits == 1 && (d == 2 || d == 4)) pl.depth = d;
     }
@@ -591,13 +592,13 @@ static void big_launch(BigArgs a, const GemmProblem& g, int splits, hipStream_t 
         const int rounds_c = big_ceil_div(big_max_tiles_per_xcd(a.m_tiles, a.n_tiles, 4), slots);
         const int rounds_r = big_ceil_div(big_max_tiles_per_xcd(a.n_tiles, a.m_tiles, 4), slots);
         if (rounds_c != rounds_r) a.by_rows = rounds_r < rounds_c;
-        if (const char* e = getenv("PHYAI_FP8_BY_ROWS")) a.by_rows = atoi(e) != 0;
+        if (const char* e = tuning_env("PHYAI_FP8_BY_ROWS")) a.by_rows = atoi(e) != 0;
     }
     // bands of 4 tile rows; a grid of up to 8 tile rows whose activation rows still fit an XCD's
     // L2 beside the weight stream is one band, so that the weights come from HBM once
     a.band = 4;
     if (!a.by_rows && a.m_tiles <= 8 && (int64_t)a.m_tiles * (64 * TM) * (g.K < 4096 ? g.K : 4096) <= (5 << 19)) a.band = a.m_tiles;
-    if (const char* e = getenv("PHYAI_FP8_BAND")) { const int b = atoi(e); if (b >= 1 && b <= 16) a.band = b; }
+    if (const char* e = tuning_env("PHYAI_FP8_BAND")) { const int b = atoi(e); if (b >= 1 && b <= 16) a.band = b; }
     const int outer = a.by_rows ? a.n_tiles : a.m_tiles, inner = a.by_rows ? a.m_tiles : a.n_tiles;
     const dim3 grid(big_grid_ids(outer, inner, a.band), 1, splits);
 #define PHYAI_BIG_ARGS a.a, a.b, a.K, a.M, a.N, a.m_tiles, a.n_tiles, a.band, a.by_rows, a.k_per_split, a.a_scale, \
@@ -625,7 +626,7 @@ static int big_launch_epi(const BigArgs& a, const GemmProblem& g, int splits, hi
 }
 
 int launch_gemm_big(const GemmProblem& g, const BigPlan& pl, hipStream_t st) {
-    // the epilogue writes 16 bytes per lane
+    // the epilogue writes 16 bytes per lane (the caller chooses this kernel only for such outputs)
     if (g.ldo % 8 != 0 || (reinterpret_cast<uintptr_t>(g.out) & 15) != 0) return -2;
     BigArgs a;
     a.a = g.xq; a.b = g.w; a.a_scale = g.x_scale; a.b_scale = g.w_scale; a.bias = g.bias;

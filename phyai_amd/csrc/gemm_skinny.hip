@@ -34,6 +34,7 @@
 //    token: scale, bias, activation, one 64-bit bf16x4 store.
 #include "fp8_device.h"
 #include "launch.h"
+#include "tuning.h"
 #include <stdio.h>
 #include <stdlib.h>
 
@@ -375,7 +376,7 @@ static int sk_ceil_div(int a, int b) { return (a + b - 1) / b; }
 // their grid is large enough (see launch_gemm) and falls back to this kernel up to here
 // (N = 1024: ahead of the 128 x 128 tile kernel up to M = 1000, 11.0 against 17.5 us at 800 x 1024 x 4096).
 static int skinny_max_m() {
-    if (const char* e = getenv("PHYAI_FP8_SKINNY_MAXM")) return atoi(e);
+    if (const char* e = tuning_env("PHYAI_FP8_SKINNY_MAXM")) return atoi(e);
     return 1024;
 }
 
@@ -424,7 +425,7 @@ SkinnyPlan skinny_plan(int M, int N, int K, int epilogue) {
         pl.tiles = sk_ceil_div(cols, per_tile * pl.nt);
         pl.msplit = sk_ceil_div(blocks, pl.mb);
     }
-    if (const char* e = getenv("PHYAI_FP8_SKINNY_PLAN")) {  // "nt,mb" tuning override
+    if (const char* e = tuning_env("PHYAI_FP8_SKINNY_PLAN")) {  // "nt,mb" tuning override
         int nt = 0, mb = 0;
         if (sscanf(e, "%d,%d", &nt, &mb) == 2 && (nt == 1 || nt == 2 || (nt == 4 && mb >= 3)) && mb >= 1 && mb <= 4) {
             pl.nt = nt; pl.tiles = sk_ceil_div(cols, per_tile * nt); pl.mb = mb; pl.msplit = sk_ceil_div(blocks, mb);
@@ -441,7 +442,7 @@ SkinnyPlan skinny_plan(int M, int N, int K, int epilogue) {
 template <int MB, int NT, int KPW, int EPI>
 static void sk_launch_one(const SkinnyArgs& a, const dim3& grid, hipStream_t st) {
     constexpr bool fits = SK_WAVES * KPW * (NT + MB) * 2048 <= 160 * 1024;
-    static const bool want = []() { const char* e = getenv("PHYAI_FP8_SKINNY_STAGED"); return !(e && atoi(e) == 0); }();
+    static const bool want = []() { const char* e = tuning_env("PHYAI_FP8_SKINNY_STAGED"); return !(e && atoi(e) == 0); }();
     if constexpr (fits) {
         if (want && a.K * (int64_t)(a.N > a.M ? a.N : a.M) < ((int64_t)1 << 32) && a.K < (1 << 24) && a.N < (1 << 24)) {
             hipLaunchKernelGGL((gemm_fp8_skinny_kernel<MB, NT, KPW, EPI, true>), grid, dim3(SK_THREADS), 0, st,

@@ -25,6 +25,7 @@
 // counter, which keeps the workspace header zero between calls.
 #include "fp8_device.h"
 #include "launch.h"
+#include "tuning.h"
 #include "splitk.h"
 #include <stdio.h>
 #include <stdlib.h>
@@ -272,7 +273,7 @@ static TileConfig pick_config(int M, int N, int K, int epilogue) {
         c.bn = 128;
     }
     int forced_splits = 0;
-    if (const char* e = getenv("PHYAI_FP8_TILE")) {  // "bm,bn,splits" tuning override
+    if (const char* e = tuning_env("PHYAI_FP8_TILE")) {  // "bm,bn,splits" tuning override
         int bm = 0, bn = 0, sp = 0;
         if (sscanf(e, "%d,%d,%d", &bm, &bn, &sp) == 3 && (bm == 64 || bm == 128 || bm == 256) &&
             (bn == 64 || bn == 128 || bn == 256) && !(bm == 64 && bn == 256) && !(bm == 256 && bn == 64) &&
@@ -290,9 +291,9 @@ static TileConfig pick_config(int M, int N, int K, int epilogue) {
         const int max_s = slabs / 2 > 0 ? slabs / 2 : 1;  // at least 2 slabs per split
         if (s > max_s) s = max_s;
         if (s > 32) s = 32;
-        if (tiles > 4096) s = 1;
     }
     if (forced_splits > 0) s = forced_splits < slabs ? forced_splits : slabs;
+    if (tiles > (int)(kGemmHeaderBytes / sizeof(int))) s = 1;   // one arrival counter per tile in the header
     // every split must own at least one slab
     const int per = ceil_div(slabs, s);
     s = ceil_div(slabs, per);
@@ -347,58 +348,91 @@ static int launch_epi(const TileArgs& a, const TileConfig& c, dim3 grid, hipStre
     }
 }
 
-int describe_gemm_plan(int M, int N, int K, int epilogue, char* buf, size_t n) {
-    // mirrors launch_gemm below for operands that satisfy every alignment requirement
-    const int64_t ldo = epi_is_gated(epilogue) ? N / 2 : N;
-    const bool skinny_ok = skinny_applicable(M, N, K, epilogue, ldo);
+// launch_gemm's choice of kernel for one problem, and the scratch that choice needs.
+struct GemmChoice {
+    enum Kind { SKINNY, BIG, GENERIC } kind;
+    SkinnyPlan sk;
+    BigPlan big;
+    TileConfig tc;
+    size_t need;   // workspace bytes (header + split-K partial sums), 0 if the kernel uses none
+};
+
+// Kernel choice (measured on the expert and prefill shapes, M = 50 .. 13056):
+//   M <= 64                      weight-streaming kernel, nothing else comes close;
+//   pipelined tile kernel        when big_plan finds a tile shape that fills the chip, or more
+//                                than 64 tiles of 128 x 128;
+//   64 < M <= 1024 otherwise     weight-streaming kernel again (few output columns: at
+//                                N = 1024 it wins up to M = 1000, at N = 2560 up to M = 300);
+//   32 .. 64 small tiles         pipelined tile kernel after all (M > 1024);
+//   the rest                     generic LDS tile kernel (any K, any alignment).
+// vec_ok: scales, bias and output are aligned for the weight-streaming kernel's 128- and 64-bit
+// accesses; out16: the output is 16-byte addressable (pointer and row stride), which the pipelined
+// tile kernel's epilogue needs.
+static GemmChoice choose_gemm(int M, int N, int K, int epilogue, int64_t ldo, bool vec_ok, bool out16) {
+    GemmChoice c = {};
+    const bool skinny_ok = vec_ok && skinny_applicable(M, N, K, epilogue, ldo);
     auto small = [&]() {
-        const SkinnyPlan pl = skinny_plan(M, N, K, epilogue);
-        return snprintf(buf, n, "small-m nt=%d mb=%d kpw=%d rounds=%d", pl.nt, pl.mb, pl.kpw, pl.rounds);
+        c.kind = GemmChoice::SKINNY;
+        c.sk = skinny_plan(M, N, K, epilogue);
+        c.need = 0;
+        return c;
     };
     if (skinny_ok && M <= 64) return small();
-    if (!getenv("PHYAI_FP8_TILE")) {
+    if (!tuning_env("PHYAI_FP8_TILE")) {
         const BigPlan bp = big_plan(M, N, K, epilogue);
-        const bool few_small_tiles = bp.tile == 128 && bp.tiles <= 64 && !getenv("PHYAI_FP8_BIG");
-        if (bp.tile && ldo % 8 == 0 && !(few_small_tiles && skinny_ok))
-            return snprintf(buf, n, "tile %dx%d depth=%d splits=%d tiles=%d", bp.tile, bp.tile == 256 ? 256 : 128,
-                            bp.depth, bp.splits, bp.tiles);
+        const bool few_small_tiles = bp.tile == 128 && bp.tiles <= 64 && !tuning_env("PHYAI_FP8_BIG");
+        if (bp.tile && out16 && !(few_small_tiles && skinny_ok)) {
+            c.kind = GemmChoice::BIG;
+            c.big = bp;
+            c.need = bp.splits > 1 ? kHeaderBytes + big_partial_bytes(M, N, epilogue, bp) : 0;
+            return c;
+        }
         if (skinny_ok) return small();
     }
-    const TileConfig c = pick_config(M, N, K, epilogue);
-    return snprintf(buf, n, "generic %dx%d splits=%d", c.bm, c.bn, c.splits);
+    c.kind = GemmChoice::GENERIC;
+    c.tc = pick_config(M, N, K, epilogue);
+    c.need = c.tc.splits > 1 ? kHeaderBytes + partial_bytes(c.tc, M, N, epilogue) : 0;
+    return c;
+}
+
+static GemmChoice choose_gemm(const GemmProblem& g) {
+    const bool vec_ok = (reinterpret_cast<uintptr_t>(g.w_scale) % 16 == 0) &&
+                        (reinterpret_cast<uintptr_t>(g.bias) % 8 == 0) &&
+                        (reinterpret_cast<uintptr_t>(g.out) % 8 == 0);
+    const bool out16 = g.ldo % 8 == 0 && (reinterpret_cast<uintptr_t>(g.out) & 15) == 0;
+    return choose_gemm(g.M, g.N, g.K, g.epilogue, g.ldo, vec_ok, out16);
+}
+
+size_t gemm_scratch_need(const GemmProblem& g) {
+    if (g.M == 0 || g.N == 0) return 0;
+    return choose_gemm(g).need;
+}
+
+int describe_gemm_plan(int M, int N, int K, int epilogue, char* buf, size_t n) {
+    // operands that satisfy every alignment requirement, dense output
+    const int64_t ldo = epi_is_gated(epilogue) ? N / 2 : N;
+    const GemmChoice c = choose_gemm(M, N, K, epilogue, ldo, true, ldo % 8 == 0);
+    switch (c.kind) {
+    case GemmChoice::SKINNY:
+        return snprintf(buf, n, "small-m nt=%d mb=%d kpw=%d rounds=%d", c.sk.nt, c.sk.mb, c.sk.kpw, c.sk.rounds);
+    case GemmChoice::BIG:
+        return snprintf(buf, n, "tile %dx%d depth=%d splits=%d tiles=%d", c.big.tile, c.big.tile == 256 ? 256 : 128,
+                        c.big.depth, c.big.splits, c.big.tiles);
+    default:
+        return snprintf(buf, n, "generic %dx%d splits=%d", c.tc.bm, c.tc.bn, c.tc.splits);
+    }
 }
 
 int launch_gemm(const GemmProblem& g, hipStream_t st) {
     if (g.M == 0 || g.N == 0) return 0;
-    // Kernel choice (measured on the expert and prefill shapes, M = 50 .. 13056):
-    //   M <= 64                      weight-streaming kernel, nothing else comes close;
-    //   pipelined tile kernel        when big_plan finds a tile shape that fills the chip, or more
-    //                                than 64 tiles of 128 x 128;
-    //   64 < M <= 1024 otherwise     weight-streaming kernel again (few output columns: at
-    //                                N = 1024 it wins up to M = 1000, at N = 2560 up to M = 300);
-    //   32 .. 64 small tiles         pipelined tile kernel after all (M > 1024);
-    //   the rest                     generic LDS tile kernel (any K, any alignment).
-    // The weight-streaming kernel reads scales / bias / output with 128- and 64-bit accesses.
-    const bool vec_ok = (reinterpret_cast<uintptr_t>(g.w_scale) % 16 == 0) &&
-                        (reinterpret_cast<uintptr_t>(g.bias) % 8 == 0) &&
-                        (reinterpret_cast<uintptr_t>(g.out) % 8 == 0);
-    const bool skinny_ok = vec_ok && skinny_applicable(g.M, g.N, g.K, g.epilogue, g.ldo);
-    if (skinny_ok && g.M <= 64) return launch_gemm_skinny(g, skinny_plan(g.M, g.N, g.K, g.epilogue), st);
-    if (!getenv("PHYAI_FP8_TILE")) {
-        const BigPlan bp = big_plan(g.M, g.N, g.K, g.epilogue);
-        const bool few_small_tiles = bp.tile == 128 && bp.tiles <= 64 && !getenv("PHYAI_FP8_BIG");
-        if (bp.tile && !(few_small_tiles && skinny_ok)) {
-            const int rc = launch_gemm_big(g, bp, st);
-            if (rc != -2) return rc;  // -2: output not 16-byte addressable, try the others
-        }
-        if (skinny_ok) return launch_gemm_skinny(g, skinny_plan(g.M, g.N, g.K, g.epilogue), st);
-    }
-    const TileConfig c = pick_config(g.M, g.N, g.K, g.epilogue);
+    const GemmChoice ch = choose_gemm(g);
+    if (ch.need > 0 && (g.workspace == nullptr || g.workspace_bytes < ch.need)) return -3;
+    if (ch.kind == GemmChoice::SKINNY) return launch_gemm_skinny(g, ch.sk, st);
+    if (ch.kind == GemmChoice::BIG) return launch_gemm_big(g, ch.big, st);
+    const TileConfig& c = ch.tc;
     const bool gated = epi_is_gated(g.epilogue);
     const int n_eff = gated ? g.N / 2 : g.N;
     const int bn_eff = gated ? c.bn / 2 : c.bn;
-    const size_t need = kHeaderBytes + partial_bytes(c, g.M, g.N, g.epilogue);
-    if (c.splits > 1 && (g.workspace == nullptr || g.workspace_bytes < need)) return -3;
 
     TileArgs a;
     a.a = g.xq; a.b = g.w; a.a_scale = g.x_scale; a.b_scale = g.w_scale; a.bias = g.bias;

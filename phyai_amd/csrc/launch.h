@@ -76,6 +76,9 @@ inline ResidualArgs residual_of(const GemmProblem& g) {
 constexpr size_t kGemmHeaderBytes = 16384;  // split-K arrival counters (4096 ints) at the workspace start
 
 size_t gemm_workspace_bytes(int64_t M, int64_t N, int64_t K, int epilogue, int64_t ldo);
+// Workspace bytes the kernel chosen for exactly this problem (pointers and strides as given) needs:
+// 0 when it uses none, else header + split-K partial sums.  launch_gemm returns -3 with less.
+size_t gemm_scratch_need(const GemmProblem& p);
 int launch_gemm(const GemmProblem& p, hipStream_t st);
 
 // Weight-streaming kernel for M <= 64 (gemm_skinny.hip).  It needs no workspace.

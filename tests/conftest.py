@@ -12,6 +12,10 @@ ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
 if ROOT not in sys.path:
     sys.path.insert(0, ROOT)
 
+# The library looks at its PHYAI_FP8_* tuning variables only when this switch was set before its
+# first call; the tests that force kernel variants need it.
+os.environ.setdefault("PHYAI_FP8_TUNING", "1")
+
 
 def pytest_configure(config):
     config.addinivalue_line("markers", "gpu: needs a real MI355X (run with -m gpu)")

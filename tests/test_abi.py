@@ -112,6 +112,26 @@ def test_kernel_selection_for_the_benchmark_shapes(monkeypatch):
         d(50, 1000, 1024)
 
 
+def test_tuning_variables_are_ignored_without_the_switch():
+    """A stray PHYAI_FP8_* variable must not change the kernel selection of a process that did not
+    set PHYAI_FP8_TUNING (fresh processes: the switch is read once)."""
+    import subprocess
+    import sys
+
+    code = ("from phyai_amd import ops; print(ops.describe_plan(816, 32768, 2048, 'geglu_tanh')); "
+            "print(ops.describe_plan(50, 2560, 1024))")
+    want = "tile 256x256 depth=2 splits=1 tiles=512\nsmall-m nt=2 mb=2 kpw=1 rounds=1\n"
+    env = {k: v for k, v in os.environ.items() if not k.startswith("PHYAI_FP8_")}
+    env.update(PHYAI_FP8_BIG="128", PHYAI_FP8_SKINNY_PLAN="1,4", PHYAI_FP8_TILE="128,128,2", PYTHONPATH=ROOT)
+    out = subprocess.run([sys.executable, "-c", code], env=env, capture_output=True, text=True, timeout=300)
+    assert out.returncode == 0, out.stderr
+    assert out.stdout == want
+    env["PHYAI_FP8_TUNING"] = "1"
+    out = subprocess.run([sys.executable, "-c", code], env=env, capture_output=True, text=True, timeout=300)
+    assert out.returncode == 0, out.stderr
+    assert out.stdout != want
+
+
 C_CLIENT = r"""
 #include <stdio.h>
 #include <string.h>
