@@ -31,7 +31,7 @@
 extern "C" {
 #endif
 
-#define PHYAI_FP8_ABI_VERSION 4
+#define PHYAI_FP8_ABI_VERSION 5
 
 enum {
     PHYAI_FP8_OK = 0,
@@ -154,6 +154,25 @@ int phyai_fp8_linear_addcmul(const void *x, int64_t ldx, const void *w, const fl
                              const void *gate, int64_t ld_gate, int64_t gate_rows, void *out,
                              int64_t ldo, int64_t M, int64_t N, int64_t K, void *workspace,
                              size_t workspace_bytes, void *stream);
+
+/*
+ * phyai_fp8_linear for callers that cannot allocate device memory or hand over a workspace: code
+ * under HIP graph capture, tight serving loops, harnesses that forbid hipMalloc.  No counterpart
+ * in the reference (its linear returns a tensor from torch's caching allocator,
+ * layers/linear/backends/torch.py:168-176).  Same kernels and same results as phyai_fp8_linear;
+ * the scratch (activation codes, per-token scales, split-K counters and partial sums) lives in a
+ * device array of PHYAI_FP8_STATIC_SCRATCH_BYTES that is part of the library's code object: every
+ * GPU the library runs on holds one until the process ends.  The call allocates nothing and frees
+ * nothing.  A shape whose phyai_fp8_linear_workspace_bytes() exceeds the array is refused with
+ * PHYAI_FP8_EWORKSPACE.  All calls on one GPU share that GPU's array: calls that may overlap there
+ * (two streams, two threads) race; serialise them or use phyai_fp8_linear with one workspace
+ * each.  The first call on a device looks the array's address up (hipGetSymbolAddress); make it
+ * outside graph capture, e.g. in the warm-up runs.
+ */
+#define PHYAI_FP8_STATIC_SCRATCH_BYTES (32 * 1024 * 1024)
+int phyai_fp8_linear_static(const void *x, int64_t ldx, const void *w, const float *w_scale,
+                            const void *bias, void *out, int64_t ldo, int64_t M, int64_t N,
+                            int64_t K, int epilogue, void *stream);
 
 /*
  * RMSNorm whose output feeds the quantizer without a round trip through memory.

@@ -4,9 +4,16 @@
 #include <stdarg.h>
 #include <stdio.h>
 
+#include <mutex>
+
 #include "../../include/phyai_fp8.h"
 #include "fp8_device.h"
 #include "launch.h"
+
+// Scratch of phyai_fp8_linear_static: one array per GPU, part of the loaded code object (zero when
+// the module is loaded), held until the process ends.  The name is only a handle on the host; the
+// array's device address comes from hipGetSymbolAddress, per device (static_scratch_of below).
+static __device__ __align__(256) uint8_t scratch[PHYAI_FP8_STATIC_SCRATCH_BYTES];
 
 namespace {
 
@@ -68,6 +75,36 @@ int check_quant_args(const char* fn, const void* x, int64_t M, int64_t K, int64_
     if (!aligned(x, 16) || !aligned(xq, 8)) return fail(PHYAI_FP8_EINVAL, "%s: x must be 16-byte and xq 8-byte aligned", fn);
     if (M * ldx >= kMaxElems * 4 || M >= kMaxElems) return fail(PHYAI_FP8_EUNSUPPORTED, "%s: tensor too large", fn);
     return 0;
+}
+
+constexpr int kMaxDevices = 64;
+std::mutex g_scratch_mutex;
+void* g_scratch_ptr[kMaxDevices] = {};
+
+// Device address of `scratch` on the current device: looked up once per device, with that device
+// current, and kept (every GPU holds its own copy of the array at its own address).
+int static_scratch_of(void** ptr) {
+    int dev = -1;
+    hipError_t e = hipGetDevice(&dev);
+    if (e != hipSuccess) return fail(PHYAI_FP8_ELAUNCH, "phyai_fp8_linear_static: hipGetDevice: %s", hipGetErrorString(e));
+    if (dev < 0 || dev >= kMaxDevices) return fail(PHYAI_FP8_EUNSUPPORTED, "phyai_fp8_linear_static: device %d out of range", dev);
+    std::lock_guard<std::mutex> lock(g_scratch_mutex);
+    if (g_scratch_ptr[dev] == nullptr) {
+        void* p = nullptr;
+        e = hipGetSymbolAddress(&p, HIP_SYMBOL(scratch));
+        if (e != hipSuccess || p == nullptr)
+            return fail(PHYAI_FP8_ELAUNCH, "phyai_fp8_linear_static: hipGetSymbolAddress: %s", hipGetErrorString(e));
+        g_scratch_ptr[dev] = p;
+    }
+    *ptr = g_scratch_ptr[dev];
+    return 0;
+}
+
+// Zeroes the split-K arrival counters at the head of a workspace (a kernel, not a memset, so that it
+// can be recorded into a graph).
+__global__ __launch_bounds__(256) void zero_header_kernel(uint32_t* __restrict__ p, int n) {
+    const int i = blockIdx.x * 256 + threadIdx.x;
+    if (i < n) p[i] = 0u;
 }
 
 }  // namespace
@@ -269,6 +306,51 @@ int phyai_fp8_linear_addcmul(const void* x, int64_t ldx, const void* w, const fl
     const ResidualSpec r = {residual, ld_res, gate, ld_gate, gate_rows};
     return run_linear("phyai_fp8_linear_addcmul", x, ldx, w, w_scale, bias, r, out, ldo, M, N, K,
                       PHYAI_FP8_EPI_NONE, workspace, workspace_bytes, stream);
+}
+
+int phyai_fp8_linear_static(const void* x, int64_t ldx, const void* w, const float* w_scale, const void* bias,
+                            void* out, int64_t ldo, int64_t M, int64_t N, int64_t K, int epilogue, void* stream) {
+    const char* fn = "phyai_fp8_linear_static";
+    constexpr size_t kScratch = PHYAI_FP8_STATIC_SCRATCH_BYTES;
+    if (M < 0 || N <= 0 || K <= 0)
+        return fail(PHYAI_FP8_EINVAL, "%s: bad shape M=%lld N=%lld K=%lld", fn, (long long)M, (long long)N, (long long)K);
+    if (M == 0) return PHYAI_FP8_OK;
+    // Layout of the array: [split-K counters | partial sums ...        ... codes | per-token scales].
+    // The GEMM gets whatever the staging at the tail leaves; its need depends on the kernel that
+    // serves exactly this call and is checked before anything is launched.
+    if (M >= kMaxElems || K >= kMaxElems) return fail(PHYAI_FP8_EUNSUPPORTED, "%s: tensor too large", fn);
+    const size_t xs_bytes = align_up((size_t)M * sizeof(float), 256), xq_bytes = align_up((size_t)M * (size_t)K, 256);
+    if (xs_bytes + xq_bytes + PHYAI_FP8_WORKSPACE_HEADER_BYTES > kScratch)
+        return fail(PHYAI_FP8_EWORKSPACE, "%s: the activation codes of this shape need %zu bytes, the static array holds %zu; "
+                    "use phyai_fp8_linear with a caller-owned workspace", fn, xs_bytes + xq_bytes, kScratch);
+    void* base = nullptr;
+    if (int rc = static_scratch_of(&base)) return rc;
+    uint8_t* ws = static_cast<uint8_t*>(base);
+    const size_t xq_off = kScratch - xs_bytes - xq_bytes, gemm_bytes = xq_off;
+    void* xq = ws + xq_off;
+    float* xs = reinterpret_cast<float*>(ws + xq_off + xq_bytes);
+    if (int rc = check_quant_args(fn, x, M, K, ldx, xq)) return rc;
+    phyai::GemmProblem g;
+    if (int rc = prepare_gemm(fn, xq, xs, 0, w, w_scale, bias, ResidualSpec{}, out, ldo, M, N, K, epilogue, ws,
+                              gemm_bytes, &g)) {
+        if (rc == PHYAI_FP8_EWORKSPACE)
+            return fail(rc, "%s: this shape needs more scratch than the static array holds (%zu bytes, %zu of them for "
+                        "activation codes); use phyai_fp8_linear with a caller-owned workspace", fn, kScratch, xs_bytes + xq_bytes);
+        return rc;
+    }
+    const hipStream_t st = static_cast<hipStream_t>(stream);
+    // The array keeps what the last call left.  Codes, scales and partial sums are written before
+    // they are read; the split-K arrival counters must start at zero, and although the kernels put
+    // them back to zero themselves, a call that uses them clears them first (with a kernel, not a
+    // memset, so that the call can be recorded into a graph).
+    if (phyai::gemm_scratch_need(g) > 0) {
+        const int n = PHYAI_FP8_WORKSPACE_HEADER_BYTES / 4;
+        hipLaunchKernelGGL(zero_header_kernel, dim3((n + 255) / 256), dim3(256), 0, st, reinterpret_cast<uint32_t*>(ws), n);
+        if (int rc = check_launch(fn)) return rc;
+    }
+    phyai::launch_quant_rowwise(x, M, K, ldx, xq, xs, st);
+    if (int rc = check_launch(fn)) return rc;
+    return launch_prepared(fn, g, stream);
 }
 
 namespace {
