@@ -12,6 +12,9 @@ be recorded into a HIP graph once their workspace exists (see
 
 from __future__ import annotations
 
+import contextlib
+import contextvars
+
 import torch
 
 from phyai_amd import _lib
@@ -68,9 +71,38 @@ def _as_rows(op: str, x: torch.Tensor, name: str, dtype: torch.dtype) -> torch.T
 
 
 # ---- workspace --------------------------------------------------------------
-# One zero-initialised scratch tensor per (device, stream), grown on demand
-# outside graph capture.  The kernels keep its header zero between calls.
+# Scratch of the GEMM (split-K counters and partial sums) and of the whole-linear entry points
+# (activation codes and per-token scales): zero-initialised byte tensors whose header the kernels
+# keep zero between calls.  Eager calls share one tensor per (device, stream).  A HIP graph bakes
+# the addresses it was recorded with into its kernel nodes, so a graph owns its workspace
+# (`WorkspaceOwner`, entered by `HipGraph.capture` around warm-up and recording): it lives as long
+# as the graph and is shared with nobody - not with eager work that later runs on the pooled
+# stream the graph was recorded on, not with other graphs.  A workspace that has to grow is
+# replaced, never freed while anything may still hold its address: the old tensor stays with its
+# owner (or, for the eager ones, in `_retired` until the process ends).
 _workspaces: dict[tuple[int, int], torch.Tensor] = {}
+_retired: list[torch.Tensor] = []
+
+
+class WorkspaceOwner:
+    """Scratch that lives as long as its owner (one captured graph): device index -> tensor."""
+
+    def __init__(self) -> None:
+        self.tensors: dict[int, torch.Tensor] = {}
+        self.retired: list[torch.Tensor] = []
+
+
+_owner: contextvars.ContextVar[WorkspaceOwner | None] = contextvars.ContextVar("phyai_amd_workspace_owner", default=None)
+
+
+@contextlib.contextmanager
+def workspace_owner(owner: WorkspaceOwner):
+    """Calls inside the scope take their workspace from ``owner`` instead of the per-stream table."""
+    token = _owner.set(owner)
+    try:
+        yield owner
+    finally:
+        _owner.reset(token)
 
 
 def workspace_bytes(M: int, N: int, K: int, epilogue=EPI_NONE) -> int:
@@ -89,20 +121,24 @@ def describe_plan(M: int, N: int, K: int, epilogue=EPI_NONE) -> str:
 
 
 def reserve_workspace(nbytes: int, device: torch.device | None = None) -> torch.Tensor:
-    """Make sure the current stream's workspace on ``device`` holds ``nbytes``."""
+    """Make sure the workspace in scope on ``device`` (the enclosing graph's, else the current
+    stream's) holds ``nbytes``."""
     dev = torch.device("cuda", torch.cuda.current_device()) if device is None else torch.device(device)
     idx = dev.index if dev.index is not None else torch.cuda.current_device()
-    key = (idx, _stream_ptr())
-    ws = _workspaces.get(key)
+    owner = _owner.get()
+    store, key, retired = (owner.tensors, idx, owner.retired) if owner is not None else (_workspaces, (idx, _stream_ptr()), _retired)
+    ws = store.get(key)
     if ws is None or ws.numel() < nbytes:
-        # Outside capture this is a one-off allocation.  Inside a capture (an op met on a
-        # stream that never ran it before) the tensor comes from the graph's memory pool and
-        # the zero fill is recorded as a fill kernel - never a memset node - and replayed
-        # with the graph; warming the op up on the capture stream avoids that extra node.
-        size = max(int(nbytes), 1 << 20)
+        # Outside capture this is a one-off allocation.  Inside a capture (an op met for the first
+        # time while recording) the tensor comes from the graph's memory pool and the zero fill is
+        # recorded as a fill kernel - never a memset node - and replayed with the graph; warming
+        # the op up before recording avoids that extra node.
+        size = max(int(nbytes), 1 << 20, 2 * ws.numel() if ws is not None else 0)
         size = (size + 0xFFFFF) & ~0xFFFFF
+        if ws is not None:
+            retired.append(ws)     # recorded kernels or queued launches may still write through it
         ws = torch.zeros(size, dtype=torch.uint8, device=torch.device("cuda", idx))
-        _workspaces[key] = ws
+        store[key] = ws
     return ws
 
 
@@ -283,8 +319,14 @@ def fp8_weight_quant(w: torch.Tensor, *, out: torch.Tensor | None = None,
         raise _err(op, f"K={K} must be a multiple of 8")
     if out is None:
         out = torch.empty((N, K), dtype=torch.float8_e4m3fn, device=w.device)
+    elif not (isinstance(out, torch.Tensor) and tuple(out.shape) == (N, K) and out.device == w.device
+              and out.dtype in (torch.float8_e4m3fn, torch.uint8) and out.is_contiguous()):
+        raise _err(op, f"out must be a contiguous float8_e4m3fn tensor of shape ({N}, {K}) on {w.device}")
     if scale_out is None:
         scale_out = torch.empty((N,), dtype=torch.float32, device=w.device)
+    elif not (isinstance(scale_out, torch.Tensor) and tuple(scale_out.shape) == (N,) and scale_out.device == w.device
+              and scale_out.dtype == torch.float32 and scale_out.is_contiguous()):
+        raise _err(op, f"scale_out must be a contiguous float32 tensor of shape ({N},) on {w.device}")
     if N == 0:
         return out, scale_out
     rc = _lib.load().phyai_fp8_weight_quant_rowwise(w2.data_ptr(), N, K, w2.stride(0) if N > 1 else K,

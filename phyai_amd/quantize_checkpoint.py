@@ -8,6 +8,13 @@ weight-quantizer kernel), every other tensor unchanged, and ``config.json`` with
 ``quantization_config = {"quant_method": "fp8", "activation_scheme": "dynamic", "ignored_layers":
 [...]}`` - the form ``Fp8Importer`` reads (``quant/importers/fp8.py:14-36``).
 
+Only matrices that the model builds as fp8 linears may be converted: an embedding table, the
+``lm_head`` tied to it, position tables and norm weights are read by modules that have no
+``weight_scale`` and would take the codes for values.  Modules whose name matches
+``DEFAULT_KEEP`` are therefore left alone unless ``--only`` names them explicitly, and everything
+left unquantized is listed in ``ignored_layers``.  A sharded checkpoint's
+``model.safetensors.index.json`` is rewritten with the added ``weight_scale`` keys.
+
     python -m phyai_amd.quantize_checkpoint SRC_DIR DST_DIR [--ignore NAME ...] [--only GLOB ...]
 """
 
@@ -21,16 +28,27 @@ from pathlib import Path
 import torch
 
 
+# Module-name patterns (matched against every dotted component) that are never fp8 linears.
+DEFAULT_KEEP = ("*embed*", "lm_head", "*norm*", "*position*", "*pos_emb*", "wte", "wpe")
+
+
 def _selected(module: str, only: list[str], ignore: list[str]) -> bool:
     if any(module == n or module.split(".")[-1] == n for n in ignore):
         return False
-    return not only or any(fnmatch.fnmatch(module, g) for g in only)
+    if only:
+        return any(fnmatch.fnmatch(module, g) for g in only)
+    return not any(fnmatch.fnmatch(part, pat) for part in module.split(".") for pat in DEFAULT_KEEP)
+
+
+_DTYPE_BYTES = {"F64": 8, "F32": 4, "F16": 2, "BF16": 2, "I64": 8, "I32": 4, "I16": 2, "I8": 1, "U8": 1, "BOOL": 1,
+                "F8_E4M3": 1, "F8_E5M2": 1}
 
 
 def quantize_state(tensors: dict, *, only: list[str] | None = None, ignore: list[str] | None = None,
                    device: torch.device | str = "cuda") -> tuple[dict, list[str]]:
     """``(new tensors, quantized module names)``.  A ``.weight`` is quantized when it is 2-D, bf16 /
-    fp16 / fp32, has K % 16 == 0 and N % 16 == 0 (what the kernels accept) and its module is selected."""
+    fp16 / fp32, has K % 16 == 0 and N % 16 == 0 (what the kernels accept) and its module is selected:
+    named by ``only`` when that is given, otherwise not matching ``DEFAULT_KEEP``; never one in ``ignore``."""
     from phyai_amd import ops
 
     only, ignore = list(only or []), list(ignore or [])
@@ -66,6 +84,26 @@ def quantize_checkpoint(src: str | Path, dst: str | Path, *, only: list[str] | N
         skipped += [k.rpartition(".")[0] for k, t in new.items()
                     if k.endswith(".weight") and t.dim() == 2 and t.dtype != torch.float8_e4m3fn]
         save_file(new, str(dst / path.name))
+    index_path = src / "model.safetensors.index.json"
+    if index_path.is_file():
+        index = json.loads(index_path.read_text(encoding="utf-8"))
+        weight_map = dict(index.get("weight_map", {}))
+        for module in done:
+            shard = weight_map.get(f"{module}.weight")
+            if shard is not None:
+                weight_map[f"{module}.weight_scale"] = shard
+        index["weight_map"] = dict(sorted(weight_map.items()))
+        total = 0
+        for path in sorted(dst.glob("*.safetensors")):
+            with safe_open(str(path), framework="pt", device="cpu") as f:
+                for k in f.keys():
+                    sl = f.get_slice(k)
+                    n = 1
+                    for d in sl.get_shape():
+                        n *= d
+                    total += n * _DTYPE_BYTES.get(sl.get_dtype(), 0)
+        index.setdefault("metadata", {})["total_size"] = total
+        (dst / index_path.name).write_text(json.dumps(index, indent=2), encoding="utf-8")
     cfg_path = src / "config.json"
     cfg = json.loads(cfg_path.read_text(encoding="utf-8")) if cfg_path.is_file() else {}
     cfg["quantization_config"] = {"quant_method": "fp8", "activation_scheme": "dynamic",

@@ -3,7 +3,7 @@
 Semantics follow the reference's ``phyai/runtime/cuda_graph_manager.py:76-317``
 (``CudaGraph`` / ``CudaGraphRegistry``): example inputs are cloned into static
 buffers, the function is run a few times on a side stream so every lazy
-allocation (here: the kernels' workspace) exists, then it is recorded once into
+allocation (here: the kernels' workspace, which the graph owns) exists, then it is recorded once into
 a graph with the dispatcher in capture mode; ``replay`` copies new inputs into
 the static buffers and launches the whole recording with a single call.  The
 returned tensors alias static storage and are overwritten by the next replay.
@@ -19,6 +19,7 @@ from typing import Any, Callable, Hashable
 
 import torch
 
+from phyai_amd.ops import WorkspaceOwner, workspace_owner
 from phyai_amd.state import graph_capture
 
 
@@ -35,6 +36,9 @@ class HipGraph:
         self._graph: torch.cuda.CUDAGraph | None = None
         self._inputs: dict[str, torch.Tensor] = {}
         self._output: Any = None
+        # The kernels' scratch, owned by this graph: its addresses are part of the recording.
+        self._workspace = WorkspaceOwner()
+        self.capture_stream: torch.cuda.Stream | None = None
 
     @property
     def is_captured(self) -> bool:
@@ -69,7 +73,7 @@ class HipGraph:
 
         side = torch.cuda.Stream()
         side.wait_stream(torch.cuda.current_stream())
-        with torch.cuda.stream(side):
+        with torch.cuda.stream(side), workspace_owner(self._workspace):
             for _ in range(self.num_warmup_iters):
                 fn(**bufs)
         torch.cuda.current_stream().wait_stream(side)
@@ -78,11 +82,11 @@ class HipGraph:
         kwargs = {"stream": side}
         if self.mempool is not None:
             kwargs["pool"] = self.mempool
-        # Capture on the stream the warm-up ran on, so that per-stream state the ops keep
-        # (their workspace) is the one that already exists.
-        with graph_capture(), torch.cuda.graph(graph, **kwargs):
+        # The warm-up created this graph's workspace; recording finds it through the same owner.
+        # Streams come from a pool and are handed out again: nothing may be keyed by them alone.
+        with graph_capture(), workspace_owner(self._workspace), torch.cuda.graph(graph, **kwargs):
             out = fn(**bufs)
-        self._graph, self._inputs, self._output = graph, bufs, out
+        self._graph, self._inputs, self._output, self.capture_stream = graph, bufs, out, side
 
     def replay(self, inputs: dict[str, torch.Tensor] | None = None) -> Any:
         self._need_capture()

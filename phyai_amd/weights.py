@@ -42,6 +42,11 @@ def _as_param_dtype(loaded: torch.Tensor, param: nn.Parameter) -> torch.Tensor:
         return loaded
     if param.dtype == torch.float8_e4m3fn and loaded.dtype == torch.uint8:
         return loaded.view(torch.float8_e4m3fn)
+    if loaded.dtype in (torch.float8_e4m3fn, torch.float8_e5m2):
+        # codes without their scale are not values: a quantized tensor for a module that was not
+        # built as an fp8 linear (an embedding, a head) would silently load garbage
+        raise ValueError(f"the checkpoint holds {loaded.dtype} codes for a {param.dtype} parameter; the module was not "
+                         "built as an fp8 linear (is it missing from the checkpoint's ignored_layers?)")
     return loaded.to(param.dtype)
 
 

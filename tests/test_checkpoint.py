@@ -202,6 +202,33 @@ def test_per_tensor_scales_of_fused_legs(tmp_path):
     assert float(layer.input_scale) == pytest.approx(0.3)
 
 
+def test_fp8_codes_for_an_unquantized_parameter_are_refused(tmp_path):
+    """A quantized tensor for a module that was not built as an fp8 linear must not be cast into it."""
+    from safetensors.torch import save_file
+
+    from phyai_amd.linear.layers import ReplicatedLinear
+    from phyai_amd.weights import load_pretrained
+
+    layer = ReplicatedLinear(32, 16, bias=False, params_dtype=torch.bfloat16, device="cpu", prefix="head")
+    assert layer.weight.dtype == torch.bfloat16
+    save_file({"head.weight": torch.zeros(16, 32, dtype=torch.uint8).view(torch.float8_e4m3fn)}, str(tmp_path / "m.safetensors"))
+    with pytest.raises(ValueError, match="not built as an fp8 linear"):
+        load_pretrained(layer, tmp_path / "m.safetensors", strict=False)
+
+
+def test_offline_quantizer_selects_linears_only():
+    from phyai_amd.quantize_checkpoint import _selected
+
+    for name in ("model.embed_tokens", "lm_head", "model.norm", "model.layers.0.input_layernorm",
+                 "vision_tower.embeddings.position_embedding", "transformer.wte"):
+        assert not _selected(name, [], [])
+    for name in ("model.layers.0.self_attn.q_proj", "model.layers.3.mlp.down_proj", "vision_tower.encoder.layers.0.mlp.fc1"):
+        assert _selected(name, [], [])
+    assert not _selected("model.layers.0.self_attn.q_proj", [], ["q_proj"])
+    assert _selected("lm_head", ["lm_*"], [])                      # an explicit allow-list wins over the defaults
+    assert not _selected("model.layers.0.mlp.down_proj", ["lm_*"], [])
+
+
 # ---- offline quantizer + end to end (GPU) ------------------------------------------------------------
 
 @pytest.mark.gpu
@@ -219,17 +246,26 @@ def test_quantize_checkpoint_then_load_and_run(dev, tmp_path):
     src.mkdir()
     bf16 = _bf16_checkpoint()
     bf16["model.norm.weight"] = seeded((64,), seed=1)                      # not a matrix: copied through
-    bf16["lm_head.weight"] = seeded((96, 64), seed=2, scale=0.05)          # ignored by name: stays bf16
+    bf16["lm_head.weight"] = seeded((96, 64), seed=2, scale=0.05)          # a head and an embedding table are
+    bf16["model.embed_tokens.weight"] = seeded((96, 64), seed=3, scale=0.05)   # never fp8 linears: kept by default
     save_file(bf16, str(src / "model.safetensors"))
     (src / "config.json").write_text(json.dumps({"hidden_size": 64}))
-    done = quantize_checkpoint(src, dst, ignore=["lm_head"])
+    (src / "model.safetensors.index.json").write_text(json.dumps(
+        {"metadata": {"total_size": 0}, "weight_map": {k: "model.safetensors" for k in bf16}}))
+    done = quantize_checkpoint(src, dst)
     assert len(done) == 7
     cfg = json.loads((dst / "config.json").read_text())
     assert cfg["hidden_size"] == 64 and cfg["quantization_config"]["quant_method"] == "fp8"
-    assert cfg["quantization_config"]["ignored_layers"] == ["lm_head"]
+    assert cfg["quantization_config"]["ignored_layers"] == ["lm_head", "model.embed_tokens"]
+    index = json.loads((dst / "model.safetensors.index.json").read_text())
+    assert all(index["weight_map"].get(f"{m}.weight_scale") == "model.safetensors" for m in done)
+    assert index["metadata"]["total_size"] == sum(
+        (v.numel() * (1 if k.rpartition(".")[0] in done and k.endswith(".weight") else v.element_size())
+         for k, v in bf16.items())) + sum(4 * bf16[f"{m}.weight"].shape[0] for m in done)
     want = _oracle_fp8_checkpoint({k: v for k, v in bf16.items() if k.startswith("model.layers")})
     with safe_open(str(dst / "model.safetensors"), framework="pt", device="cpu") as f:
         got = {k: f.get_tensor(k) for k in f.keys()}
+    assert got["model.embed_tokens.weight"].dtype == torch.bfloat16
     assert got["lm_head.weight"].dtype == torch.bfloat16 and torch.equal(got["model.norm.weight"], bf16["model.norm.weight"])
     for k, v in want.items():                                             # the kernel's codes and scales are the oracle's
         assert torch.equal(got[k].view(torch.uint8) if v.dtype == torch.float8_e4m3fn else got[k],
@@ -243,7 +279,7 @@ def test_quantize_checkpoint_then_load_and_run(dev, tmp_path):
             block = _Block(dev)
         assert block.qkv_proj.spec.spec_id == "fp8_per_channel"
         rep = load_pretrained(block, dst, strict=False)
-        assert sorted(rep.unexpected) == ["lm_head.weight", "model.norm.weight"] and not rep.missing
+        assert sorted(rep.unexpected) == ["lm_head.weight", "model.embed_tokens.weight", "model.norm.weight"] and not rep.missing
         x = seeded((50, 64), seed=9).to(dev)
         y, _ = block.qkv_proj(x)
         p = "model.layers.0.self_attn"

@@ -271,3 +271,44 @@ def test_graph_replays_of_the_split_k_tile_kernel(L, dev):
         torch.cuda.synchronize()
         assert torch.equal(again, eager)
 
+
+
+def test_a_graph_keeps_its_workspace_when_other_work_outgrows_it(L, dev):
+    """A recorded graph holds the addresses of its scratch (activation codes, split-K counters and
+    partial sums).  Larger problems that later run eagerly - on the pooled stream the graph was
+    recorded on as well as on the current one - must neither free nor share that scratch: the
+    replays stay bit-equal to the eager result while other tensors are allocated and overwritten."""
+    from phyai_amd import ops
+    from phyai_amd.runtime import HipGraph
+
+    x = seeded((200, 1040), 60).to(dev)                      # generic kernel, K split: counters + partial sums
+    wq, ws = ops.fp8_weight_quant(seeded((512, 1040), 61, 0.02).to(dev))
+    assert ops.describe_plan(200, 512, 1040).startswith("generic 128x128 splits=")
+    eager = ops.fp8_linear(x, wq, ws)
+    g = HipGraph()
+    g.capture(lambda x: ops.fp8_linear(x, wq, ws), {"x": x})
+    owned = list(g._workspace.tensors.values())
+    assert len(owned) == 1 and not g._workspace.retired
+    # now outgrow every per-stream workspace in sight, on the graph's recording stream too
+    xb = seeded((816, 16384), 62).to(dev)
+    wqb, wsb = ops.fp8_weight_quant(seeded((2048, 16384), 63, 0.02).to(dev))
+    big_eager = ops.fp8_linear(xb, wqb, wsb)
+    g.capture_stream.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.stream(g.capture_stream):
+        big_side = ops.fp8_linear(xb, wqb, wsb)
+    torch.cuda.current_stream().wait_stream(g.capture_stream)
+    torch.cuda.synchronize()
+    assert torch.equal(big_side, big_eager)
+    assert list(g._workspace.tensors.values())[0] is owned[0]        # untouched by all that
+    junk = [torch.full((1 << 20,), 0x7F, dtype=torch.uint8, device=dev) for _ in range(64)]   # reuse anything freed
+    for seed in (64, 65, 66):
+        xi = seeded((200, 1040), seed).to(dev)
+        out = g.replay({"x": xi})
+        for t in junk:
+            t.add_(1)
+        torch.cuda.synchronize()
+        assert torch.equal(out, ops.fp8_linear(xi, wq, ws))
+    # an eager workspace that grows is replaced, not freed: queued launches may still use it
+    n_retired = len(ops._retired)
+    ops.reserve_workspace(ops.reserve_workspace(1).numel() + 1)
+    assert len(ops._retired) == n_retired + 1
