@@ -5,9 +5,33 @@
 // few hundred workgroups do it.  Instead every access to data that crosses
 // workgroups (partial sums, arrival counters) is a relaxed device-scope atomic:
 // stores are written through to memory, loads never hit a stale L2 line, and no
-// fence wider than the workgroup is issued.  Ordering inside a workgroup:
-// each lane waits for its own stores to complete (vmcnt(0)), the workgroup
-// barrier collects all lanes, then one lane bumps the tile's counter.
+// fence wider than the workgroup is issued.
+//
+// Why the last arriver sees every partial sum (gfx950 only; this is an argument about that
+// hardware, not about the HIP memory model, under which relaxed atomics order nothing):
+//  1. A relaxed agent-scope atomic store is a write-through store (sc1 set): it does not stay
+//     in the issuing XCD's L2 but goes to the memory side, the coherence point of all XCDs.
+//     The AMDGPU memory model's own agent-scope release on this target is "write back the L2's
+//     dirty lines, then s_waitcnt vmcnt(0), then the releasing store"; nothing here is ever
+//     dirty in L2, so the write-back has nothing to do and is left out.
+//  2. vmcnt counts stores as well as loads on this target and a store leaves the count when
+//     the memory side has acknowledged it: after wait_own_stores() (s_waitcnt vmcnt(0), an
+//     asm statement with a memory clobber, so the compiler moves no access across it) every
+//     store of that lane is visible device-wide.
+//  3. __syncthreads() in splitk_arrive() is a workgroup-scope release + s_barrier + acquire:
+//     every lane of the workgroup has passed step 2 before thread 0 goes on, and the compiler
+//     keeps the counter update behind it.
+//  4. Only then does thread 0 add to the tile's counter, an atomic executed at the memory side:
+//     the adds of the S splits are totally ordered there, and the one that reads S - 1 was
+//     issued after the partial sums of all S splits were acknowledged.
+//  5. The gathering workgroup's loads are relaxed agent-scope atomic loads (sc1): they are
+//     served from the memory side, never from a line its own L2 might hold, and they are issued
+//     after the second barrier of splitk_arrive(), i.e. after the counter value was read.
+// The same reasoning covers the reset: the gatherer stores 0 to the counter after its loads have
+// returned (their values feed the epilogue), and the next call that touches the counter is a later
+// kernel on the same stream or graph, ordered behind this one by the queue.
+// tests/test_gpu_parity.py runs split-K shapes repeatedly against one fixed result (and under graph
+// replay and from two streams) to catch a toolchain or target change that breaks an assumption.
 //
 // Partials are summed by the last workgroup to arrive, in split order, so the
 // result does not depend on arrival order.  That workgroup also resets the

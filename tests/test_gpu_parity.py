@@ -570,6 +570,29 @@ def _as_bits(t):
     return t.contiguous().view(torch.int16)
 
 
+@pytest.mark.parametrize("force,shape", [(("PHYAI_FP8_BIG", "128"), (300, 384, 4096)), (("PHYAI_FP8_BIG", "256"), (300, 384, 4096)),
+                                         (("PHYAI_FP8_TILE", "128,128,4"), (200, 512, 1040))])
+def test_split_k_many_runs_one_result(dev, monkeypatch, force, shape):
+    """The split-K hand-over (write-through partial sums, own-store wait, barrier, arrival counter,
+    write-through reads) orders nothing on paper; it rests on how gfx950 executes those accesses.
+    200 back-to-back launches, no synchronisation in between, against the first result: stops at the
+    first mismatch."""
+    ops = _ops()
+    monkeypatch.setenv(*force)
+    if force[0] == "PHYAI_FP8_BIG":
+        monkeypatch.setenv("PHYAI_FP8_BIG_SPLITS", "4")
+    M, N, K = shape
+    x, wq, ws, b = _problem(M, N, K, seed=1234)
+    xd, wd, sd, bd = x.to(dev), wq.to(dev), ws.to(dev), b.to(dev)
+    xq, xs = ops.fp8_quant_rowwise(xd)
+    first = ops.fp8_gemm(xq, xs, wd, sd, bd)
+    assert_close_to_ref(first, ref.gemm_f32(*ref.quant_rowwise(x), wq, ws, b), "split-K")
+    outs = [ops.fp8_gemm(xq, xs, wd, sd, bd) for _ in range(200)]
+    torch.cuda.synchronize()
+    for i, o in enumerate(outs):
+        assert torch.equal(_as_bits(o), _as_bits(first)), f"launch {i} differs from the first"
+
+
 def test_two_streams_run_split_k_linears_concurrently(dev, monkeypatch):
     """Each (device, stream) pair has its own workspace (split-K counters and partials, code
     staging), so linears issued on two streams at once must give the serial results bit for bit."""
