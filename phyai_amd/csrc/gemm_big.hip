@@ -146,7 +146,10 @@ __device__ __forceinline__ v8i big_frag(const uint8_t* buf, int row, int h, int 
 // Variants whose ring leaves room for two workgroups per CU are held to the register budget of
 // two wavefronts per SIMD: while one workgroup is in its prologue or epilogue the other one
 // keeps the MFMA pipe busy.
-template <int TM, int TN, int DEPTH, int EPI, bool SPLIT>
+//
+// WGM x WGN: how the four wavefronts tile the workgroup's output (2 x 2, or 1 x 4 for the
+// 224 x 256 tile: every wavefront then walks all the tile's token rows and a quarter of its columns).
+template <int TM, int TN, int DEPTH, int EPI, bool SPLIT, int WGM = 2, int WGN = 2>
 __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu((DEPTH == 2 && TM < 4) ? 2 : 1)))
 void gemm_fp8_big_kernel(
     const uint8_t* __restrict__ a_a, const uint8_t* __restrict__ a_b, int a_K, int a_M, int a_N, int a_m_tiles,
@@ -161,19 +164,21 @@ void gemm_fp8_big_kernel(
     p.k_per_split = a_k_per_split; p.partials = a_partials; p.counters = a_counters;
     p.m_tiles = a_m_tiles; p.n_tiles = a_n_tiles; p.band = a_band; p.by_rows = a_by_rows; p.res = a_res;
     constexpr bool GATED = epi_is_gated(EPI);
-    constexpr int BM = 64 * TM, BN = 64 * TN;        // workgroup tile
+    static_assert(WGM * WGN == 4, "four wavefronts per workgroup");
+    constexpr int BM = WGM * 32 * TM, BN = WGN * 32 * TN;   // workgroup tile
     constexpr int WM = 32 * TM, WN = 32 * TN;        // wavefront tile
     constexpr int STAGE_BYTES = (BM + BN) * BIG_BK;  // one stage: A rows, then B rows
     constexpr int CA = BM / 32, CB = BN / 32;        // copy instructions (8 rows each) per wavefront per stage
     constexpr int COPIES = CA + CB;
     constexpr int SLOTS_PER_STAGE = 2 * TM * TN;     // MFMAs of a wavefront per stage
     constexpr int CPS = (COPIES * 2 + SLOTS_PER_STAGE - 1) / SLOTS_PER_STAGE;   // copies per MFMA: done by mid-stage
-    static_assert((TM == TN && TM % 2 == 0) || (TM == 3 && TN == 2), "supported wavefront tiles");
+    static_assert((TM == TN && TM % 2 == 0) || (TM == 3 && TN == 2) || (TM == 7 && TN == 2), "supported wavefront tiles");
+    static_assert(BM % 32 == 0 && BN % 32 == 0, "every wavefront copies whole groups of 8 rows");
     static_assert(DEPTH == 2 || DEPTH == 4, "ring depth");
     __shared__ __attribute__((aligned(1024))) uint8_t lds[DEPTH * STAGE_BYTES];
 
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
-    const int wm = wave >> 1, wn = wave & 1;
+    const int wm = wave / WGN, wn = wave % WGN;
     const int l32 = lane & 31, h = lane >> 5;
     const int half_n = p.N / 2;
     BigTile tile_id;
@@ -502,7 +507,7 @@ static int big_tiles(int M, int N, int epilogue, int bm, int bn) {
 // tiles, and those are split along K when even the small tiles leave CUs idle: a CU can pull
 // only about 45 GB/s from L2, so a mid-sized GEMM finishes sooner on more CUs even though the
 // partial sums then make a round trip through memory.
-static int big_tile_cols(int tile) { return tile == 256 ? 256 : 128; }
+static int big_tile_cols(int tile) { return (tile == 256 || tile == 224) ? 256 : 128; }
 
 // Fraction of the tile slots that hold a tile, over all rounds of `slots` concurrent tiles.
 static double big_fill(int tiles, int slots) {
@@ -516,7 +521,7 @@ BigPlan big_plan(int M, int N, int K, int epilogue) {
     int forced = -1;
     if (const char* e = tuning_env("PHYAI_FP8_BIG")) forced = atoi(e);   // "0": never; "256"/"192"/"128": force
     if (forced == 0) return pl;
-    if (forced == 256 || forced == 192 || forced == 128) pl.tile = forced;
+    if (forced == 256 || forced == 224 || forced == 192 || forced == 128) pl.tile = forced;
     else if (M < 128) return pl;
     // 256 x 256 tiles need the fewest bytes from L2 per flop but run one workgroup per CU, so a
     // tile's prologue and epilogue leave the MFMA pipe idle; 192 x 128 tiles fit twice and overlap
@@ -534,7 +539,13 @@ BigPlan big_plan(int M, int N, int K, int epilogue) {
     else if (K <= 8192 && big_tiles(M, N, epilogue, 256, 256) < 200 && big_tiles(M, N, epilogue, 192, 128) > 256 &&
              big_tiles(M, N, epilogue, 192, 128) <= 512 && big_tiles(M, N, epilogue, 128, 128) > 512)
         pl.tile = 192;
-    else if (big_tiles(M, N, epilogue, 256, 256) >= 200) pl.tile = 256;
+    else if (big_tiles(M, N, epilogue, 256, 256) >= 200)
+        // 224 x 256 tiles (every wavefront walks all 224 token rows) when they need no more tile
+        // rows than 256 x 256: the same number of workgroups, fewer MFMAs on padding (816 rows:
+        // 896 instead of 1024, gate_up 2048 -> 32768 at M = 816 67.4 -> 64.2 us).  The gain is
+        // smaller than the saved MFMAs because each wavefront then reads all of the tile's
+        // activation rows from LDS, which is the next limit (113 of 128 bytes per clock).
+        pl.tile = big_ceil_div(M, 224) == big_ceil_div(M, 256) ? 224 : 256;
     else if (big_tiles(M, N, epilogue, 128, 128) >= 32) pl.tile = 128;   // fewer: the weight-streaming kernel wins
     else return pl;
     const int tiles = big_tiles(M, N, epilogue, pl.tile, big_tile_cols(pl.tile));
@@ -552,7 +563,7 @@ BigPlan big_plan(int M, int N, int K, int epilogue) {
     }
     if (const char* e = tuning_env("PHYAI_FP8_BIG_SPLITS")) {
         const int s = atoi(e);
-        if (pl.tile != 192 && s >= 1 && K % (s * 128) == 0 && K / s >= 512 && tiles * s <= 4096) pl.splits = s;
+        if (pl.tile != 192 && pl.tile != 224 && s >= 1 && K % (s * 128) == 0 && K / s >= 512 && tiles * s <= 4096) pl.splits = s;
     }
     if (const char* e = tuning_env("PHYAI_FP8_BIG_DEPTH")) {
         const int d = atoi(e);
@@ -567,12 +578,13 @@ size_t big_partial_bytes(int M, int N, int epilogue, const BigPlan& pl) {
     return (size_t)big_tiles(M, N, epilogue, pl.tile, bn) * pl.splits * pl.tile * bn * sizeof(float);
 }
 
-template <int TM, int TN, int DEPTH, int EPI>
+template <int TM, int TN, int DEPTH, int EPI, int WGM = 2, int WGN = 2>
 static void big_launch(BigArgs a, const GemmProblem& g, int splits, hipStream_t st) {
     const bool gated = epi_is_gated(EPI);
-    const int bn_eff = gated ? 32 * TN : 64 * TN;
+    constexpr int BM = WGM * 32 * TM, BN = WGN * 32 * TN;
+    const int bn_eff = gated ? BN / 2 : BN;
     a.n_tiles = big_ceil_div(gated ? g.N / 2 : g.N, bn_eff);
-    a.m_tiles = big_ceil_div(g.M, 64 * TM);
+    a.m_tiles = big_ceil_div(g.M, BM);
     // Which operand the XCDs share.  By default an XCD takes tile columns: its L2 then holds the
     // weight rows of those columns once, but every XCD streams all activation rows it meets.
     // With few tile columns and long rows of activations (816 x B tokens into a 16384 -> 2048
@@ -597,7 +609,7 @@ static void big_launch(BigArgs a, const GemmProblem& g, int splits, hipStream_t 
     // bands of 4 tile rows; a grid of up to 8 tile rows whose activation rows still fit an XCD's
     // L2 beside the weight stream is one band, so that the weights come from HBM once
     a.band = 4;
-    if (!a.by_rows && a.m_tiles <= 8 && (int64_t)a.m_tiles * (64 * TM) * (g.K < 4096 ? g.K : 4096) <= (5 << 19)) a.band = a.m_tiles;
+    if (!a.by_rows && a.m_tiles <= 8 && (int64_t)a.m_tiles * BM * (g.K < 4096 ? g.K : 4096) <= (5 << 19)) a.band = a.m_tiles;
     if (const char* e = tuning_env("PHYAI_FP8_BAND")) { const int b = atoi(e); if (b >= 1 && b <= 16) a.band = b; }
     const int outer = a.by_rows ? a.n_tiles : a.m_tiles, inner = a.by_rows ? a.m_tiles : a.n_tiles;
     const dim3 grid(big_grid_ids(outer, inner, a.band), 1, splits);
@@ -605,22 +617,22 @@ static void big_launch(BigArgs a, const GemmProblem& g, int splits, hipStream_t 
                        a.b_scale, a.bias, a.out, a.ldo, a.a_scale_scalar, a.partials, a.counters, a.res
     if (splits > 1) {
         if constexpr (TM == TN && (TM == 4 || DEPTH == 4))
-            hipLaunchKernelGGL((gemm_fp8_big_kernel<TM, TN, DEPTH, EPI, true>), grid, dim3(256), 0, st, PHYAI_BIG_ARGS);
+            hipLaunchKernelGGL((gemm_fp8_big_kernel<TM, TN, DEPTH, EPI, true, WGM, WGN>), grid, dim3(256), 0, st, PHYAI_BIG_ARGS);
     } else {
-        hipLaunchKernelGGL((gemm_fp8_big_kernel<TM, TN, DEPTH, EPI, false>), grid, dim3(256), 0, st, PHYAI_BIG_ARGS);
+        hipLaunchKernelGGL((gemm_fp8_big_kernel<TM, TN, DEPTH, EPI, false, WGM, WGN>), grid, dim3(256), 0, st, PHYAI_BIG_ARGS);
     }
 #undef PHYAI_BIG_ARGS
 }
 
-template <int TM, int TN, int DEPTH>
+template <int TM, int TN, int DEPTH, int WGM = 2, int WGN = 2>
 static int big_launch_epi(const BigArgs& a, const GemmProblem& g, int splits, hipStream_t st) {
     switch (g.epilogue) {
-    case EPI_NONE: big_launch<TM, TN, DEPTH, EPI_NONE>(a, g, splits, st); return 0;
-    case EPI_GEGLU_TANH: big_launch<TM, TN, DEPTH, EPI_GEGLU_TANH>(a, g, splits, st); return 0;
-    case EPI_GEGLU_ERF: big_launch<TM, TN, DEPTH, EPI_GEGLU_ERF>(a, g, splits, st); return 0;
-    case EPI_SWIGLU: big_launch<TM, TN, DEPTH, EPI_SWIGLU>(a, g, splits, st); return 0;
-    case EPI_GELU_TANH: big_launch<TM, TN, DEPTH, EPI_GELU_TANH>(a, g, splits, st); return 0;
-    case EPI_GELU_ERF: big_launch<TM, TN, DEPTH, EPI_GELU_ERF>(a, g, splits, st); return 0;
+    case EPI_NONE: big_launch<TM, TN, DEPTH, EPI_NONE, WGM, WGN>(a, g, splits, st); return 0;
+    case EPI_GEGLU_TANH: big_launch<TM, TN, DEPTH, EPI_GEGLU_TANH, WGM, WGN>(a, g, splits, st); return 0;
+    case EPI_GEGLU_ERF: big_launch<TM, TN, DEPTH, EPI_GEGLU_ERF, WGM, WGN>(a, g, splits, st); return 0;
+    case EPI_SWIGLU: big_launch<TM, TN, DEPTH, EPI_SWIGLU, WGM, WGN>(a, g, splits, st); return 0;
+    case EPI_GELU_TANH: big_launch<TM, TN, DEPTH, EPI_GELU_TANH, WGM, WGN>(a, g, splits, st); return 0;
+    case EPI_GELU_ERF: big_launch<TM, TN, DEPTH, EPI_GELU_ERF, WGM, WGN>(a, g, splits, st); return 0;
     default: return -2;
     }
 }
@@ -640,6 +652,7 @@ int launch_gemm_big(const GemmProblem& g, const BigPlan& pl, hipStream_t st) {
                           g.workspace_bytes < kGemmHeaderBytes + big_partial_bytes(g.M, g.N, g.epilogue, pl)))
         return -3;
     if (pl.tile == 256) return big_launch_epi<4, 4, 2>(a, g, pl.splits, st);
+    if (pl.tile == 224 && pl.splits == 1) return big_launch_epi<7, 2, 2, 1, 4>(a, g, 1, st);
     if (pl.tile == 192 && pl.splits == 1) return big_launch_epi<3, 2, 2>(a, g, 1, st);
     if (pl.tile == 128 && pl.depth == 4) return big_launch_epi<2, 2, 4>(a, g, pl.splits, st);
     if (pl.tile == 128 && pl.splits == 1) return big_launch_epi<2, 2, 2>(a, g, 1, st);

@@ -416,7 +416,7 @@ int describe_gemm_plan(int M, int N, int K, int epilogue, char* buf, size_t n) {
     case GemmChoice::SKINNY:
         return snprintf(buf, n, "small-m nt=%d mb=%d kpw=%d rounds=%d", c.sk.nt, c.sk.mb, c.sk.kpw, c.sk.rounds);
     case GemmChoice::BIG:
-        return snprintf(buf, n, "tile %dx%d depth=%d splits=%d tiles=%d", c.big.tile, c.big.tile == 256 ? 256 : 128,
+        return snprintf(buf, n, "tile %dx%d depth=%d splits=%d tiles=%d", c.big.tile, (c.big.tile == 256 || c.big.tile == 224) ? 256 : 128,
                         c.big.depth, c.big.splits, c.big.tiles);
     default:
         return snprintf(buf, n, "generic %dx%d splits=%d", c.tc.bm, c.tc.bn, c.tc.splits);
