@@ -192,118 +192,64 @@ def decoder_layer_times(dev, layers, M, denoise_steps, steps, warmup):
 
 
 def whole_step_times(dev, layers, M, prefix_len, denoise_steps, steps, warmup):
-    """The whole flow-matching loop as ONE hipGraph (reference models/pi05/model_runner_pi05.py:689-738:
-    per step action embedding, 18 decoder layers, final adaptive norm, action projection, Euler
-    update), with the decoder layer of models/pi05/modeling_pi05.py:804-835 including RoPE and the
-    joint attention over the prefix KV plus the chunk's own keys and values.  Attention
-    (torch SDPA), RoPE, embedding and projection are plain torch ops in BOTH variants: stand-ins
-    for the reference's attention back end, which this library does not replace.  The variants
-    differ in the linear path only: `library` = this library's fused layer (norm+quantizer,
-    GEMM, GEMM+gated residual), `torch_path` = the reference's structure on torch ops
-    (norm, quantizer expressions, torch._scaled_mm, gelu*mul, addcmul).  Data chains through
-    the layers.  Returns us per denoise step for each, or a reason string."""
-    import torch.nn.functional as F
+    """The whole flow-matching loop as ONE hipGraph - phyai_amd.runtime.expert_loop.ExpertDenoiseLoop,
+    the mirror of the reference's runner loop (models/pi05/model_runner_pi05.py:689-738) and decoder
+    layer (models/pi05/modeling_pi05.py:801-835) - on this benchmark's weights.  Attention (RoPE +
+    torch SDPA over the prefix KV plus the chunk's own keys and values), embedding and projection
+    are plain torch ops in BOTH variants: stand-ins for the reference's attention back end, which
+    this library does not replace.  The variants differ in the linear path only: `library` = the
+    fused layer (norm+quantizer, GEMM, GEMM+gated residual), `torch_path` = the reference's
+    structure on torch ops (norm, quantizer expressions, torch._scaled_mm, gelu*mul, addcmul).
+    Data chains through the layers.  Returns us per denoise step for each, or a reason string."""
+    import phyai_amd.linear as L
+    from phyai_amd.runtime.expert_loop import ExpertDenoiseLoop, ExpertLayer, PrefixAttentionStandIn
 
-    from phyai_amd import ops
-    from phyai_amd.runtime import HipGraph
-
-    D, H, HD, ADIM = 1024, 8, 256, 32
+    D, ADIM = 1024, 32
     g = torch.Generator().manual_seed(4242)
 
     def rnd(*shape, scale=1.0):
         return (torch.randn(*shape, generator=g) * scale).to(torch.bfloat16).to(dev)
 
-    L = len(layers)
-    mods = [[(rnd(1, 3 * D, scale=0.1), rnd(1, 3 * D, scale=0.1)) for _ in range(L)] for _ in range(denoise_steps)]
-    final_mod = [rnd(1, 3 * D, scale=0.1) for _ in range(denoise_steps)]
-    kc = [torch.cat([rnd(prefix_len, 1, HD), torch.zeros(M, 1, HD, dtype=torch.bfloat16, device=dev)]) for _ in range(L)]
-    vc = [torch.cat([rnd(prefix_len, 1, HD), torch.zeros(M, 1, HD, dtype=torch.bfloat16, device=dev)]) for _ in range(L)]
-    pos = torch.arange(prefix_len, prefix_len + M, dtype=torch.float32)
-    inv = 1.0 / (10000.0 ** (torch.arange(0, HD, 2, dtype=torch.float32) / HD))
-    ang = pos[:, None] * inv[None, :]
-    cos, sin = ang.cos()[:, None, :].to(dev), ang.sin()[:, None, :].to(dev)
-    w_in, w_out = rnd(D, ADIM, scale=0.1), rnd(ADIM, D, scale=0.02)
-    dt = -1.0 / denoise_steps
-
-    def rope(t):
-        t1, t2 = t[..., : HD // 2].float(), t[..., HD // 2:].float()
-        return torch.cat([t1 * cos - t2 * sin, t2 * cos + t1 * sin], dim=-1).to(torch.bfloat16)
-
-    def attention(fused, li):
-        q, k, v = fused.split([H * HD, HD, HD], dim=-1)
-        q, k = rope(q.reshape(M, H, HD)), rope(k.reshape(M, 1, HD))
-        kc[li][prefix_len:].copy_(k)
-        vc[li][prefix_len:].copy_(v.reshape(M, 1, HD))
-        S = prefix_len + M
-        o = F.scaled_dot_product_attention(q.transpose(0, 1)[None], kc[li].transpose(0, 1)[None].expand(1, H, S, HD),
-                                           vc[li].transpose(0, 1)[None].expand(1, H, S, HD))
-        return o[0].transpose(0, 1).reshape(M, H * HD)
-
-    def torch_norm(h, mod):
-        scale, shift, gate = mod.float().chunk(3, dim=-1)
-        hf = h.float()
-        n = hf * torch.rsqrt(hf.pow(2).mean(-1, keepdim=True) + 1e-6)
-        return (n * (1.0 + scale) + shift).to(torch.bfloat16), gate.to(torch.bfloat16)
-
-    def torch_linear(x, t, act=False):
-        a = x.abs().amax(dim=-1, keepdim=True).clamp_min(1e-12)
-        s = (a / 448.0).to(torch.float32)
-        xq = (x / s).to(torch.float8_e4m3fn)
-        y = torch._scaled_mm(xq, t["w"].t(), scale_a=s, scale_b=t["ws"].reshape(1, -1), out_dtype=torch.bfloat16)
-        if act:
-            half = y.shape[-1] // 2
-            y = F.gelu(y[:, :half], approximate="tanh") * y[:, half:]
-        return y
-
-    def layer_library(h, layer, li, mod):
-        nq, ns, gate = ops.adarmsnorm_fp8(h, mod[0], 1e-6)
-        fused = ops.fp8_gemm(nq, ns, layer["qkv"]["w"], layer["qkv"]["ws"], None)
-        h = ops.fp8_linear(attention(fused, li), layer["o"]["w"], layer["o"]["ws"], None, residual=h, gate=gate)
-        mq, ms, gate2 = ops.adarmsnorm_fp8(h, mod[1], 1e-6)
-        a = ops.fp8_gemm(mq, ms, layer["gate_up"]["w"], layer["gate_up"]["ws"], None, epilogue="geglu_tanh",
-                         stream_weights=layer["gate_up"].get("stream", False))
-        return ops.fp8_linear(a, layer["down"]["w"], layer["down"]["ws"], None, residual=h, gate=gate2)
-
-    def layer_torch(h, layer, li, mod):
-        n, gate = torch_norm(h, mod[0])
-        fused = torch_linear(n, layer["qkv"])
-        h = torch.addcmul(h, torch_linear(attention(fused, li), layer["o"]), gate)
-        m, gate2 = torch_norm(h, mod[1])
-        return torch.addcmul(h, torch_linear(torch_linear(m, layer["gate_up"], act=True), layer["down"]), gate2)
-
-    def loop(layer_fn, final_norm):
-        def run(noise):
-            x_t = noise
-            for step in range(denoise_steps):
-                h = x_t @ w_in.t()
-                for li, layer in enumerate(layers):
-                    h = layer_fn(h, layer, li, mods[step][li])
-                v_t = final_norm(h, final_mod[step]) @ w_out.t()
-                x_t = x_t + dt * v_t
-            return x_t
-        return run
-
-    variants = {
-        "library": loop(layer_library, lambda h, m: ops.adarmsnorm(h, m, 1e-6)[0]),
-        "torch_path": loop(layer_torch, lambda h, m: torch_norm(h, m)[0]),
-    }
-    noise = rnd(M, ADIM)
-    res = {}
-    for name, fn in variants.items():
-        try:
-            out = fn(noise)      # eager first: anything this image cannot run shows up here, not inside a capture
-            torch.cuda.synchronize()
-            if not bool(torch.isfinite(out.float()).all()):
-                res[name] = "non-finite result"
-                continue
-            gr = HipGraph()
-            gr.capture(fn, {"noise": noise})
-            ts, _ = time_replays(gr, steps, warmup)
-            res[name] = round(statistics.median(ts) * 1e3 / denoise_steps, 2)
-            del gr
-        except Exception as e:  # noqa: BLE001 - report, do not fail the bench line
-            res[name] = f"unavailable: {str(e)[:160]}"
-    return res
+    L.init()
+    try:
+        mods = []
+        for li, layer in enumerate(layers):
+            lay = ExpertLayer(prefix=f"model.layers.{li}")
+            for lin, name in ((lay.qkv_proj, "qkv"), (lay.o_proj, "o"), (lay.mlp.gate_up_proj, "gate_up"),
+                              (lay.mlp.down_proj, "down")):
+                lin.weight.data, lin.weight_scale.data = layer[name]["w"], layer[name]["ws"]
+                lin.stream_weights = bool(layer[name].get("stream", False))
+            for norm in (lay.input_layernorm, lay.post_attention_layernorm):
+                norm.dense.weight.data.copy_(rnd(3 * D, D, scale=0.003))
+                norm.dense.bias.data.copy_(rnd(3 * D, scale=0.03))
+            mods.append(lay)
+        attend = PrefixAttentionStandIn(len(layers), M, prefix_len, device=dev)
+        time_emb = rnd(denoise_steps, D)
+        noise = rnd(M, ADIM)
+        res = {}
+        for name, variant in (("library", "fused"), ("torch_path", "torch")):
+            try:
+                loop = ExpertDenoiseLoop(mods, attend, chunk_size=M, action_dim=ADIM, variant=variant, use_graph=False)
+                loop.embed_action.weight.data.copy_(rnd(D, ADIM, scale=0.1))
+                loop.project_action.weight.data.copy_(rnd(ADIM, D, scale=0.02))
+                loop.embed_action.bias.data.zero_()
+                loop.project_action.bias.data.zero_()
+                loop.bind_euler_schedule(time_emb, -1.0 / denoise_steps, denoise_steps)
+                out = loop.run(noise)    # eager first: anything this image cannot run shows up here, not inside a capture
+                torch.cuda.synchronize()
+                if not bool(torch.isfinite(out.float()).all()):
+                    res[name] = "non-finite result"
+                    continue
+                loop.use_graph = True
+                loop.setup()
+                ts, _ = time_replays(loop.graph, steps, warmup)
+                res[name] = round(statistics.median(ts) * 1e3 / denoise_steps, 2)
+                del loop
+            except Exception as e:  # noqa: BLE001 - report, do not fail the bench line
+                res[name] = f"unavailable: {str(e)[:160]}"
+        return res
+    finally:
+        L._reset_for_test()
 
 
 def separate_qkv_times(dev, M, n_layers, denoise_steps, steps, warmup):

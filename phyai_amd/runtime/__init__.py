@@ -8,3 +8,5 @@ CudaGraphError = HipGraphError
 CudaGraphRegistry = HipGraphRegistry
 
 __all__ = ["HipGraph", "HipGraphError", "HipGraphRegistry", "CudaGraph", "CudaGraphError", "CudaGraphRegistry"]
+# The denoise loop (phyai_amd.runtime.expert_loop) is imported from its module: it pulls in the
+# layers, which import this package for the capture-mode flag.
