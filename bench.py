@@ -53,10 +53,19 @@ DIT_SET = [("qkv", 6144, 2048, None, 4800), ("out", 2048, 2048, None, 4800),
            ("adaLN", 12288, 2048, None, 1)]
 
 
-# HBM bytes moved by one layer's four GEMM launches at M = 50 (20.87 MB fetched + 0.87 MB written),
-# measured with rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE on `bench.py --probe` and calibrated against
-# a 64 MiB copy (profiles/expert_m50_hbm_traffic.md has the counter values).
-EXPERT_LAYER_HBM_TRAFFIC = 21_790_000
+def profiled_layer_traffic():
+    """HBM bytes moved by one layer's four GEMM launches at M = 50, as measured with rocprofv3 --pmc
+    FETCH_SIZE / WRITE_SIZE on `bench.py --probe` and calibrated against a 64 MiB copy: read from the
+    committed counter summary (its `traffic_bytes_per_layer` line), so that the figure in the JSON
+    line is the one the profile holds.  None when the summary is missing."""
+    import re
+
+    path = os.path.join(ROOT, "profiles", "expert_m50_hbm_traffic.md")
+    try:
+        m = re.search(r"^\s*traffic_bytes_per_layer\s*=\s*(\d+)", open(path, encoding="utf-8").read(), flags=re.M)
+    except OSError:
+        return None
+    return int(m.group(1)) if m else None
 
 
 def algorithmic_bytes(M: int, N: int, K: int, epilogue, bias: bool = False) -> int:
@@ -296,6 +305,87 @@ def separate_qkv_times(dev, M, n_layers, denoise_steps, steps, warmup):
     return res
 
 
+def hardware_probe(dev):
+    """Peaks re-measured on this box in the manner of the reference's probe
+    (benchmark/pi05/hardware_probe.py:36-131): a large device-to-device copy counted as 2 x bytes, best
+    of the runs, and a large square GEMM at the path's precision (fp8 x fp8, 8192^3), best of the runs,
+    through this library and through torch._scaled_mm (hipBLASLt)."""
+    from phyai_amd import ops
+
+    res = {}
+    src = torch.empty(1 << 30, dtype=torch.uint8, device=dev).fill_(1)
+    dst = torch.empty_like(src)
+    for _ in range(3):
+        dst.copy_(src)
+    torch.cuda.synchronize()
+    best = float("inf")
+    for _ in range(12):
+        a, b = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        a.record()
+        dst.copy_(src)
+        b.record()
+        torch.cuda.synchronize()
+        best = min(best, a.elapsed_time(b))
+    res["copy_GBps"] = round(2.0 * src.numel() / (best * 1e-3) / 1e9, 1)
+    del src, dst
+    n = 8192
+    g = torch.Generator(device=dev).manual_seed(1)
+    xq, xs = ops.fp8_quant_rowwise(torch.randn(n, n, generator=g, device=dev).to(torch.bfloat16))
+    wq, ws = ops.fp8_weight_quant((torch.randn(n, n, generator=g, device=dev) * 0.02).to(torch.bfloat16))
+    out = torch.empty(n, n, dtype=torch.bfloat16, device=dev)
+
+    def best_of(fn, iters=10):
+        for _ in range(3):
+            fn()
+        torch.cuda.synchronize()
+        best = float("inf")
+        for _ in range(iters):
+            a, b = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+            a.record()
+            fn()
+            b.record()
+            torch.cuda.synchronize()
+            best = min(best, a.elapsed_time(b))
+        return round(2.0 * n ** 3 / (best * 1e-3) / 1e12, 1)
+
+    res["fp8_gemm_8192_TFLOPs_this_library"] = best_of(lambda: ops.fp8_gemm(xq, xs, wq, ws, None, out=out))
+    try:
+        res["fp8_gemm_8192_TFLOPs_scaled_mm"] = best_of(
+            lambda: torch._scaled_mm(xq, wq.t(), scale_a=xs, scale_b=ws.reshape(1, -1), out_dtype=torch.bfloat16, out=out))
+    except Exception as e:  # noqa: BLE001 - torch._scaled_mm may not run on every image
+        res["fp8_gemm_8192_TFLOPs_scaled_mm"] = f"unavailable: {str(e)[:80]}"
+    nums = [v for k, v in res.items() if k.startswith("fp8_gemm") and not isinstance(v, str)]
+    res["fp8_TFLOPs"] = max(nums)
+    return res
+
+
+def launch_floor_us(dev, nodes=2000):
+    """Duration of one kernel node that does next to nothing (the quantizer on a single 8-element
+    row: one wavefront), from a graph of `nodes` such launches in a row: what every kernel node of
+    a replayed graph costs on this stack before it moves a byte."""
+    from phyai_amd import ops
+    from phyai_amd.runtime import HipGraph
+
+    x = torch.zeros(1, 8, dtype=torch.bfloat16, device=dev)
+    q = torch.empty(1, 8, dtype=torch.float8_e4m3fn, device=dev)
+    sc = torch.empty(1, 1, dtype=torch.float32, device=dev)
+
+    def fn():
+        for _ in range(nodes):
+            ops.fp8_quant_rowwise(x, out=q, scale_out=sc)
+
+    g = HipGraph()
+    g.capture(fn, {})
+    ts, _ = time_replays(g, 10, 2)
+    return statistics.median(ts) * 1e3 / nodes
+
+
+def ops_plan(M, N, K, epi):
+    from phyai_amd import ops
+
+    return ops.describe_plan(M, N, K, epi)
+
+
 def time_replays(graph, n, warmup):
     """HIP events around each replay, on the stream the replays are launched on."""
     for _ in range(warmup):
@@ -461,28 +551,92 @@ def probe(dev, layers, M, shapes=EXPERT_SET):
     print("probe done")
 
 
-def cpu_baseline(layers, shapes, M, budget_s=12.0):
-    """torch CPU dequantize + matmul (+ quantizer, + GeGLU) on layer 0's tensors."""
+def cpu_info():
+    """CPU model string and physical core count of the host (from /proc/cpuinfo)."""
+    model, cores = "unknown", set()
+    try:
+        phys = core = None
+        for line in open("/proc/cpuinfo", encoding="utf-8"):
+            key, _, val = line.partition(":")
+            key, val = key.strip(), val.strip()
+            if key == "model name":
+                model = val
+            elif key == "physical id":
+                phys = val
+            elif key == "core id":
+                core = val
+            elif not key and phys is not None:
+                cores.add((phys, core))
+                phys = core = None
+        if phys is not None:
+            cores.add((phys, core))
+    except OSError:
+        pass
+    return model, (len(cores) or os.cpu_count() or 1)
+
+
+def _cpu_time(fn, budget_s, min_iters=20, warmup=5):
+    for _ in range(warmup):
+        fn()
+    ts = []
+    t_end = time.perf_counter() + budget_s
+    while len(ts) < min_iters or (time.perf_counter() < t_end and len(ts) < 200):
+        t0 = time.perf_counter()
+        fn()
+        ts.append(time.perf_counter() - t0)
+    return {"p50_us": round(statistics.median(ts) * 1e6, 1), "min_us": round(min(ts) * 1e6, 1), "iters": len(ts)}
+
+
+def cpu_baseline(layers, shapes, M, n_layers):
+    """The reference's CPU form of the same linears - torch dequantize + matmul - on this box's host
+    cores, on layer 0's tensors (the bits the GPU run uses): GEMM only (codes and scales ready) and
+    quantizer + GEMM (+ GeGLU), at all threads and at one thread, plus benchmark configuration 1
+    (50 x 4096 x 1024 with bias).  Per-layer times; the headline value scales the all-threads
+    quantizer + GEMM figure by the number of layers."""
     from oracle import ref
 
     items = []
     for name, N, K, epi in shapes:
         t = layers[0][name]
         wq, ws = ref.weight_quant(t["w_bf16_cpu"])
-        items.append((t["x_cpu"], wq, ws, {None: 0, "geglu_tanh": 1}[epi]))
+        xq, xs = ref.quant_rowwise(t["x_cpu"])
+        items.append((t["x_cpu"], xq, xs, wq, ws, {None: 0, "geglu_tanh": 1}[epi]))
+    g = torch.Generator().manual_seed(0)
+    x1 = torch.randn(50, 1024, generator=g).to(torch.bfloat16)
+    w1q, w1s = ref.weight_quant((torch.randn(4096, 1024, generator=g) * 0.02).to(torch.bfloat16))
+    b1 = (torch.randn(4096, generator=g) * 0.01).to(torch.bfloat16)
 
-    def layer_once():
-        for x, wq, ws, epi in items:
+    def layer_full():
+        for x, _, _, wq, ws, epi in items:
             ref.linear(x, wq, ws, None, epi)
 
-    layer_once()
-    ts = []
-    t_end = time.perf_counter() + budget_s
-    while time.perf_counter() < t_end or len(ts) < 3:
-        t0 = time.perf_counter()
-        layer_once()
-        ts.append(time.perf_counter() - t0)
-    return statistics.median(ts), len(ts)
+    def layer_gemm_only():
+        for _, xq, xs, wq, ws, epi in items:
+            ref.epilogue(ref.gemm_f32(xq, xs, wq, ws, None), epi)
+
+    def config1():
+        ref.linear(x1, w1q, w1s, b1, 0)
+
+    all_threads = torch.get_num_threads()
+    out = {}
+    try:
+        for label, nthreads, budget in (("all_threads", all_threads, 4.0), ("one_thread", 1, 2.5)):
+            torch.set_num_threads(nthreads)
+            out[label] = {"threads": nthreads,
+                          "layer_quantizer_gemm": _cpu_time(layer_full, budget),
+                          "layer_gemm_only": _cpu_time(layer_gemm_only, budget),
+                          "config1_linear": _cpu_time(config1, budget / 4)}
+    finally:
+        torch.set_num_threads(all_threads)
+    model, phys = cpu_info()
+    full = out["all_threads"]["layer_quantizer_gemm"]
+    return {"value": round(full["p50_us"] * n_layers, 1), "unit": "us per denoise step", "cores": all_threads,
+            "kind": "port", "cpu_model": model, "physical_cores": phys,
+            "sample": f"torch CPU dequantize+matmul incl. quantizer and GeGLU on 1 of {n_layers} layers (4 linears, "
+                      f"M={M}), p50 of {full['iters']} passes at {all_threads} threads, scaled x{n_layers}; `variants` "
+                      "holds the per-layer times (us) of GEMM only and quantizer+GEMM at all threads and at one "
+                      "thread, and benchmark configuration 1",
+            "variants": out}
 
 
 def main() -> int:
@@ -560,7 +714,7 @@ def main() -> int:
     achieved = layer_bytes / (layer_us * 1e-6) / 1e9
     roofline = {
         "bound": "hbm", "achieved": round(achieved, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
-        "frac": round(achieved / HBM_PEAK_GBS, 4), "traffic": EXPERT_LAYER_HBM_TRAFFIC,
+        "frac": round(achieved / HBM_PEAK_GBS, 4), "traffic": profiled_layer_traffic(),
         "kernel": "gemm_fp8_skinny_kernel (M=50, four expert shapes)",
         "bytes_per_layer": layer_bytes, "us_per_layer": round(layer_us, 3),
         "note": "achieved = bytes_per_layer / us_per_layer, the four GEMM launches of a layer timed in a graph of GEMM "
@@ -571,12 +725,26 @@ def main() -> int:
                       for name, N, K, epi in EXPERT_SET},
         "whole_path_frac": round(layer_bytes * n_layers / (value_us * 1e-6) / 1e9 / HBM_PEAK_GBS, 4),
     }
+    measured = hardware_probe(dev)
+    roofline["measured_peak_GBps"] = measured["copy_GBps"]
+    roofline["frac_of_measured_peak"] = round(achieved / measured["copy_GBps"], 4)
+    node_us = launch_floor_us(dev)
+    nodes_per_layer = 2 * len(EXPERT_SET)          # a quantizer and a GEMM per linear
+    floor_us = node_us * nodes_per_layer
+    launch_floor = {
+        "node_us": round(node_us, 3), "nodes_per_layer": nodes_per_layer, "floor_us_per_layer": round(floor_us, 2),
+        "floor_us_per_denoise_step": round(floor_us * n_layers, 1),
+        "ceiling_whole_path_frac": round(layer_bytes / (floor_us * 1e-6) / 1e9 / HBM_PEAK_GBS, 4),
+        "note": "time of a kernel node that moves nothing, times the nodes a layer's four quantized linears take "
+                "(quantizer + GEMM each): no kernel, however fast, brings the layer below floor_us_per_layer in this "
+                "structure, i.e. the whole path cannot exceed ceiling_whole_path_frac of HBM peak"}
 
     # ---- prefix prefill (M = 816): MFMA-bound regime -----------------------------
     srt = sorted(ts_ms)
     extra = {"denoise_step_us": {"p50": round(value_us, 2),
                                  "p90": round(srt[min(len(srt) - 1, (9 * len(srt)) // 10)] * 1e3 / denoise_steps, 2),
                                  "min": round(srt[0] * 1e3 / denoise_steps, 2), "replays": len(srt)}}
+    roofline_prefill = None
     if not args.no_prefill:
         pl = make_layers(dev, PREFILL_SET, 816, 4, seed0=10_000)
         pg = HipGraph()
@@ -589,6 +757,26 @@ def main() -> int:
                                  "us_per_layer": round(p_layer_us, 2),
                                  "TFLOP/s": round(flops / (p_layer_us * 1e-6) / 1e12, 1),
                                  "frac_fp8_peak": round(flops / (p_layer_us * 1e-6) / 1e12 / FP8_PEAK_TFLOPS, 4)}
+        # the MFMA-bound regime's own roofline object: the GEMM launches alone, per shape, and the
+        # dominant one (gate_up + GeGLU, 61 % of the layer's flops) against the fp8 peak
+        p_gemm_us = gemm_only_times(dev, pl, PREFILL_SET, 816, reps=4, iters=15)
+        per_shape = {name: {"us": round(p_gemm_us[name], 2),
+                            "TFLOP/s": round(2.0 * 816 * N * K / p_gemm_us[name] / 1e6, 1),
+                            "kernel": ops_plan(816, N, K, epi)}
+                     for name, N, K, epi in PREFILL_SET}
+        dom = per_shape["gate_up"]
+        roofline_prefill = {
+            "bound": "mfma", "kernel": "gemm_fp8_big_kernel (gate_up 2048->32768 + GeGLU at M=816: " + dom["kernel"] + ")",
+            "achieved": dom["TFLOP/s"], "peak": FP8_PEAK_TFLOPS, "unit": "TFLOP/s",
+            "frac": round(dom["TFLOP/s"] / FP8_PEAK_TFLOPS, 4), "us": dom["us"],
+            "measured_peak_TFLOPs": measured["fp8_TFLOPs"],
+            "frac_of_measured_peak": round(dom["TFLOP/s"] / measured["fp8_TFLOPs"], 4),
+            "per_shape": per_shape,
+            "layer_gemms_us": round(sum(v["us"] for v in per_shape.values()), 2),
+            "layer_gemms_frac": round(flops / (sum(v["us"] for v in per_shape.values()) * 1e-6) / 1e12 / FP8_PEAK_TFLOPS, 4),
+            "whole_layer_frac": extra["prefill_M816"]["frac_fp8_peak"],
+            "note": "GEMM launches alone on ready codes (graphs of one shape over 4 distinct weight sets); whole_layer_frac "
+                    "includes the four quantizer launches"}
         del pl, pg
     if not args.no_extras:
         dl = decoder_layer_times(dev, layers, M, denoise_steps, max(20, args.steps // 4), 5)
@@ -613,12 +801,7 @@ def main() -> int:
 
     cpu = None
     if not args.no_cpu_baseline:
-        threads = torch.get_num_threads()
-        layer_s, n_iter = cpu_baseline(layers, EXPERT_SET, M)
-        cpu = {"value": round(layer_s * 1e6 * n_layers, 1), "unit": "us per denoise step", "cores": threads,
-               "kind": "port",
-               "sample": f"torch CPU dequantize+matmul incl. quantizer and GeGLU on 1 of {n_layers} layers "
-                         f"(4 linears, M={M}), p50 of {n_iter} passes, scaled x{n_layers}"}
+        cpu = cpu_baseline(layers, EXPERT_SET, M, n_layers)
 
     line = {
         "metric": "p50 \u00b5s per Pi0.5 expert denoise-step linears (fp8 W8A8) + % HBM/MFMA roofline",
@@ -633,7 +816,8 @@ def main() -> int:
                     f"matrices) are read with non-temporal loads, the other {resident_mb:.0f} MB may stay cached from "
                     "step to step; nothing is pinned" if streamed_mb else
                     "311 MB of weights per denoise step cycle through HBM; every matrix is read with ordinary loads")},
-        "roofline": roofline, "cpu_baseline": cpu, "extra": extra,
+        "roofline": roofline, "roofline_prefill": roofline_prefill, "launch_floor": launch_floor,
+        "measured_peaks": measured, "cpu_baseline": cpu, "extra": extra,
     }
     print(json.dumps(line))
     return 0
