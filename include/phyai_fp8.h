@@ -31,7 +31,7 @@
 extern "C" {
 #endif
 
-#define PHYAI_FP8_ABI_VERSION 5
+#define PHYAI_FP8_ABI_VERSION 6
 
 enum {
     PHYAI_FP8_OK = 0,
@@ -223,6 +223,16 @@ int phyai_fp8_describe_plan(int64_t M, int64_t N, int64_t K, int epilogue, char 
  * CPU cast.  Not part of the reference surface.
  */
 int phyai_fp8_debug_cast_e4m3(const float *v, int64_t n, void *codes, void *stream);
+
+/*
+ * Hardware probe: `workgroups` workgroups of four wavefronts each issue iters x 16 independent
+ * v_mfma_f32_32x32x64_f8f6f4 (32 x 32 x 64 x 2 flops each) and touch no memory.  counters (device,
+ * 2 x workgroups 64-bit words) receives per workgroup the shader cycles and the 100 MHz ticks its
+ * loop took; sink is one device float that is never written.  Gives the fp8 MFMA rate the chip
+ * sustains and the clock it holds under that load - the method of the reference's roofline probe
+ * (benchmark/pi05/hardware_probe.py:36-99) applied to the instruction this path is bound by.
+ */
+int phyai_fp8_debug_mfma_rate(int workgroups, int iters, uint64_t *counters, float *sink, void *stream);
 
 #ifdef __cplusplus
 }

@@ -426,6 +426,13 @@ int phyai_fp8_describe_plan(int64_t M, int64_t N, int64_t K, int epilogue, char*
     return len;
 }
 
+int phyai_fp8_debug_mfma_rate(int workgroups, int iters, uint64_t* counters, float* sink, void* stream) {
+    if (workgroups <= 0 || workgroups > 65536 || iters <= 0 || iters > (1 << 20) || !counters || !sink)
+        return fail(PHYAI_FP8_EINVAL, "phyai_fp8_debug_mfma_rate: bad arguments");
+    phyai::launch_mfma_rate(workgroups, iters, reinterpret_cast<unsigned long long*>(counters), sink, static_cast<hipStream_t>(stream));
+    return check_launch("phyai_fp8_debug_mfma_rate");
+}
+
 int phyai_fp8_debug_cast_e4m3(const float* v, int64_t n, void* codes, void* stream) {
     if (n < 0 || (n > 0 && (!v || !codes))) return fail(PHYAI_FP8_EINVAL, "phyai_fp8_debug_cast_e4m3: bad arguments");
     phyai::launch_debug_cast(v, n, codes, static_cast<hipStream_t>(stream));

@@ -14,6 +14,8 @@ int launch_weight_quant(const void* w, int64_t N, int64_t K, int64_t ldw, void* 
 int launch_quant_static(const void* x, int64_t M, int64_t K, int64_t ldx, const float* input_scale,
                         void* xq, hipStream_t st);
 int launch_debug_cast(const float* v, int64_t n, void* codes, hipStream_t st);
+// fp8 MFMA issue-rate probe (probe_kernels.hip): out holds 2 x workgroups 64-bit counters.
+int launch_mfma_rate(int workgroups, int iters, unsigned long long* out, float* sink, hipStream_t st);
 
 // RMSNorm / adaptive RMSNorm with the activation quantizer fused behind it (quant_kernels.hip).
 struct NormQuantArgs {

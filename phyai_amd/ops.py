@@ -499,3 +499,27 @@ def debug_cast_e4m3(v: torch.Tensor) -> torch.Tensor:
     rc = _lib.load().phyai_fp8_debug_cast_e4m3(v.data_ptr(), v.numel(), out.data_ptr(), _stream_ptr())
     _lib.check(rc, "debug_cast_e4m3")
     return out
+
+
+def mfma_rate_probe(workgroups: int = 1024, iters: int = 2000, device: torch.device | None = None) -> dict:
+    """Chip-wide fp8 MFMA issue rate and the shader clock held under that load (a synchronising
+    measurement, not an op): ``{"TFLOPs", "clock_GHz", "cycles_per_mfma"}``."""
+    dev = torch.device("cuda", torch.cuda.current_device()) if device is None else torch.device(device)
+    counters = torch.zeros(2 * workgroups, dtype=torch.int64, device=dev)
+    sink = torch.zeros(1, dtype=torch.float32, device=dev)
+    lib = _lib.load()
+    best = None
+    for _ in range(3):
+        a, b = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        a.record()
+        _lib.check(lib.phyai_fp8_debug_mfma_rate(workgroups, iters, counters.data_ptr(), sink.data_ptr(), _stream_ptr()),
+                   "mfma_rate_probe")
+        b.record()
+        torch.cuda.synchronize()
+        ms = a.elapsed_time(b)
+        best = ms if best is None or ms < best else best
+    c = counters.cpu().reshape(workgroups, 2).double()
+    cycles, ticks = c[:, 0].mean().item(), c[:, 1].mean().item()
+    flops = workgroups * 4 * iters * 16 * (32 * 32 * 64 * 2)
+    return {"TFLOPs": round(flops / (best * 1e-3) / 1e12, 1), "clock_GHz": round(cycles / (ticks / 100e6) / 1e9, 3),
+            "cycles_per_mfma": round(cycles / (iters * 16), 2)}

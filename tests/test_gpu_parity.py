@@ -739,3 +739,13 @@ def test_gemm_against_torch_scaled_mm(dev, monkeypatch, M, N, K, force):
     step = want.float().abs().clamp_min(2.0 ** -126) * 2.0 ** -7
     assert bool(((got.float() - want.float()).abs() <= step).all()), "more than one bf16 step from torch._scaled_mm"
     assert float((got == want).float().mean()) > 0.97
+
+
+def test_mfma_rate_probe_reports_a_plausible_machine(dev):
+    """The hardware probe behind bench.py's measured MFMA peak: 64 cycles per 32 x 32 x 64 fp8 MFMA,
+    a clock between 1 and 3 GHz, and a chip-wide rate that follows from the two."""
+    ops = _ops()
+    r = ops.mfma_rate_probe(workgroups=512, iters=400)
+    assert 60.0 <= r["cycles_per_mfma"] <= 80.0, r
+    assert 1.0 <= r["clock_GHz"] <= 3.0, r
+    assert 1000.0 <= r["TFLOPs"] <= 6000.0, r
