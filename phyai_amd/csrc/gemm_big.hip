@@ -3,7 +3,7 @@
 // workgroup tile is 64*TM x 64*TN: 256 x 256 (TM = TN = 4, one workgroup per CU) for long K,
 // 192 x 128 (TM = 3, TN = 2, two workgroups per CU) when there are plenty of tiles and K is short,
 // 128 x 128 (TM = TN = 2; ring of four stages, or of two with two workgroups per CU) for
-// mid-sized problems.
+// mid-sized problems, 128 x 64 (TM = 2, TN = 1) when even those leave half of the CUs idle.
 //
 // Why 4 x 4 blocks per wavefront for the large tile.  One v_mfma_f32_32x32x64_f8f6f4 takes 64
 // cycles and consumes two 2 KB operand blocks.  A wavefront with TM x TN blocks reads (TM + TN)
@@ -172,7 +172,8 @@ void gemm_fp8_big_kernel(
     constexpr int COPIES = CA + CB;
     constexpr int SLOTS_PER_STAGE = 2 * TM * TN;     // MFMAs of a wavefront per stage
     constexpr int CPS = (COPIES * 2 + SLOTS_PER_STAGE - 1) / SLOTS_PER_STAGE;   // copies per MFMA: done by mid-stage
-    static_assert((TM == TN && TM % 2 == 0) || (TM == 3 && TN == 2) || (TM == 7 && TN == 2), "supported wavefront tiles");
+    static_assert((TM == TN && TM % 2 == 0) || (TM == 3 && TN == 2) || (TM == 7 && TN == 2) || (TM == 2 && TN == 1 && !GATED),
+                  "supported wavefront tiles");
     static_assert(BM % 32 == 0 && BN % 32 == 0, "every wavefront copies whole groups of 8 rows");
     static_assert(DEPTH == 2 || DEPTH == 4, "ring depth");
     __shared__ __attribute__((aligned(1024))) uint8_t lds[DEPTH * STAGE_BYTES];
@@ -516,12 +517,13 @@ static double big_fill(int tiles, int slots) {
 }
 
 BigPlan big_plan(int M, int N, int K, int epilogue) {
-    BigPlan pl = {0, 1, 0, 0};
+    BigPlan pl = {0, 0, 1, 0, 0};
     if (K % 128 != 0 || K < 512) return pl;   // slabs come in pairs and must fill the ring
     int forced = -1;
     if (const char* e = tuning_env("PHYAI_FP8_BIG")) forced = atoi(e);   // "0": never; "256"/"192"/"128": force
     if (forced == 0) return pl;
     if (forced == 256 || forced == 224 || forced == 192 || forced == 128) pl.tile = forced;
+    else if (forced == 12864 && !epi_is_gated(epilogue)) { pl.tile = 128; pl.cols = 64; }   // "12864": 128 rows x 64 columns
     else if (M < 128) return pl;
     // 256 x 256 tiles need the fewest bytes from L2 per flop but run one workgroup per CU, so a
     // tile's prologue and epilogue leave the MFMA pipe idle; 192 x 128 tiles fit twice and overlap
@@ -548,10 +550,23 @@ BigPlan big_plan(int M, int N, int K, int epilogue) {
         pl.tile = big_ceil_div(M, 224) == big_ceil_div(M, 256) ? 224 : 256;
     else if (big_tiles(M, N, epilogue, 128, 128) >= 32) pl.tile = 128;   // fewer: the weight-streaming kernel wins
     else return pl;
-    const int tiles = big_tiles(M, N, epilogue, pl.tile, big_tile_cols(pl.tile));
+    if (pl.cols == 0) pl.cols = big_tile_cols(pl.tile);
+    int tiles = big_tiles(M, N, epilogue, pl.tile, pl.cols);
+    // Few 128 x 128 tiles and a plain epilogue: 128 x 64 tiles (2 x 1 blocks per wavefront) put twice
+    // as many CUs to work.  The kernel is bound by LDS bytes, and the narrow tile reads half as many
+    // again per MFMA, so it pays only while the 128 x 128 grid leaves at least half of the CUs idle:
+    // 816 x 2048 x 2048 (112 -> 224 tiles) 12.6 -> 9.7 us, 816 x 2048 x 8192 25.8 (K split in two)
+    // -> 23.1 us unsplit, 500 x 2048 x 2048 12.1 -> 9.3 us; 816 x 2560 x 2048 (140 -> 280 tiles,
+    // a second round) 12.8 -> 15.1 us and stays; K = 16384 is level with the split form and stays.
+    if (forced < 0 && pl.tile == 128 && !epi_is_gated(epilogue) && tiles > 64 && tiles <= 128 && K < 16384) {
+        pl.cols = 64;
+        tiles = big_tiles(M, N, epilogue, 128, 64);
+    }
     pl.tiles = tiles;
     pl.depth = pl.tile == 128 ? 4 : 2;
-    if (pl.tile == 128) {
+    if (pl.tile == 128 && pl.cols == 64) {
+        // always one round of at most 256 workgroups here, or forced: deep ring, no split
+    } else if (pl.tile == 128) {
         // Measured at M = 816: splitting pays for K = 16384 (67 -> 49 us with two splits) and
         // costs for K = 2048 (19 -> 25 us): the partial-sum round trip is worth about 6 us.
         if (tiles < 200 && K >= 8192 && K % 256 == 0) pl.splits = 2;
@@ -563,18 +578,18 @@ BigPlan big_plan(int M, int N, int K, int epilogue) {
     }
     if (const char* e = tuning_env("PHYAI_FP8_BIG_SPLITS")) {
         const int s = atoi(e);
-        if (pl.tile != 192 && pl.tile != 224 && s >= 1 && K % (s * 128) == 0 && K / s >= 512 && tiles * s <= 4096) pl.splits = s;
+        if (pl.tile != 192 && pl.tile != 224 && pl.cols != 64 && s >= 1 && K % (s * 128) == 0 && K / s >= 512 && tiles * s <= 4096) pl.splits = s;
     }
     if (const char* e = tuning_env("PHYAI_FP8_BIG_DEPTH")) {
         const int d = atoi(e);
-        if (pl.tile == 128 && pl.splits == 1 && (d == 2 || d == 4)) pl.depth = d;
+        if (pl.tile == 128 && pl.cols == 128 && pl.splits == 1 && (d == 2 || d == 4)) pl.depth = d;
     }
     return pl;
 }
 
 size_t big_partial_bytes(int M, int N, int epilogue, const BigPlan& pl) {
     if (pl.splits <= 1) return 0;
-    const int bn = big_tile_cols(pl.tile);
+    const int bn = pl.cols;
     return (size_t)big_tiles(M, N, epilogue, pl.tile, bn) * pl.splits * pl.tile * bn * sizeof(float);
 }
 
@@ -654,6 +669,15 @@ int launch_gemm_big(const GemmProblem& g, const BigPlan& pl, hipStream_t st) {
     if (pl.tile == 256) return big_launch_epi<4, 4, 2>(a, g, pl.splits, st);
     if (pl.tile == 224 && pl.splits == 1) return big_launch_epi<7, 2, 2, 1, 4>(a, g, 1, st);
     if (pl.tile == 192 && pl.splits == 1) return big_launch_epi<3, 2, 2>(a, g, 1, st);
+    if (pl.tile == 128 && pl.cols == 64) {
+        if (pl.splits != 1) return -2;
+        switch (g.epilogue) {   // plain epilogues only: one column block per wavefront cannot hold a gate / up pair
+        case EPI_NONE: big_launch<2, 1, 4, EPI_NONE>(a, g, 1, st); return 0;
+        case EPI_GELU_TANH: big_launch<2, 1, 4, EPI_GELU_TANH>(a, g, 1, st); return 0;
+        case EPI_GELU_ERF: big_launch<2, 1, 4, EPI_GELU_ERF>(a, g, 1, st); return 0;
+        default: return -2;
+        }
+    }
     if (pl.tile == 128 && pl.depth == 4) return big_launch_epi<2, 2, 4>(a, g, pl.splits, st);
     if (pl.tile == 128 && pl.splits == 1) return big_launch_epi<2, 2, 2>(a, g, 1, st);
     return -2;

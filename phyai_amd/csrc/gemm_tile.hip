@@ -380,7 +380,7 @@ static GemmChoice choose_gemm(int M, int N, int K, int epilogue, int64_t ldo, bo
     if (skinny_ok && M <= 64) return small();
     if (!tuning_env("PHYAI_FP8_TILE")) {
         const BigPlan bp = big_plan(M, N, K, epilogue);
-        const bool few_small_tiles = bp.tile == 128 && bp.tiles <= 64 && !tuning_env("PHYAI_FP8_BIG");
+        const bool few_small_tiles = bp.tile == 128 && bp.cols == 128 && bp.tiles <= 64 && !tuning_env("PHYAI_FP8_BIG");
         if (bp.tile && out16 && !(few_small_tiles && skinny_ok)) {
             c.kind = GemmChoice::BIG;
             c.big = bp;
@@ -416,7 +416,7 @@ int describe_gemm_plan(int M, int N, int K, int epilogue, char* buf, size_t n) {
     case GemmChoice::SKINNY:
         return snprintf(buf, n, "small-m nt=%d mb=%d kpw=%d rounds=%d", c.sk.nt, c.sk.mb, c.sk.kpw, c.sk.rounds);
     case GemmChoice::BIG:
-        return snprintf(buf, n, "tile %dx%d depth=%d splits=%d tiles=%d", c.big.tile, (c.big.tile == 256 || c.big.tile == 224) ? 256 : 128,
+        return snprintf(buf, n, "tile %dx%d depth=%d splits=%d tiles=%d", c.big.tile, c.big.cols,
                         c.big.depth, c.big.splits, c.big.tiles);
     default:
         return snprintf(buf, n, "generic %dx%d splits=%d", c.tc.bm, c.tc.bn, c.tc.splits);

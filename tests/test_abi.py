@@ -84,7 +84,7 @@ def test_kernel_selection_for_the_benchmark_shapes(monkeypatch):
     assert d(1, 12288, 2048).startswith("small-m nt=1 mb=1")
     # prefix prefill, M = 816
     assert d(816, 2560, 2048) == "tile 128x128 depth=4 splits=1 tiles=140"
-    assert d(816, 2048, 2048) == "tile 128x128 depth=4 splits=1 tiles=112"
+    assert d(816, 2048, 2048) == "tile 128x64 depth=4 splits=1 tiles=224"      # 112 tiles of 128 x 128 would idle half the CUs
     assert d(816, 32768, 2048, "geglu_tanh") == "tile 224x256 depth=2 splits=1 tiles=512"   # four tile rows either way: less padding
     assert d(816, 2048, 16384) == "tile 128x128 depth=4 splits=2 tiles=112"
     # batched serving and the DiT block
@@ -105,7 +105,9 @@ def test_kernel_selection_for_the_benchmark_shapes(monkeypatch):
     assert d(100, 2560, 1024) == "small-m nt=2 mb=3 kpw=1 rounds=1"  # 240 workgroups x 5 blocks
     assert d(100, 8192, 1024, "geglu_tanh") == "small-m nt=4 mb=4 kpw=1 rounds=1"
     assert d(1000, 1024, 4096) == "small-m nt=4 mb=4 kpw=1 rounds=4"
-    assert d(1100, 1024, 4096) == "tile 128x128 depth=4 splits=1 tiles=72"
+    assert d(1100, 1024, 4096) == "tile 128x64 depth=4 splits=1 tiles=144"
+    assert d(816, 2048, 8192) == "tile 128x64 depth=4 splits=1 tiles=224"      # instead of 128 x 128 with K split in two
+    assert d(816, 4096, 2048, "geglu_tanh") == "tile 128x128 depth=4 splits=1 tiles=224"   # gated: no 64-column tile
     # what the fast kernels refuse goes to the generic one
     assert d(300, 384, 272).startswith("generic ")
     with pytest.raises(RuntimeError, match="multiples of 16"):
