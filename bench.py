@@ -754,7 +754,9 @@ def main() -> int:
                                  "min": round(srt[0] * 1e3 / denoise_steps, 2), "replays": len(srt)}}
     roofline_prefill = None
     if not args.no_prefill:
-        pl = make_layers(dev, PREFILL_SET, 816, 4, seed0=10_000)
+        # all 18 layers of the prefix backbone in one graph (2 GB of fp8 weights): with a handful of
+        # layers the ~20 us a graph launch costs would be a few us per layer
+        pl = make_layers(dev, PREFILL_SET, 816, n_layers, seed0=10_000)
         pg = HipGraph()
         pg.capture(lambda: run_layers(pl, PREFILL_SET), {})
         pts, _ = time_replays(pg, 30, 3)
@@ -767,7 +769,7 @@ def main() -> int:
                                  "frac_fp8_peak": round(flops / (p_layer_us * 1e-6) / 1e12 / FP8_PEAK_TFLOPS, 4)}
         # the MFMA-bound regime's own roofline object: the GEMM launches alone, per shape, and the
         # dominant one (gate_up + GeGLU, 61 % of the layer's flops) against the fp8 peak
-        p_gemm_us = gemm_only_times(dev, pl, PREFILL_SET, 816, reps=4, iters=15)
+        p_gemm_us = gemm_only_times(dev, pl, PREFILL_SET, 816, reps=1, iters=15)
         per_shape = {name: {"us": round(p_gemm_us[name], 2),
                             "TFLOP/s": round(2.0 * 816 * N * K / p_gemm_us[name] / 1e6, 1),
                             "kernel": ops_plan(816, N, K, epi)}
@@ -783,7 +785,7 @@ def main() -> int:
             "layer_gemms_us": round(sum(v["us"] for v in per_shape.values()), 2),
             "layer_gemms_frac": round(flops / (sum(v["us"] for v in per_shape.values()) * 1e-6) / 1e12 / FP8_PEAK_TFLOPS, 4),
             "whole_layer_frac": extra["prefill_M816"]["frac_fp8_peak"],
-            "note": "GEMM launches alone on ready codes (graphs of one shape over 4 distinct weight sets); whole_layer_frac "
+            "note": "GEMM launches alone on ready codes (graphs of one shape over the 18 layers' distinct weights); whole_layer_frac "
                     "includes the four quantizer launches"}
         del pl, pg
     if not args.no_extras:

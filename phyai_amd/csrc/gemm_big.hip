@@ -554,11 +554,12 @@ BigPlan big_plan(int M, int N, int K, int epilogue) {
     int tiles = big_tiles(M, N, epilogue, pl.tile, pl.cols);
     // Few 128 x 128 tiles and a plain epilogue: 128 x 64 tiles (2 x 1 blocks per wavefront) put twice
     // as many CUs to work.  The kernel is bound by LDS bytes, and the narrow tile reads half as many
-    // again per MFMA, so it pays only while the 128 x 128 grid leaves at least half of the CUs idle:
-    // 816 x 2048 x 2048 (112 -> 224 tiles) 12.6 -> 9.7 us, 816 x 2048 x 8192 25.8 (K split in two)
-    // -> 23.1 us unsplit, 500 x 2048 x 2048 12.1 -> 9.3 us; 816 x 2560 x 2048 (140 -> 280 tiles,
-    // a second round) 12.8 -> 15.1 us and stays; K = 16384 is level with the split form and stays.
-    if (forced < 0 && pl.tile == 128 && !epi_is_gated(epilogue) && tiles > 64 && tiles <= 128 && K < 16384) {
+    // again per MFMA, so it pays only while the 128 x 128 grid leaves at least half of the CUs idle
+    // (weights from HBM, 18 weight sets): 816 x 2048 x 2048 (112 -> 224 tiles) 11.4 -> 8.9 us,
+    // 816 x 2048 x 4096 17.7 -> 13.8 us, 1100 x 1024 x 4096 16.6 -> 12.4 us; 816 x 2560 x 2048
+    // (140 -> 280 tiles, a second round) 12.8 -> 15.1 us and stays; from K = 8192 on the 128 x 128
+    // form with K split in two is level or ahead (27.9 against 28.7 us, K = 16384: 44 against 51).
+    if (forced < 0 && pl.tile == 128 && !epi_is_gated(epilogue) && tiles > 64 && tiles <= 128 && K < 8192) {
         pl.cols = 64;
         tiles = big_tiles(M, N, epilogue, 128, 64);
     }

@@ -106,7 +106,8 @@ def test_kernel_selection_for_the_benchmark_shapes(monkeypatch):
     assert d(100, 8192, 1024, "geglu_tanh") == "small-m nt=4 mb=4 kpw=1 rounds=1"
     assert d(1000, 1024, 4096) == "small-m nt=4 mb=4 kpw=1 rounds=4"
     assert d(1100, 1024, 4096) == "tile 128x64 depth=4 splits=1 tiles=144"
-    assert d(816, 2048, 8192) == "tile 128x64 depth=4 splits=1 tiles=224"      # instead of 128 x 128 with K split in two
+    assert d(816, 2048, 4096) == "tile 128x64 depth=4 splits=1 tiles=224"
+    assert d(816, 2048, 8192) == "tile 128x128 depth=4 splits=2 tiles=112"     # long K: the split form is level or ahead
     assert d(816, 4096, 2048, "geglu_tanh") == "tile 128x128 depth=4 splits=1 tiles=224"   # gated: no 64-column tile
     # what the fast kernels refuse goes to the generic one
     assert d(300, 384, 272).startswith("generic ")
