@@ -7,13 +7,9 @@
 // e4m3fn and stores 8 codes per 64-bit store.
 #include "fp8_device.h"
 #include "launch.h"
+#include "quant_device.h"
 
 namespace phyai {
-
-enum QuantMode : int {
-    QUANT_ACT_DYNAMIC = 0,  // bf16 amax floored at bf16(1e-12); scale = fp32(bf16(amax/448)); no clamp
-    QUANT_WEIGHT = 1,       // fp32 amax/448 floored at FLT_MIN; clamp to +-448
-};
 
 template <int THREADS>
 __device__ __forceinline__ uint32_t block_max_u32(uint32_t v, uint32_t* smem) {
@@ -29,85 +25,6 @@ __device__ __forceinline__ uint32_t block_max_u32(uint32_t v, uint32_t* smem) {
         v = r;
     }
     return v;
-}
-
-__device__ __forceinline__ uint32_t absmax8(uint4 q, uint32_t m) {
-    const uint32_t w[4] = {q.x, q.y, q.z, q.w};
-#pragma unroll
-    for (int i = 0; i < 4; ++i) {
-        uint32_t lo = w[i] & 0x7FFFu, hi = (w[i] >> 16) & 0x7FFFu;
-        m = lo > m ? lo : m;
-        m = hi > m ? hi : m;
-    }
-    return m;
-}
-
-// Divisor of one row.  The reference divides every element by the row scale with an IEEE fp32
-// division.  For a finite scale the same quotient bits come from a multiplication by the
-// (correctly rounded) reciprocal followed by one residual correction,
-//     q0 = x * r;   q = fma(fma(-q0, s, x), r, q0),
-// which is exact whenever the true quotient is representable and within one ulp otherwise.
-// Both operands are bf16 values (8 significant bits), so a quotient is either exactly on an
-// e4m3 rounding boundary or at least 2^-13 (relative) away from it, far more than an ulp: the
-// codes are identical to those of the true division.  This is verified exhaustively on the
-// device over every finite bf16 value against every possible scale.  Rows with a non-finite
-// scale (an Inf or NaN in the row) take the true division.
-struct RowDivisor {
-    float s, r;
-    bool fast;
-};
-__device__ __forceinline__ RowDivisor make_divisor(float s) {
-    RowDivisor d;
-    d.s = s;
-    d.fast = (__float_as_uint(s) & 0x7FFFFFFFu) < 0x7F800000u;
-    d.r = 1.0f / s;
-    return d;
-}
-__device__ __forceinline__ float div_exact(float x, const RowDivisor& d) {
-    const float q0 = x * d.r;
-    const float q = __builtin_fmaf(__builtin_fmaf(-q0, d.s, x), d.r, q0);
-    return __builtin_copysignf(q, x);  // the scale is positive; keeps -0 -> -0 (the sum above gives +0)
-}
-
-template <int MODE>
-__device__ __forceinline__ uint2 encode8(uint4 q, const RowDivisor& d) {
-    const uint32_t w[4] = {q.x, q.y, q.z, q.w};
-    uint32_t c[4];
-    if (MODE == QUANT_ACT_DYNAMIC && d.fast) {
-        // every |x| <= amax is finite, so |x / s| < 464: the hardware convert needs no guard
-#pragma unroll
-        for (int i = 0; i < 4; ++i) {
-            const float a = div_exact(bf16_bits_to_f32(w[i] & 0xFFFFu), d);
-            const float b = div_exact(bf16_bits_to_f32(w[i] >> 16), d);
-            c[i] = (uint32_t)__builtin_amdgcn_cvt_pk_fp8_f32(a, b, 0, false) & 0xFFFFu;
-        }
-    } else {
-#pragma unroll
-        for (int i = 0; i < 4; ++i) {
-            float a = bf16_bits_to_f32(w[i] & 0xFFFFu) / d.s;
-            float b = bf16_bits_to_f32(w[i] >> 16) / d.s;
-            if constexpr (MODE == QUANT_WEIGHT) {
-                a = fminf(fmaxf(a, -kFp8Max), kFp8Max);
-                b = fminf(fmaxf(b, -kFp8Max), kFp8Max);
-            }
-            c[i] = e4m3_pack2(a, b);
-        }
-    }
-    return make_uint2(c[0] | (c[1] << 16), c[2] | (c[3] << 16));
-}
-
-// Row absmax as bf16 bits.  |bf16| bit patterns order like the values they
-// encode, so an unsigned max over (bits & 0x7FFF) is the bf16 amax; a NaN in the
-// row has the largest pattern and therefore wins, as torch.amax propagates it.
-template <int MODE>
-__device__ __forceinline__ float scale_from_amax_bits(uint32_t amax_bits) {
-    if constexpr (MODE == QUANT_ACT_DYNAMIC) {
-        amax_bits = amax_bits < kAmaxFloorBf16 ? kAmaxFloorBf16 : amax_bits;
-        return bf16_bits_to_f32(f32_to_bf16_bits(bf16_bits_to_f32(amax_bits) / kFp8Max));
-    } else {
-        float s = bf16_bits_to_f32(amax_bits) / kFp8Max;
-        return s >= 1.17549435e-38f ? s : 1.17549435e-38f;
-    }
 }
 
 // A tensor that is far larger than the caches and read once is loaded without keeping its lines
