@@ -389,7 +389,7 @@ def launch_floor_us(dev, nodes=2000):
 def ops_plan(M, N, K, epi):
     from phyai_amd import ops
 
-    return ops.describe_plan(M, N, K, epi)
+    return ops.describe_linear_plan(M, N, K, epi)
 
 
 def time_replays(graph, n, warmup):
@@ -408,9 +408,27 @@ def time_replays(graph, n, warmup):
     return [a.elapsed_time(b) for a, b in evs], wall
 
 
+def one_launch(M, N, K, epi) -> bool:
+    """Does the whole linear run as one kernel (the GEMM that quantizes its own token rows)?"""
+    from phyai_amd import ops
+
+    return ops.describe_linear_plan(M, N, K, epi).startswith("one launch")
+
+
+def weight_kernel_launch(xq, xs, t):
+    """The kernel of a linear that reads its weights: the whole linear where that is one kernel,
+    else the GEMM on codes and scales the quantizer left (its launch is not part of this figure)."""
+    from phyai_amd import ops
+
+    if one_launch(t["x"].shape[0], t["N"], t["K"], t["epi"]):
+        ops.fp8_linear(t["x"], t["w"], t["ws"], None, epilogue=t["epi"], out=t["out"], stream_weights=t.get("stream", False))
+    else:
+        ops.fp8_gemm(xq, xs, t["w"], t["ws"], None, epilogue=t["epi"], out=t["out"], stream_weights=t.get("stream", False))
+
+
 def gemm_only_times(dev, layers, shapes, M, reps=8, iters=30):
-    """Average launch duration of the GEMM kernel per shape: a graph holding only
-    pre-quantized GEMM launches (reps passes over the distinct per-layer weights)."""
+    """Average launch duration of the weight-reading kernel per shape: a graph holding only those
+    launches (reps passes over the distinct per-layer weights)."""
     from phyai_amd import ops
     from phyai_amd.runtime import HipGraph
 
@@ -425,8 +443,7 @@ def gemm_only_times(dev, layers, shapes, M, reps=8, iters=30):
         def fn():
             for _ in range(reps):
                 for xq, xs, t in pre:
-                    ops.fp8_gemm(xq, xs, t["w"], t["ws"], None, epilogue=t["epi"], out=t["out"],
-                                 stream_weights=t.get("stream", False))
+                    weight_kernel_launch(xq, xs, t)
 
         g = HipGraph()
         g.capture(fn, {})
@@ -437,8 +454,8 @@ def gemm_only_times(dev, layers, shapes, M, reps=8, iters=30):
 
 
 def gemm_only_layer_time(dev, layers, shapes, reps=8, iters=30):
-    """Average duration of one layer's GEMM launches in the order and under the cache conditions of
-    the benchmark: a graph holding only pre-quantized GEMM launches, all shapes of a layer, layer
+    """Average duration of one layer's weight-reading kernels in the order and under the cache conditions
+    of the benchmark: a graph holding only those launches, all shapes of a layer, layer
     after layer (the whole 311 MB of weights per pass, so no matrix is cache-warm by accident; a
     graph of one shape alone holds 47-151 MB, which fits the 256 MB Infinity Cache)."""
     from phyai_amd import ops
@@ -454,8 +471,7 @@ def gemm_only_layer_time(dev, layers, shapes, reps=8, iters=30):
     def fn():
         for _ in range(reps):
             for xq, xs, t in pre:
-                ops.fp8_gemm(xq, xs, t["w"], t["ws"], None, epilogue=t["epi"], out=t["out"],
-                             stream_weights=t.get("stream", False))
+                weight_kernel_launch(xq, xs, t)
 
     g = HipGraph()
     g.capture(fn, {})
@@ -721,11 +737,14 @@ def main() -> int:
     roofline = {
         "bound": "hbm", "achieved": round(achieved, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
         "frac": round(achieved / HBM_PEAK_GBS, 4), "traffic": profiled_layer_traffic(),
-        "kernel": "gemm_fp8_skinny_kernel (M=50, four expert shapes)",
+        "kernel": " + ".join(sorted({"gemm_fp8_fusedq_kernel" if one_launch(M, N, K, epi) else "gemm_fp8_skinny_kernel"
+                                     for _, N, K, epi in EXPERT_SET})) + " (M=50, four expert shapes)",
         "bytes_per_layer": layer_bytes, "us_per_layer": round(layer_us, 3),
-        "note": "achieved = bytes_per_layer / us_per_layer, the four GEMM launches of a layer timed in a graph of GEMM "
-                "launches only that walks all 18 layers (311 MB of weights per pass); per_shape times come from graphs "
-                "of one shape alone, whose 47-151 MB of weights fit the Infinity Cache",
+        "note": "achieved = bytes_per_layer / us_per_layer, the four weight-reading launches of a layer (the whole "
+                "linear where it is one kernel that quantizes its own rows, else the GEMM behind the quantizer) timed "
+                "in a graph of those launches only that walks all 18 layers (311 MB of weights per pass); per_shape "
+                "times come from graphs of one shape alone, whose 47-151 MB of weights fit the Infinity Cache",
+        "plans": {name: ops_plan(M, N, K, epi) for name, N, K, epi in EXPERT_SET},
         "per_shape": {name: {"us": round(per_launch_us[name], 3),
                              "GB/s": round(algorithmic_bytes(M, N, K, epi) / per_launch_us[name] / 1e3, 1)}
                       for name, N, K, epi in EXPERT_SET},
@@ -737,14 +756,16 @@ def main() -> int:
         roofline["measured_peak_GBps"] = measured["copy_GBps"]
         roofline["frac_of_measured_peak"] = round(achieved / measured["copy_GBps"], 4)
     node_us = launch_floor_us(dev)
-    nodes_per_layer = 2 * len(EXPERT_SET)          # a quantizer and a GEMM per linear
+    # one kernel per linear where it quantizes its own rows, else a quantizer and a GEMM
+    nodes_per_layer = sum(1 if one_launch(M, N, K, epi) else 2 for _, N, K, epi in EXPERT_SET)
     floor_us = node_us * nodes_per_layer
     launch_floor = {
         "node_us": round(node_us, 3), "nodes_per_layer": nodes_per_layer, "floor_us_per_layer": round(floor_us, 2),
         "floor_us_per_denoise_step": round(floor_us * n_layers, 1),
         "ceiling_whole_path_frac": round(layer_bytes / (floor_us * 1e-6) / 1e9 / HBM_PEAK_GBS, 4),
         "note": "time of a kernel node that moves nothing, times the nodes a layer's four quantized linears take "
-                "(quantizer + GEMM each): no kernel, however fast, brings the layer below floor_us_per_layer in this "
+                "(one where the GEMM quantizes its own rows, else quantizer + GEMM): no kernel, however fast, brings "
+                "the layer below floor_us_per_layer in this "
                 "structure, i.e. the whole path cannot exceed ceiling_whole_path_frac of HBM peak"}
 
     # ---- prefix prefill (M = 816): MFMA-bound regime -----------------------------

@@ -31,7 +31,7 @@
 extern "C" {
 #endif
 
-#define PHYAI_FP8_ABI_VERSION 6
+#define PHYAI_FP8_ABI_VERSION 7
 
 enum {
     PHYAI_FP8_OK = 0,
@@ -128,6 +128,13 @@ int phyai_fp8_gemm(const void *xq, const float *x_scale, int x_scale_is_scalar,
  * The whole quantized linear: per-token quantization of bf16 x followed by the
  * GEMM above, as one call.  Replaces TorchKernel._fp8_per_channel
  * (layers/linear/backends/torch.py:155-176) end to end.
+ *
+ * Up to 64 token rows, K <= 2048 (a multiple of 128), with x and its row stride 16-byte
+ * aligned and a grid that fits the chip at once, this is ONE kernel: every workgroup
+ * quantizes the token rows it multiplies (same codes, same scales, same output bits as
+ * the two launches) and the workspace is not touched.  Otherwise the quantizer writes
+ * codes and scales into the workspace and a GEMM kernel follows.
+ * phyai_fp8_describe_linear_plan tells which.
  */
 int phyai_fp8_linear(const void *x, int64_t ldx, const void *w, const float *w_scale,
                      const void *bias, void *out, int64_t ldo, int64_t M, int64_t N,
@@ -216,6 +223,13 @@ int phyai_fp8_adarmsnorm_quant(const void *x, int64_t ldx, const void *modulatio
  * layers/linear/dispatch.py:28-95); this is for logs and for tests of the selection rules.
  */
 int phyai_fp8_describe_plan(int64_t M, int64_t N, int64_t K, int epilogue, char *buf, size_t n);
+
+/*
+ * The same for phyai_fp8_linear (bf16 activations in, dense rows): either
+ *   "one launch: small-m rows=16 nt=4 kpw=1 grid=40x4"     the kernel that quantizes its own token rows
+ * or "quantizer + " followed by what phyai_fp8_describe_plan reports.  Host only.
+ */
+int phyai_fp8_describe_linear_plan(int64_t M, int64_t N, int64_t K, int epilogue, char *buf, size_t n);
 
 /*
  * Test hook: run the device fp32 -> e4m3fn cast used by the quantizers over n

@@ -13,7 +13,7 @@ import subprocess
 _PKG = os.path.dirname(os.path.abspath(__file__))
 LIB_PATH = os.path.join(_PKG, "lib", "libphyai_fp8.so")
 CSRC_DIR = os.path.join(_PKG, "csrc")
-ABI_VERSION = 6
+ABI_VERSION = 7
 
 # name -> (restype, argtypes); mirrors include/phyai_fp8.h one to one.
 _i64, _vp, _int, _sz = ctypes.c_int64, ctypes.c_void_p, ctypes.c_int, ctypes.c_size_t
@@ -35,6 +35,7 @@ SIGNATURES: dict[str, tuple[object, list[object]]] = {
     "phyai_fp8_adarmsnorm_quant": (_int, [_vp, _i64, _vp, _i64, _i64, _i64, _i64, ctypes.c_float, _vp, _i64, _vp,
                                           _i64, _vp, _vp, _vp]),
     "phyai_fp8_describe_plan": (_int, [_i64, _i64, _i64, _int, ctypes.c_char_p, _sz]),
+    "phyai_fp8_describe_linear_plan": (_int, [_i64, _i64, _i64, _int, ctypes.c_char_p, _sz]),
     "phyai_fp8_debug_cast_e4m3": (_int, [_vp, _i64, _vp, _vp]),
     "phyai_fp8_debug_mfma_rate": (_int, [_int, _int, _vp, _vp, _vp]),
 }

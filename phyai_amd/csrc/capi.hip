@@ -172,7 +172,7 @@ int check_residual(const char* fn, const ResidualSpec& r, int64_t M, int64_t N, 
 int prepare_gemm(const char* fn, const void* xq, const float* x_scale, int x_scale_is_scalar, const void* w,
                  const float* w_scale, const void* bias, const ResidualSpec& res, void* out, int64_t ldo, int64_t M,
                  int64_t N, int64_t K, int flagged_epilogue, void* workspace, size_t workspace_bytes,
-                 phyai::GemmProblem* problem) {
+                 phyai::GemmProblem* problem, const void* x_bf16 = nullptr, int64_t ldx = 0) {
     if (M < 0 || N <= 0 || K <= 0)
         return fail(PHYAI_FP8_EINVAL, "%s: bad shape M=%lld N=%lld K=%lld", fn, (long long)M, (long long)N, (long long)K);
     const int flags = flagged_epilogue & ~PHYAI_FP8_EPILOGUE_MASK;
@@ -207,6 +207,8 @@ int prepare_gemm(const char* fn, const void* xq, const float* x_scale, int x_sca
     g.workspace = workspace;
     g.workspace_bytes = workspace_bytes;
     g.gate_group = 1;
+    g.x_bf16 = static_cast<const uint16_t*>(x_bf16);
+    g.ldx = ldx;
     if (res.residual) {
         g.residual = static_cast<const uint16_t*>(res.residual);
         g.ld_res = res.ld_res;
@@ -248,10 +250,13 @@ int run_linear_at(const char* fn, const void* x, int64_t ldx, const void* w, con
     if (int rc = check_quant_args(fn, x, M, K, ldx, xq)) return rc;
     phyai::GemmProblem g;
     if (int rc = prepare_gemm(fn, xq, xs, 0, w, w_scale, bias, res, out, ldo, M, N, K, epilogue, gemm_ws,
-                              gemm_ws_bytes, &g))
+                              gemm_ws_bytes, &g, x, ldx))
         return rc;
-    phyai::launch_quant_rowwise(x, M, K, ldx, xq, xs, static_cast<hipStream_t>(stream));
-    if (int rc = check_launch(fn)) return rc;
+    // small token counts: one kernel quantizes its rows and multiplies them; otherwise two launches
+    if (!phyai::gemm_quantizes_itself(g)) {
+        phyai::launch_quant_rowwise(x, M, K, ldx, xq, xs, static_cast<hipStream_t>(stream));
+        if (int rc = check_launch(fn)) return rc;
+    }
     return launch_prepared(fn, g, stream);
 }
 
@@ -332,7 +337,7 @@ int phyai_fp8_linear_static(const void* x, int64_t ldx, const void* w, const flo
     if (int rc = check_quant_args(fn, x, M, K, ldx, xq)) return rc;
     phyai::GemmProblem g;
     if (int rc = prepare_gemm(fn, xq, xs, 0, w, w_scale, bias, ResidualSpec{}, out, ldo, M, N, K, epilogue, ws,
-                              gemm_bytes, &g)) {
+                              gemm_bytes, &g, x, ldx)) {
         if (rc == PHYAI_FP8_EWORKSPACE)
             return fail(rc, "%s: this shape needs more scratch than the static array holds (%zu bytes, %zu of them for "
                         "activation codes); use phyai_fp8_linear with a caller-owned workspace", fn, kScratch, xs_bytes + xq_bytes);
@@ -348,8 +353,10 @@ int phyai_fp8_linear_static(const void* x, int64_t ldx, const void* w, const flo
         hipLaunchKernelGGL(zero_header_kernel, dim3((n + 255) / 256), dim3(256), 0, st, reinterpret_cast<uint32_t*>(ws), n);
         if (int rc = check_launch(fn)) return rc;
     }
-    phyai::launch_quant_rowwise(x, M, K, ldx, xq, xs, st);
-    if (int rc = check_launch(fn)) return rc;
+    if (!phyai::gemm_quantizes_itself(g)) {
+        phyai::launch_quant_rowwise(x, M, K, ldx, xq, xs, st);
+        if (int rc = check_launch(fn)) return rc;
+    }
     return launch_prepared(fn, g, stream);
 }
 
@@ -422,6 +429,20 @@ int phyai_fp8_describe_plan(int64_t M, int64_t N, int64_t K, int epilogue, char*
     if (K % 16 != 0 || N % 16 != 0)
         return fail(PHYAI_FP8_EUNSUPPORTED, "phyai_fp8_describe_plan: K=%lld and N=%lld must be multiples of 16", (long long)K, (long long)N);
     const int len = phyai::describe_gemm_plan((int)M, (int)N, (int)K, epilogue, buf, n);
+    buf[n - 1] = 0;
+    return len;
+}
+
+int phyai_fp8_describe_linear_plan(int64_t M, int64_t N, int64_t K, int epilogue, char* buf, size_t n) {
+    if (!buf || n == 0) return fail(PHYAI_FP8_EINVAL, "phyai_fp8_describe_linear_plan: no buffer");
+    buf[0] = 0;
+    if (M < 0 || N <= 0 || K <= 0 || M >= kMaxElems || N >= kMaxElems || K >= kMaxElems)
+        return fail(PHYAI_FP8_EINVAL, "phyai_fp8_describe_linear_plan: bad shape M=%lld N=%lld K=%lld", (long long)M, (long long)N, (long long)K);
+    epilogue &= PHYAI_FP8_EPILOGUE_MASK;
+    if (int rc = check_epilogue(epilogue, N)) return rc;
+    if (K % 16 != 0 || N % 16 != 0)
+        return fail(PHYAI_FP8_EUNSUPPORTED, "phyai_fp8_describe_linear_plan: K=%lld and N=%lld must be multiples of 16", (long long)K, (long long)N);
+    const int len = phyai::describe_linear_plan((int)M, (int)N, (int)K, epilogue, buf, n);
     buf[n - 1] = 0;
     return len;
 }

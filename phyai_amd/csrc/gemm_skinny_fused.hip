@@ -1,0 +1,459 @@
+// The whole quantized linear for small token counts in ONE launch: every workgroup quantizes the
+// activation rows it multiplies, then runs the weight-streaming GEMM of gemm_skinny.hip on them.
+//
+// Two launches (row-wise quantizer, then GEMM) cost two kernel-node floors per linear, and at
+// M = 50 a node floor is as long as the work.  Quantizing inside the GEMM repeats the conversion in
+// every workgroup that shares token rows, so the shape of a workgroup is chosen for that cost:
+//
+//  * total conversions = (column tiles) x M x K, so a workgroup owns MANY weight tiles (NT up to 8:
+//    128 output columns) and FEW token rows (ROWS = 8, 16 or 32), the opposite of the
+//    two-launch kernel's choice; the chip is filled along M instead (grid.y), weight tiles shared
+//    between the workgroups of a tile column come from L2;
+//  * a wavefront converts only the K steps it multiplies (w, w + 8, ...): the bf16 rows of those
+//    steps go global -> VGPR with loads whose arrival is awaited by hand, so that the wait leaves
+//    the younger global -> LDS copies of the weights in flight; conversion then runs while the
+//    weights are still landing;
+//  * the row maximum needs all of K: per-wavefront maxima (packed 16-bit max, then DPP inside the 16
+//    lanes that share a row) meet in a small LDS table, one barrier, and every wavefront derives all
+//    row scales itself (lane l: row l), handing them to the converting lanes with ds_bpermute;
+//  * arithmetic is that of the stand-alone quantizer (quant_device.h): bit-equal codes and scales,
+//    so the output equals quantizer + GEMM bit for bit.
+//
+// Codes are written into the wavefront's own LDS staging slice in the layout the weight-streaming
+// kernel's copies produce (128-byte rows, 16-byte chunks XOR-swizzled by row), and from there on
+// the kernel is that kernel: MFMA over the wavefront's K steps, partial sums through LDS in
+// wavefront order, epilogue of four output columns per lane.
+#include "fp8_device.h"
+#include "launch.h"
+#include "quant_device.h"
+#include "tuning.h"
+#include <stdio.h>
+
+namespace phyai {
+
+constexpr int FQ_WAVES = 8;
+constexpr int FQ_THREADS = FQ_WAVES * kWave;
+
+// A 16-byte load whose arrival the compiler does not track: the value may be used only after
+// landed() has waited for it.
+__device__ __forceinline__ v4i fq_load16_async(const uint8_t* base, uint32_t lane_offset) {
+    v4i v;
+    asm volatile("global_load_dwordx4 %0, %1, %2" : "=v"(v) : "v"(lane_offset), "s"(base) : "memory");
+    return v;
+}
+// At most YOUNGER memory instructions of this wavefront issued after the load are still in flight;
+// ties the register to the wait so that no use can move above it.
+template <int YOUNGER>
+__device__ __forceinline__ void fq_landed(v4i& a) {
+    static_assert(YOUNGER >= 0 && YOUNGER < 64, "vmcnt is a 6-bit counter");
+    asm volatile("s_waitcnt vmcnt(%1)" : "+v"(a) : "n"(YOUNGER) : "memory");
+}
+__device__ __forceinline__ uint4 fq_as_uint4(v4i v) {
+    return make_uint4((uint32_t)v[0], (uint32_t)v[1], (uint32_t)v[2], (uint32_t)v[3]);
+}
+__device__ __forceinline__ v8i fq_join(v4i lo, v4i hi) {
+    v8i f;
+    f[0] = lo[0]; f[1] = lo[1]; f[2] = lo[2]; f[3] = lo[3];
+    f[4] = hi[0]; f[5] = hi[1]; f[6] = hi[2]; f[7] = hi[3];
+    return f;
+}
+__device__ __forceinline__ float fq_bpermute(float v, int src_lane) {
+    return __uint_as_float((uint32_t)__builtin_amdgcn_ds_bpermute(src_lane << 2, (int)__float_as_uint(v)));
+}
+
+// ROWS: token rows per workgroup (8, 16, 32, 64; grid.y workgroups cover M); NT: 16-row weight tiles
+// per workgroup; KPW: K steps per wavefront (K <= 128 * 8 * KPW, one round).
+//
+// Between the row loads and the wait for them the code is straight-line on purpose: the loaded
+// registers are live behind the compiler's back, and any branch there lets it merge values with
+// copies that would read them too early.  Hence the weight copies are issued for every K step slot
+// (a slot past the end copies the last step again; it is never multiplied), which also keeps the
+// number of copies younger than the row loads a compile-time constant, and the cache policy of the
+// weight copies (STREAM: non-temporal) is a template parameter, not a run-time branch.
+template <int ROWS, int NT, int KPW, int EPI, bool STREAM>
+__global__ __launch_bounds__(FQ_THREADS) void gemm_fp8_fusedq_kernel(
+    const uint8_t* __restrict__ a_w, const uint8_t* __restrict__ a_x, const float* __restrict__ a_w_scale,
+    const uint16_t* __restrict__ a_bias, int a_K, int a_N, int a_m_flags, int a_ldx_bytes, uint16_t* __restrict__ a_out,
+    int64_t a_ldo, const ResidualArgs a_res) {
+    const int a_M = a_m_flags & 0x0FFFFFFF;
+    constexpr bool GATED = epi_is_gated(EPI);
+    constexpr int MB = (ROWS + 15) / 16;              // 16-row token blocks (the last one may be half used)
+    constexpr int COLS_PER_TILE = GATED ? 8 : 16;
+    constexpr int BLOCKS = NT + MB;
+    constexpr int RED_PER_WAVE = NT * MB * kWave * (int)sizeof(v4f);
+    constexpr int STAGE_PER_WAVE = KPW * BLOCKS * 2048;
+    constexpr int PER_WAVE = STAGE_PER_WAVE > RED_PER_WAVE ? STAGE_PER_WAVE : RED_PER_WAVE;
+    static_assert(ROWS == 8 || ROWS % 16 == 0, "token rows per workgroup");
+    static_assert(FQ_WAVES * PER_WAVE + FQ_WAVES * 64 * 4 <= 160 * 1024, "staging does not fit the LDS");
+    constexpr int ROLE_ROUNDS = (NT * MB + FQ_WAVES - 1) / FQ_WAVES;
+    auto rows_in_block = [](int mb) constexpr { return ROWS - 16 * mb < 16 ? ROWS - 16 * mb : 16; };
+
+    __shared__ __attribute__((aligned(1024))) uint8_t smem[FQ_WAVES * PER_WAVE];
+    __shared__ uint32_t amax_tbl[FQ_WAVES][64];
+    auto red = [&](int w, int nt, int mb, int l) -> v4f& {
+        return reinterpret_cast<v4f*>(smem + w * PER_WAVE)[(nt * MB + mb) * kWave + l];
+    };
+
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const int l16 = lane & 15, q = lane >> 4;
+    const int M = a_M, N = a_N, K = a_K;
+    const int half_n = N / 2;
+    const int n_out_total = GATED ? half_n : N;
+    const int col0 = blockIdx.x * (COLS_PER_TILE * NT);
+    const int total_steps = K >> 7;
+    const int m_base = blockIdx.y * ROWS;
+
+    // ---- epilogue roles and their column operands (requested first) ------------------------------
+    int e_mb[ROLE_ROUNDS], e_nt[ROLE_ROUNDS], e_m[ROLE_ROUNDS], e_n[ROLE_ROUNDS];
+    bool e_role[ROLE_ROUNDS], e_live[ROLE_ROUNDS];
+    v4f sw4[ROLE_ROUNDS], su4[ROLE_ROUNDS];
+    uint2 bw2[ROLE_ROUNDS], bu2[ROLE_ROUNDS];
+#pragma unroll
+    for (int rr = 0; rr < ROLE_ROUNDS; ++rr) {
+        const int role = rr * FQ_WAVES + wave;
+        e_mb[rr] = role % MB;
+        e_nt[rr] = role / MB;
+        e_role[rr] = (e_nt[rr] < NT) && (!GATED || q < 2);
+        const int r_in = e_mb[rr] * 16 + l16;                 // token row within the workgroup
+        e_m[rr] = m_base + r_in;
+        e_n[rr] = col0 + (e_nt[rr] < NT ? e_nt[rr] : 0) * COLS_PER_TILE + 4 * q;
+        e_live[rr] = e_role[rr] && r_in < ROWS && e_m[rr] < M && e_n[rr] < n_out_total;
+        const int e_n_safe = e_live[rr] ? e_n[rr] : 0;
+        sw4[rr] = *reinterpret_cast<const v4f*>(a_w_scale + e_n_safe);
+        su4[rr] = v4f{0.f, 0.f, 0.f, 0.f};
+        if constexpr (GATED) su4[rr] = *reinterpret_cast<const v4f*>(a_w_scale + half_n + e_n_safe);
+        bw2[rr] = make_uint2(0, 0); bu2[rr] = make_uint2(0, 0);
+        if (a_bias) {
+            bw2[rr] = *reinterpret_cast<const uint2*>(a_bias + e_n_safe);
+            if constexpr (GATED) bu2[rr] = *reinterpret_cast<const uint2*>(a_bias + half_n + e_n_safe);
+        }
+    }
+
+    // ---- 1a. this wavefront's K steps of the activation rows, bf16, straight into registers --------
+    // instruction i of block mb covers rows 4i .. 4i+3 of the block: 16 lanes per row, 16 bytes
+    // (8 elements) per lane, 256 bytes = one K step per row.  Rows past M repeat row M - 1.
+    const int xr = lane >> 4, xc = lane & 15;
+    v4i xv[KPW][MB][4];
+#pragma unroll
+    for (int j = 0; j < KPW; ++j) {
+        const int s = __builtin_amdgcn_readfirstlane(j * FQ_WAVES + wave);
+#pragma unroll
+        for (int mb = 0; mb < MB; ++mb)
+#pragma unroll
+            for (int i = 0; i < 4; ++i) {
+                // The load is unconditional at run time (a K step past the end re-reads the last one:
+                // the same rows, so the row maxima are unchanged, and its codes are never multiplied):
+                // a value that arrives behind the compiler's back must not pass through a conditional
+                // copy before fq_landed() has waited for it.
+                if (4 * i < rows_in_block(mb)) {
+                    int r = m_base + mb * 16 + 4 * i + xr;
+                    r = r < M ? r : M - 1;
+                    const int s_safe = s < total_steps ? s : total_steps - 1;
+                    xv[j][mb][i] = fq_load16_async(a_x + ((size_t)s_safe << 8), (uint32_t)r * (uint32_t)a_ldx_bytes + xc * 16);
+                } else {
+                    xv[j][mb][i] = v4i{0, 0, 0, 0};
+                }
+            }
+    }
+    // ---- 1b. the weights of the same K steps, global -> LDS (as in gemm_skinny.hip) -----------------
+    const int c_row = lane >> 3, c_slot = lane & 7;
+    uint32_t woff[NT][2];
+#pragma unroll
+    for (int hf = 0; hf < 2; ++hf) {
+        const int r16 = hf * 8 + c_row;
+        const uint32_t chunk = (uint32_t)((c_slot ^ ((r16 >> 1) & 7)) << 4);
+#pragma unroll
+        for (int nt = 0; nt < NT; ++nt) {
+            int wr;
+            if constexpr (GATED) {
+                const int g = col0 + nt * 8 + (r16 & 7);
+                wr = (r16 < 8 ? 0 : half_n) + (g < half_n ? g : half_n - 1);
+            } else {
+                const int r = col0 + nt * 16 + r16;
+                wr = r < N ? r : N - 1;
+            }
+            woff[nt][hf] = __umul24((uint32_t)wr, (uint32_t)K) + chunk;
+        }
+    }
+    const uint32_t lds_wave = __builtin_amdgcn_readfirstlane((uint32_t)(uintptr_t)smem + wave * PER_WAVE);
+    uint8_t* my_stage = smem + wave * PER_WAVE;
+#pragma unroll
+    for (int j = 0; j < KPW; ++j) {
+        const int s = __builtin_amdgcn_readfirstlane(j * FQ_WAVES + wave);
+        const int s_safe = s < total_steps ? s : total_steps - 1;
+        const uint32_t dst = lds_wave + j * (BLOCKS * 2048);
+#pragma unroll
+        for (int nt = 0; nt < NT; ++nt)
+#pragma unroll
+            for (int hf = 0; hf < 2; ++hf) {
+                if constexpr (STREAM) copy16_to_lds_nt(a_w + ((size_t)s_safe << 7), woff[nt][hf], dst + (nt * 2 + hf) * 1024);
+                else copy16_to_lds(a_w + ((size_t)s_safe << 7), woff[nt][hf], dst + (nt * 2 + hf) * 1024);
+            }
+    }
+
+    // ---- 1c. row maxima of this wavefront's K steps (the weight copies stay in flight) -------------
+    // exactly KPW * NT * 2 copies are younger than the row loads
+#pragma unroll
+    for (int j = 0; j < KPW; ++j)
+#pragma unroll
+        for (int mb = 0; mb < MB; ++mb)
+#pragma unroll
+            for (int i = 0; i < 4; ++i)
+                if (4 * i < rows_in_block(mb)) fq_landed<KPW * NT * 2>(xv[j][mb][i]);
+#pragma unroll
+    for (int mb = 0; mb < MB; ++mb)
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+            if (4 * i >= rows_in_block(mb)) continue;
+            uint32_t m2 = 0;
+#pragma unroll
+            for (int j = 0; j < KPW; ++j) m2 = absmax8_pk(fq_as_uint4(xv[j][mb][i]), m2);
+            uint32_t v = absmax_finish(m2), o;
+            o = dpp_move_u32<0xB1>(v);  v = o > v ? o : v;      // the 16 lanes of a row
+            o = dpp_move_u32<0x4E>(v);  v = o > v ? o : v;
+            o = dpp_move_u32<0x141>(v); v = o > v ? o : v;
+            o = dpp_move_u32<0x140>(v); v = o > v ? o : v;
+            if (xc == 0) amax_tbl[wave][mb * 16 + 4 * i + xr] = v;
+        }
+    __syncthreads();
+    // every wavefront derives all scales: lane l holds row l's scale and its reciprocal
+    float s_row = 1.0f, r_row = 1.0f;
+    bool slow_row = false;
+    if (lane < ROWS) {
+        uint32_t a = amax_tbl[0][lane];
+#pragma unroll
+        for (int w = 1; w < FQ_WAVES; ++w) a = amax_tbl[w][lane] > a ? amax_tbl[w][lane] : a;
+        s_row = scale_from_amax_bits<QUANT_ACT_DYNAMIC>(a);
+        r_row = 1.0f / s_row;
+        slow_row = (__float_as_uint(s_row) & 0x7FFFFFFFu) >= 0x7F800000u;   // an Inf or NaN in the row
+    }
+    const bool any_slow = __builtin_amdgcn_ballot_w64(slow_row) != 0;       // wavefront-uniform
+    float sa[ROLE_ROUNDS];
+#pragma unroll
+    for (int rr = 0; rr < ROLE_ROUNDS; ++rr) sa[rr] = fq_bpermute(s_row, (e_mb[rr] * 16 + l16) & 63);
+
+    // gated residual: requested now, behind the row loads whose wait counted instructions
+    uint2 res2[ROLE_ROUNDS], gate2[ROLE_ROUNDS];
+#pragma unroll
+    for (int rr = 0; rr < ROLE_ROUNDS; ++rr) { res2[rr] = make_uint2(0, 0); gate2[rr] = make_uint2(0, 0); }
+    if constexpr (EPI == EPI_NONE) {
+#pragma unroll
+        for (int rr = 0; rr < ROLE_ROUNDS; ++rr) {
+            if (a_res.residual != nullptr && e_live[rr]) {
+                res2[rr] = *reinterpret_cast<const uint2*>(a_res.residual + (int64_t)e_m[rr] * a_res.ld_res + e_n[rr]);
+                gate2[rr] = *reinterpret_cast<const uint2*>(
+                    a_res.gate + (int64_t)(e_m[rr] / a_res.gate_group) * a_res.ld_gate + e_n[rr]);
+            }
+        }
+    }
+
+    // ---- 1d. codes into the staging slice, in the layout the copies would have produced -----------
+#pragma unroll
+    for (int mb = 0; mb < MB; ++mb)
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+            if (4 * i >= rows_in_block(mb)) continue;
+            const int r16 = 4 * i + xr;
+            RowDivisor dv;
+            dv.s = fq_bpermute(s_row, mb * 16 + r16);
+            dv.r = fq_bpermute(r_row, mb * 16 + r16);
+            dv.fast = !any_slow;
+            const int at = r16 * 128 + (((xc >> 1) ^ ((r16 >> 1) & 7)) << 4) + (xc & 1) * 8;
+#pragma unroll
+            for (int j = 0; j < KPW; ++j)
+                *reinterpret_cast<uint2*>(my_stage + j * (BLOCKS * 2048) + (NT + mb) * 2048 + at) =
+                    encode8<QUANT_ACT_DYNAMIC>(fq_as_uint4(xv[j][mb][i]), dv);
+        }
+    wait_copies<0>();   // the weights (and everything else this wavefront asked for)
+
+    // ---- 2. MFMA over this wavefront's K steps -------------------------------------------------------
+    v4f acc[NT][MB];
+#pragma unroll
+    for (int nt = 0; nt < NT; ++nt)
+#pragma unroll
+        for (int mb = 0; mb < MB; ++mb) acc[nt][mb] = v4f{0.f, 0.f, 0.f, 0.f};
+    const int swz = (l16 >> 1) & 7;
+    const int rd_lo = l16 * 128 + ((q ^ swz) << 4), rd_hi = l16 * 128 + (((4 + q) ^ swz) << 4);
+#pragma unroll
+    for (int j = 0; j < KPW; ++j) {
+        const int s = __builtin_amdgcn_readfirstlane(j * FQ_WAVES + wave);
+        if (s < total_steps) {
+            const uint8_t* blk = my_stage + j * (BLOCKS * 2048);
+            v8i xb[MB];
+#pragma unroll
+            for (int mb = 0; mb < MB; ++mb)
+                xb[mb] = fq_join(*reinterpret_cast<const v4i*>(blk + (NT + mb) * 2048 + rd_lo),
+                                 *reinterpret_cast<const v4i*>(blk + (NT + mb) * 2048 + rd_hi));
+#pragma unroll
+            for (int nt = 0; nt < NT; ++nt) {
+                const v8i a = fq_join(*reinterpret_cast<const v4i*>(blk + nt * 2048 + rd_lo),
+                                      *reinterpret_cast<const v4i*>(blk + nt * 2048 + rd_hi));
+#pragma unroll
+                for (int mb = 0; mb < MB; ++mb)
+                    acc[nt][mb] = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(a, xb[mb], acc[nt][mb], 0, 0, 0, 0, 0, 0);
+            }
+        }
+    }
+    // the partial sums below overwrite this wavefront's own staging: its reads must be done
+    asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
+
+    // ---- 3. add the eight wavefronts' partial sums, in wavefront order ---------------------------
+#pragma unroll
+    for (int nt = 0; nt < NT; ++nt)
+#pragma unroll
+        for (int mb = 0; mb < MB; ++mb) red(wave, nt, mb, lane) = acc[nt][mb];
+    __syncthreads();
+#pragma unroll
+    for (int rr = 0; rr < ROLE_ROUNDS; ++rr) {
+        if (e_nt[rr] >= NT) continue;   // wavefront-uniform: no block for this wavefront in this round
+        v4f g = red(0, e_nt[rr], e_mb[rr], lane);
+#pragma unroll
+        for (int w = 1; w < FQ_WAVES; ++w) g += red(w, e_nt[rr], e_mb[rr], lane);
+        v4f u = v4f{0.f, 0.f, 0.f, 0.f};
+        if constexpr (GATED) {
+            const int from = ((lane + 32) & 63) << 2;      // the up half of a gated tile sits 32 lanes further on
+#pragma unroll
+            for (int r = 0; r < 4; ++r)
+                u[r] = __uint_as_float((uint32_t)__builtin_amdgcn_ds_bpermute(from, (int)__float_as_uint(g[r])));
+        }
+        if (!e_role[rr]) continue;
+
+        // ---- 4. epilogue (the arithmetic of gemm_skinny.hip, operation for operation) --------------
+        const float bwf[4] = {bf16_bits_to_f32(bw2[rr].x & 0xFFFFu), bf16_bits_to_f32(bw2[rr].x >> 16),
+                              bf16_bits_to_f32(bw2[rr].y & 0xFFFFu), bf16_bits_to_f32(bw2[rr].y >> 16)};
+        const float buf[4] = {bf16_bits_to_f32(bu2[rr].x & 0xFFFFu), bf16_bits_to_f32(bu2[rr].x >> 16),
+                              bf16_bits_to_f32(bu2[rr].y & 0xFFFFu), bf16_bits_to_f32(bu2[rr].y >> 16)};
+        uint32_t o[4];
+        float vf[4];
+#pragma unroll
+        for (int r = 0; r < 4; ++r) {
+            float v = __builtin_fmaf(g[r], sa[rr] * sw4[rr][r], bwf[r]);
+            if constexpr (GATED) {
+                const float up = __builtin_fmaf(u[r], sa[rr] * su4[rr][r], buf[r]);
+                v = apply_act<EPI>(round_bf16(v)) * round_bf16(up);
+            } else if constexpr (EPI != EPI_NONE) {
+                v = apply_act<EPI>(round_bf16(v));
+            }
+            vf[r] = v;
+        }
+        if constexpr (EPI == EPI_NONE) {
+            if (a_res.residual != nullptr) addcmul4(vf, res2[rr], gate2[rr]);
+        }
+#pragma unroll
+        for (int r = 0; r < 4; ++r) o[r] = f32_to_bf16_bits(vf[r]);
+        if (e_live[rr])
+            *reinterpret_cast<uint2*>(a_out + (int64_t)e_m[rr] * a_ldo + e_n[rr]) =
+                make_uint2(o[0] | (o[1] << 16), o[2] | (o[3] << 16));
+    }
+}
+
+// ---- host side -------------------------------------------------------------------------------------
+
+static int fq_ceil_div(int a, int b) { return (a + b - 1) / b; }
+
+static bool fq_fits(int rows, int nt, int kpw) {
+    const int mb = (rows + 15) / 16;
+    const int stage = kpw * (nt + mb) * 2048, redb = nt * mb * 1024;
+    return FQ_WAVES * (stage > redb ? stage : redb) + FQ_WAVES * 64 * 4 <= 160 * 1024;
+}
+
+// Shapes that exist as kernels: (rows, nt) below, with kpw = 1, 2 or 4 as K asks.
+// Beyond K = 2048 only the 16 x 16 shape fits the LDS and every workgroup would pull eight times the
+// bf16 rows it has weights for: measured 7.7 us against 6.6 us for quantizer + GEMM at 50 x 1024 x 4096.
+// (The kernels with four K steps per wavefront stay compiled: the plan can be forced for tests.)
+static const int kFusedMaxK = 2048;
+static const int kFusedShapes[][2] = {{8, 2}, {8, 4}, {16, 1}, {16, 2}, {16, 4}, {16, 8}, {32, 2}, {32, 4}, {64, 2}};
+
+FusedPlan fused_plan(int M, int N, int K, int epilogue, int64_t ldo) {
+    FusedPlan pl = {0, 0, 0, 0, 0};
+    if (const char* e = tuning_env("PHYAI_FP8_FUSED")) { if (atoi(e) == 0) return pl; }
+    if (M < 1 || M > 64 || K % 128 != 0 || K > 4096 || ldo % 4 != 0) return pl;
+    const bool gated = epi_is_gated(epilogue);
+    const int cols = gated ? N / 2 : N;
+    if (cols % 8 != 0) return pl;
+    const int per_wave = fq_ceil_div(K / 128, FQ_WAVES);
+    const int kpw = per_wave > 2 ? 4 : (per_wave > 1 ? 2 : 1);
+    const int per_tile = gated ? 8 : 16;
+    // A workgroup's time: the conversions it repeats (rows x K elements on its 512 lanes) beside the
+    // operand blocks it pulls through its vector cache.  Only grids that fit the 256 CUs at once are
+    // taken: with a second round of workgroups the repeated conversions cost more than the quantizer's
+    // launch (measured at 12288 x 2048 and 32768 x 2048: up to 3 x slower at M = 50), and the ranking
+    // below agrees with the measured order of the shapes at 50 x {2560, 8192} x 1024 and 50 x 1024 x 2048.
+    double best = 1e30;
+    int forced_rows = 0, forced_nt = 0;
+    if (const char* e = tuning_env("PHYAI_FP8_FUSED_PLAN")) sscanf(e, "%d,%d", &forced_rows, &forced_nt);
+    if (K > kFusedMaxK && !forced_rows) return pl;
+    for (const auto& sh : kFusedShapes) {
+        const int rows = sh[0], nt = sh[1];
+        if (!fq_fits(rows, nt, kpw)) continue;
+        if (forced_rows && (rows != forced_rows || nt != forced_nt)) continue;
+        const int tiles = fq_ceil_div(cols, per_tile * nt), msplit = fq_ceil_div(M, rows);
+        if (!forced_rows) {
+            if (rows > 16 && rows >= 2 * M) continue;                           // token blocks that do not exist
+            if ((int64_t)tiles * msplit > 256) continue;
+        }
+        const double conv = (double)rows * K * 5.5 / 64.0;                      // cycles of VALU per workgroup
+        const double pull = (double)(nt * 16 + rows * 2) * K / 50.0;           // bytes through the vector cache
+        const double cost = conv + pull;
+        if (cost < best) { best = cost; pl.rows = rows; pl.nt = nt; pl.tiles = tiles; pl.msplit = msplit; }
+    }
+    pl.kpw = pl.rows ? kpw : 0;
+    return pl;
+}
+
+template <int ROWS, int NT, int KPW, int EPI>
+static int fq_launch_one(const GemmProblem& g, const FusedPlan& pl, hipStream_t st) {
+    if constexpr (FQ_WAVES * (KPW * (NT + (ROWS + 15) / 16) * 2048) + FQ_WAVES * 256 > 160 * 1024) {
+        return -2;
+    } else {
+        if (g.stream_weights)
+            hipLaunchKernelGGL((gemm_fp8_fusedq_kernel<ROWS, NT, KPW, EPI, true>), dim3(pl.tiles, pl.msplit), dim3(FQ_THREADS), 0, st,
+                               g.w, reinterpret_cast<const uint8_t*>(g.x_bf16), g.w_scale, g.bias, g.K, g.N, g.M,
+                               (int)(g.ldx * 2), g.out, g.ldo, residual_of(g));
+        else
+            hipLaunchKernelGGL((gemm_fp8_fusedq_kernel<ROWS, NT, KPW, EPI, false>), dim3(pl.tiles, pl.msplit), dim3(FQ_THREADS), 0, st,
+                               g.w, reinterpret_cast<const uint8_t*>(g.x_bf16), g.w_scale, g.bias, g.K, g.N, g.M,
+                               (int)(g.ldx * 2), g.out, g.ldo, residual_of(g));
+        return 0;
+    }
+}
+
+template <int ROWS, int NT, int EPI>
+static int fq_launch_kpw(const GemmProblem& g, const FusedPlan& pl, hipStream_t st) {
+    switch (pl.kpw) {
+    case 1: return fq_launch_one<ROWS, NT, 1, EPI>(g, pl, st);
+    case 2: return fq_launch_one<ROWS, NT, 2, EPI>(g, pl, st);
+    case 4: return fq_launch_one<ROWS, NT, 4, EPI>(g, pl, st);
+    default: return -2;
+    }
+}
+
+template <int EPI>
+static int fq_launch_epi(const GemmProblem& g, const FusedPlan& pl, hipStream_t st) {
+    switch (pl.rows * 100 + pl.nt) {
+    case 802: return fq_launch_kpw<8, 2, EPI>(g, pl, st);
+    case 804: return fq_launch_kpw<8, 4, EPI>(g, pl, st);
+    case 1601: return fq_launch_kpw<16, 1, EPI>(g, pl, st);
+    case 1602: return fq_launch_kpw<16, 2, EPI>(g, pl, st);
+    case 1604: return fq_launch_kpw<16, 4, EPI>(g, pl, st);
+    case 1608: return fq_launch_kpw<16, 8, EPI>(g, pl, st);
+    case 3202: return fq_launch_kpw<32, 2, EPI>(g, pl, st);
+    case 3204: return fq_launch_kpw<32, 4, EPI>(g, pl, st);
+    case 6402: return fq_launch_kpw<64, 2, EPI>(g, pl, st);
+    default: return -2;
+    }
+}
+
+int launch_gemm_fused(const GemmProblem& g, const FusedPlan& pl, hipStream_t st) {
+    switch (g.epilogue) {
+    case EPI_NONE: return fq_launch_epi<EPI_NONE>(g, pl, st);
+    case EPI_GEGLU_TANH: return fq_launch_epi<EPI_GEGLU_TANH>(g, pl, st);
+    case EPI_GEGLU_ERF: return fq_launch_epi<EPI_GEGLU_ERF>(g, pl, st);
+    case EPI_SWIGLU: return fq_launch_epi<EPI_SWIGLU>(g, pl, st);
+    case EPI_GELU_TANH: return fq_launch_epi<EPI_GELU_TANH>(g, pl, st);
+    case EPI_GELU_ERF: return fq_launch_epi<EPI_GELU_ERF>(g, pl, st);
+    default: return -2;
+    }
+}
+
+}  // namespace phyai

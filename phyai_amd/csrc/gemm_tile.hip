@@ -350,7 +350,8 @@ static int launch_epi(const TileArgs& a, const TileConfig& c, dim3 grid, hipStre
 
 // launch_gemm's choice of kernel for one problem, and the scratch that choice needs.
 struct GemmChoice {
-    enum Kind { SKINNY, BIG, GENERIC } kind;
+    enum Kind { SKINNY, BIG, GENERIC, FUSED } kind;
+    FusedPlan fq;
     SkinnyPlan sk;
     BigPlan big;
     TileConfig tc;
@@ -368,8 +369,14 @@ struct GemmChoice {
 // vec_ok: scales, bias and output are aligned for the weight-streaming kernel's 128- and 64-bit
 // accesses; out16: the output is 16-byte addressable (pointer and row stride), which the pipelined
 // tile kernel's epilogue needs.
-static GemmChoice choose_gemm(int M, int N, int K, int epilogue, int64_t ldo, bool vec_ok, bool out16) {
+// have_x: the bf16 activations are at hand (whole-linear entry points), so a kernel that quantizes
+// its own rows may serve the call.
+static GemmChoice choose_gemm(int M, int N, int K, int epilogue, int64_t ldo, bool vec_ok, bool out16, bool have_x) {
     GemmChoice c = {};
+    if (have_x && vec_ok) {
+        c.fq = fused_plan(M, N, K, epilogue, ldo);
+        if (c.fq.rows) { c.kind = GemmChoice::FUSED; c.need = 0; return c; }
+    }
     const bool skinny_ok = vec_ok && skinny_applicable(M, N, K, epilogue, ldo);
     auto small = [&]() {
         c.kind = GemmChoice::SKINNY;
@@ -400,7 +407,15 @@ static GemmChoice choose_gemm(const GemmProblem& g) {
                         (reinterpret_cast<uintptr_t>(g.bias) % 8 == 0) &&
                         (reinterpret_cast<uintptr_t>(g.out) % 8 == 0);
     const bool out16 = g.ldo % 8 == 0 && (reinterpret_cast<uintptr_t>(g.out) & 15) == 0;
-    return choose_gemm(g.M, g.N, g.K, g.epilogue, g.ldo, vec_ok, out16);
+    const bool have_x = g.x_bf16 != nullptr && (reinterpret_cast<uintptr_t>(g.x_bf16) & 15) == 0 && g.ldx % 8 == 0 &&
+                        (int64_t)g.M * g.ldx * 2 < ((int64_t)1 << 32) && (int64_t)g.N * g.K < ((int64_t)1 << 32) &&
+                        g.K < (1 << 24) && g.N < (1 << 24) && !g.x_scale_is_scalar;
+    return choose_gemm(g.M, g.N, g.K, g.epilogue, g.ldo, vec_ok, out16, have_x);
+}
+
+bool gemm_quantizes_itself(const GemmProblem& g) {
+    if (g.M == 0 || g.N == 0) return false;
+    return choose_gemm(g).kind == GemmChoice::FUSED;
 }
 
 size_t gemm_scratch_need(const GemmProblem& g) {
@@ -411,7 +426,7 @@ size_t gemm_scratch_need(const GemmProblem& g) {
 int describe_gemm_plan(int M, int N, int K, int epilogue, char* buf, size_t n) {
     // operands that satisfy every alignment requirement, dense output
     const int64_t ldo = epi_is_gated(epilogue) ? N / 2 : N;
-    const GemmChoice c = choose_gemm(M, N, K, epilogue, ldo, true, ldo % 8 == 0);
+    const GemmChoice c = choose_gemm(M, N, K, epilogue, ldo, true, ldo % 8 == 0, false);
     switch (c.kind) {
     case GemmChoice::SKINNY:
         return snprintf(buf, n, "small-m nt=%d mb=%d kpw=%d rounds=%d", c.sk.nt, c.sk.mb, c.sk.kpw, c.sk.rounds);
@@ -423,10 +438,21 @@ int describe_gemm_plan(int M, int N, int K, int epilogue, char* buf, size_t n) {
     }
 }
 
+int describe_linear_plan(int M, int N, int K, int epilogue, char* buf, size_t n) {
+    const int64_t ldo = epi_is_gated(epilogue) ? N / 2 : N;
+    const GemmChoice c = choose_gemm(M, N, K, epilogue, ldo, true, ldo % 8 == 0, true);
+    if (c.kind == GemmChoice::FUSED)
+        return snprintf(buf, n, "one launch: small-m rows=%d nt=%d kpw=%d grid=%dx%d", c.fq.rows, c.fq.nt, c.fq.kpw, c.fq.tiles, c.fq.msplit);
+    const int len = snprintf(buf, n, "quantizer + ");
+    if (len < 0 || (size_t)len >= n) return len;
+    return len + describe_gemm_plan(M, N, K, epilogue, buf + len, n - len);
+}
+
 int launch_gemm(const GemmProblem& g, hipStream_t st) {
     if (g.M == 0 || g.N == 0) return 0;
     const GemmChoice ch = choose_gemm(g);
     if (ch.need > 0 && (g.workspace == nullptr || g.workspace_bytes < ch.need)) return -3;
+    if (ch.kind == GemmChoice::FUSED) return launch_gemm_fused(g, ch.fq, st);
     if (ch.kind == GemmChoice::SKINNY) return launch_gemm_skinny(g, ch.sk, st);
     if (ch.kind == GemmChoice::BIG) return launch_gemm_big(g, ch.big, st);
     const TileConfig& c = ch.tc;

@@ -59,6 +59,11 @@ struct GemmProblem {
     int gate_group;
     // Hint: read the weights with non-temporal loads (honoured by the weight-streaming kernel).
     int stream_weights;
+    // Set by the whole-linear entry points: the bf16 activations behind xq / x_scale (row stride ldx
+    // elements).  A kernel that quantizes its own rows reads these and ignores xq / x_scale, which are
+    // then never written; null for the GEMM entry points.
+    const uint16_t* x_bf16;
+    int64_t ldx;
 };
 
 // What the kernels need of the above, by value.
@@ -82,6 +87,11 @@ size_t gemm_workspace_bytes(int64_t M, int64_t N, int64_t K, int epilogue, int64
 // 0 when it uses none, else header + split-K partial sums.  launch_gemm returns -3 with less.
 size_t gemm_scratch_need(const GemmProblem& p);
 int launch_gemm(const GemmProblem& p, hipStream_t st);
+// True when launch_gemm would serve this problem (x_bf16 set) with the kernel that quantizes its own
+// rows: the caller then skips the quantizer launch.
+bool gemm_quantizes_itself(const GemmProblem& p);
+// Text form of the whole-linear choice for aligned operands and dense activations / output.
+int describe_linear_plan(int M, int N, int K, int epilogue, char* buf, size_t n);
 
 // Weight-streaming kernel for M <= 64 (gemm_skinny.hip).  It needs no workspace.
 struct SkinnyPlan {
@@ -95,6 +105,18 @@ struct SkinnyPlan {
 bool skinny_applicable(int M, int N, int K, int epilogue, int64_t ldo);
 SkinnyPlan skinny_plan(int M, int N, int K, int epilogue);
 int launch_gemm_skinny(const GemmProblem& p, const SkinnyPlan& pl, hipStream_t st);
+
+// Small-M GEMM that quantizes its own activation rows (gemm_skinny_fused.hip): the whole linear in
+// one launch.  rows == 0: does not apply.
+struct FusedPlan {
+    int rows;    // token rows per workgroup (8, 16, 32 or 64)
+    int nt;      // 16-row weight tiles per workgroup
+    int kpw;     // K steps per wavefront
+    int tiles;   // workgroups along N
+    int msplit;  // workgroups along M
+};
+FusedPlan fused_plan(int M, int N, int K, int epilogue, int64_t ldo);
+int launch_gemm_fused(const GemmProblem& p, const FusedPlan& pl, hipStream_t st);
 
 // Pipelined tile kernel for large M (gemm_big.hip), 256 x 256 or 128 x 128 tiles; the small
 // tiles may be split along K (partials in the workspace, as for the generic tile kernel).

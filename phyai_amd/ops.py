@@ -120,6 +120,18 @@ def describe_plan(M: int, N: int, K: int, epilogue=EPI_NONE) -> str:
     return buf.value.decode()
 
 
+def describe_linear_plan(M: int, N: int, K: int, epilogue=EPI_NONE) -> str:
+    """What the whole-linear entry point would launch (one kernel that quantizes its own rows, or the
+    quantizer followed by a GEMM); host only."""
+    import ctypes
+
+    buf = ctypes.create_string_buffer(160)
+    rc = _lib.load().phyai_fp8_describe_linear_plan(M, N, K, _epi("describe_linear_plan", epilogue), buf, len(buf))
+    if rc < 0:
+        raise _err("describe_linear_plan", _lib.load().phyai_fp8_last_error().decode())
+    return buf.value.decode()
+
+
 def reserve_workspace(nbytes: int, device: torch.device | None = None) -> torch.Tensor:
     """Make sure the workspace in scope on ``device`` (the enclosing graph's, else the current
     stream's) holds ``nbytes``."""

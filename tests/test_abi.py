@@ -115,6 +115,35 @@ def test_kernel_selection_for_the_benchmark_shapes(monkeypatch):
         d(50, 1000, 1024)
 
 
+def test_whole_linear_selection_one_launch_or_two(monkeypatch):
+    """phyai_fp8_linear runs one kernel that quantizes its own token rows where that was measured
+    faster (up to 64 rows, K <= 2048, a grid of at most 256 workgroups), and quantizer + GEMM
+    elsewhere.  Host only."""
+    from phyai_amd import ops
+
+    for var in ("PHYAI_FP8_FUSED", "PHYAI_FP8_FUSED_PLAN", "PHYAI_FP8_SKINNY_PLAN", "PHYAI_FP8_BIG"):
+        monkeypatch.delenv(var, raising=False)
+    d = ops.describe_linear_plan
+    assert d(50, 2560, 1024) == "one launch: small-m rows=16 nt=4 kpw=1 grid=40x4"
+    assert d(50, 1024, 2048) == "one launch: small-m rows=8 nt=2 kpw=2 grid=32x7"
+    assert d(50, 8192, 1024, "geglu_tanh") == "one launch: small-m rows=16 nt=8 kpw=1 grid=64x4"
+    assert d(50, 4096, 1024) == "one launch: small-m rows=16 nt=4 kpw=1 grid=64x4"
+    assert d(1, 2048, 2048) == "one launch: small-m rows=8 nt=2 kpw=2 grid=64x1"
+    assert d(50, 1024, 4096) == "quantizer + small-m nt=1 mb=1 kpw=4 rounds=1"       # K too long for the LDS
+    assert d(50, 12288, 2048).startswith("quantizer + small-m")                       # more than one round of workgroups
+    assert d(65, 1024, 1024).startswith("quantizer + small-m")
+    assert d(50, 1024, 1040).startswith("quantizer + ")                               # K not a multiple of 128
+    assert d(816, 2048, 2048) == "quantizer + tile 128x64 depth=4 splits=1 tiles=224"
+    monkeypatch.setenv("PHYAI_FP8_FUSED", "0")
+    assert d(50, 2560, 1024) == "quantizer + small-m nt=2 mb=2 kpw=1 rounds=1"
+    monkeypatch.setenv("PHYAI_FP8_FUSED", "1")
+    monkeypatch.setenv("PHYAI_FP8_FUSED_PLAN", "32,2")
+    assert d(50, 2560, 1024) == "one launch: small-m rows=32 nt=2 kpw=1 grid=80x2"
+    assert d(50, 1024, 4096).startswith("quantizer + ")                               # no such kernel at four K steps per wavefront
+    monkeypatch.setenv("PHYAI_FP8_FUSED_PLAN", "16,1")
+    assert d(50, 1024, 4096) == "one launch: small-m rows=16 nt=1 kpw=4 grid=64x4"    # exists, forced for tests only
+
+
 def test_tuning_variables_are_ignored_without_the_switch():
     """A stray PHYAI_FP8_* variable must not change the kernel selection of a process that did not
     set PHYAI_FP8_TUNING (fresh processes: the switch is read once)."""
