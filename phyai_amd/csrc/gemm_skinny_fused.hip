@@ -103,32 +103,6 @@ __global__ __launch_bounds__(FQ_THREADS) void gemm_fp8_fusedq_kernel(
     const int total_steps = K >> 7;
     const int m_base = blockIdx.y * ROWS;
 
-    // ---- epilogue roles and their column operands (requested first) ------------------------------
-    int e_mb[ROLE_ROUNDS], e_nt[ROLE_ROUNDS], e_m[ROLE_ROUNDS], e_n[ROLE_ROUNDS];
-    bool e_role[ROLE_ROUNDS], e_live[ROLE_ROUNDS];
-    v4f sw4[ROLE_ROUNDS], su4[ROLE_ROUNDS];
-    uint2 bw2[ROLE_ROUNDS], bu2[ROLE_ROUNDS];
-#pragma unroll
-    for (int rr = 0; rr < ROLE_ROUNDS; ++rr) {
-        const int role = rr * FQ_WAVES + wave;
-        e_mb[rr] = role % MB;
-        e_nt[rr] = role / MB;
-        e_role[rr] = (e_nt[rr] < NT) && (!GATED || q < 2);
-        const int r_in = e_mb[rr] * 16 + l16;                 // token row within the workgroup
-        e_m[rr] = m_base + r_in;
-        e_n[rr] = col0 + (e_nt[rr] < NT ? e_nt[rr] : 0) * COLS_PER_TILE + 4 * q;
-        e_live[rr] = e_role[rr] && r_in < ROWS && e_m[rr] < M && e_n[rr] < n_out_total;
-        const int e_n_safe = e_live[rr] ? e_n[rr] : 0;
-        sw4[rr] = *reinterpret_cast<const v4f*>(a_w_scale + e_n_safe);
-        su4[rr] = v4f{0.f, 0.f, 0.f, 0.f};
-        if constexpr (GATED) su4[rr] = *reinterpret_cast<const v4f*>(a_w_scale + half_n + e_n_safe);
-        bw2[rr] = make_uint2(0, 0); bu2[rr] = make_uint2(0, 0);
-        if (a_bias) {
-            bw2[rr] = *reinterpret_cast<const uint2*>(a_bias + e_n_safe);
-            if constexpr (GATED) bu2[rr] = *reinterpret_cast<const uint2*>(a_bias + half_n + e_n_safe);
-        }
-    }
-
     // ---- 1a. this wavefront's K steps of the activation rows, bf16, straight into registers --------
     // instruction i of block mb covers rows 4i .. 4i+3 of the block: 16 lanes per row, 16 bytes
     // (8 elements) per lane, 256 bytes = one K step per row.  Rows past M repeat row M - 1.
@@ -216,6 +190,33 @@ __global__ __launch_bounds__(FQ_THREADS) void gemm_fp8_fusedq_kernel(
             if (xc == 0) amax_tbl[wave][mb * 16 + 4 * i + xr] = v;
         }
     __syncthreads();
+    // ---- epilogue roles and their column operands: requested here, off the path from the row loads
+    // to the row maxima, and hidden behind the conversions -------------------------------------------
+    int e_mb[ROLE_ROUNDS], e_nt[ROLE_ROUNDS], e_m[ROLE_ROUNDS], e_n[ROLE_ROUNDS];
+    bool e_role[ROLE_ROUNDS], e_live[ROLE_ROUNDS];
+    v4f sw4[ROLE_ROUNDS], su4[ROLE_ROUNDS];
+    uint2 bw2[ROLE_ROUNDS], bu2[ROLE_ROUNDS];
+#pragma unroll
+    for (int rr = 0; rr < ROLE_ROUNDS; ++rr) {
+        const int role = rr * FQ_WAVES + wave;
+        e_mb[rr] = role % MB;
+        e_nt[rr] = role / MB;
+        e_role[rr] = (e_nt[rr] < NT) && (!GATED || q < 2);
+        const int r_in = e_mb[rr] * 16 + l16;                 // token row within the workgroup
+        e_m[rr] = m_base + r_in;
+        e_n[rr] = col0 + (e_nt[rr] < NT ? e_nt[rr] : 0) * COLS_PER_TILE + 4 * q;
+        e_live[rr] = e_role[rr] && r_in < ROWS && e_m[rr] < M && e_n[rr] < n_out_total;
+        const int e_n_safe = e_live[rr] ? e_n[rr] : 0;
+        sw4[rr] = *reinterpret_cast<const v4f*>(a_w_scale + e_n_safe);
+        su4[rr] = v4f{0.f, 0.f, 0.f, 0.f};
+        if constexpr (GATED) su4[rr] = *reinterpret_cast<const v4f*>(a_w_scale + half_n + e_n_safe);
+        bw2[rr] = make_uint2(0, 0); bu2[rr] = make_uint2(0, 0);
+        if (a_bias) {
+            bw2[rr] = *reinterpret_cast<const uint2*>(a_bias + e_n_safe);
+            if constexpr (GATED) bu2[rr] = *reinterpret_cast<const uint2*>(a_bias + half_n + e_n_safe);
+        }
+    }
+
     // every wavefront derives all scales: lane l holds row l's scale and its reciprocal
     float s_row = 1.0f, r_row = 1.0f;
     bool slow_row = false;
@@ -224,7 +225,7 @@ __global__ __launch_bounds__(FQ_THREADS) void gemm_fp8_fusedq_kernel(
 #pragma unroll
         for (int w = 1; w < FQ_WAVES; ++w) a = amax_tbl[w][lane] > a ? amax_tbl[w][lane] : a;
         s_row = scale_from_amax_bits<QUANT_ACT_DYNAMIC>(a);
-        r_row = 1.0f / s_row;
+        r_row = biased_reciprocal(s_row);
         slow_row = (__float_as_uint(s_row) & 0x7FFFFFFFu) >= 0x7F800000u;   // an Inf or NaN in the row
     }
     const bool any_slow = __builtin_amdgcn_ballot_w64(slow_row) != 0;       // wavefront-uniform
