@@ -25,6 +25,8 @@
 // wavefront order, epilogue of four output columns per lane.
 #include "fp8_device.h"
 #include "launch.h"
+#include <type_traits>
+
 #include "quant_device.h"
 #include "tuning.h"
 #include <stdio.h>
@@ -56,6 +58,12 @@ __device__ __forceinline__ v8i fq_join(v4i lo, v4i hi) {
     f[0] = lo[0]; f[1] = lo[1]; f[2] = lo[2]; f[3] = lo[3];
     f[4] = hi[0]; f[5] = hi[1]; f[6] = hi[2]; f[7] = hi[3];
     return f;
+}
+// m / group for the token rows of this kernel (0 <= m < 64, 1 <= group <= 64) without the integer
+// division sequence: (m + 0.5) / group is at least 0.5 / 64 away from an integer, and the float
+// product with the hardware reciprocal is off by less than 64.5 * 2^-22.
+__device__ __forceinline__ int gate_row_of(int m, int group) {
+    return group == 1 ? m : (int)(((float)m + 0.5f) * __builtin_amdgcn_rcpf((float)group));
 }
 __device__ __forceinline__ float fq_bpermute(float v, int src_lane) {
     return __uint_as_float((uint32_t)__builtin_amdgcn_ds_bpermute(src_lane << 2, (int)__float_as_uint(v)));
@@ -165,6 +173,23 @@ __global__ __launch_bounds__(FQ_THREADS) void gemm_fp8_fusedq_kernel(
             }
     }
 
+    // ---- epilogue roles: index arithmetic in the shadow of the row loads (no memory operation and no
+    // branch here, see above) ---------------------------------------------------------------------------
+    int e_mb[ROLE_ROUNDS], e_nt[ROLE_ROUNDS], e_m[ROLE_ROUNDS], e_n[ROLE_ROUNDS], e_n_safe[ROLE_ROUNDS];
+    bool e_role[ROLE_ROUNDS], e_live[ROLE_ROUNDS];
+#pragma unroll
+    for (int rr = 0; rr < ROLE_ROUNDS; ++rr) {
+        const int role = rr * FQ_WAVES + wave;
+        e_mb[rr] = role % MB;
+        e_nt[rr] = role / MB;
+        e_role[rr] = (e_nt[rr] < NT) && (!GATED || q < 2);
+        const int r_in = e_mb[rr] * 16 + l16;                 // token row within the workgroup
+        e_m[rr] = m_base + r_in;
+        e_n[rr] = col0 + (e_nt[rr] < NT ? e_nt[rr] : 0) * COLS_PER_TILE + 4 * q;
+        e_live[rr] = e_role[rr] && r_in < ROWS && e_m[rr] < M && e_n[rr] < n_out_total;
+        e_n_safe[rr] = e_live[rr] ? e_n[rr] : 0;
+    }
+
     // ---- 1c. row maxima of this wavefront's K steps (the weight copies stay in flight) -------------
     // exactly KPW * NT * 2 copies are younger than the row loads
 #pragma unroll
@@ -190,30 +215,19 @@ __global__ __launch_bounds__(FQ_THREADS) void gemm_fp8_fusedq_kernel(
             if (xc == 0) amax_tbl[wave][mb * 16 + 4 * i + xr] = v;
         }
     __syncthreads();
-    // ---- epilogue roles and their column operands: requested here, off the path from the row loads
-    // to the row maxima, and hidden behind the conversions -------------------------------------------
-    int e_mb[ROLE_ROUNDS], e_nt[ROLE_ROUNDS], e_m[ROLE_ROUNDS], e_n[ROLE_ROUNDS];
-    bool e_role[ROLE_ROUNDS], e_live[ROLE_ROUNDS];
+    // ---- the column operands of the epilogue: requested here, off the path from the row loads to the
+    // row maxima, and hidden behind the conversions ------------------------------------------------------
     v4f sw4[ROLE_ROUNDS], su4[ROLE_ROUNDS];
     uint2 bw2[ROLE_ROUNDS], bu2[ROLE_ROUNDS];
 #pragma unroll
     for (int rr = 0; rr < ROLE_ROUNDS; ++rr) {
-        const int role = rr * FQ_WAVES + wave;
-        e_mb[rr] = role % MB;
-        e_nt[rr] = role / MB;
-        e_role[rr] = (e_nt[rr] < NT) && (!GATED || q < 2);
-        const int r_in = e_mb[rr] * 16 + l16;                 // token row within the workgroup
-        e_m[rr] = m_base + r_in;
-        e_n[rr] = col0 + (e_nt[rr] < NT ? e_nt[rr] : 0) * COLS_PER_TILE + 4 * q;
-        e_live[rr] = e_role[rr] && r_in < ROWS && e_m[rr] < M && e_n[rr] < n_out_total;
-        const int e_n_safe = e_live[rr] ? e_n[rr] : 0;
-        sw4[rr] = *reinterpret_cast<const v4f*>(a_w_scale + e_n_safe);
+        sw4[rr] = *reinterpret_cast<const v4f*>(a_w_scale + e_n_safe[rr]);
         su4[rr] = v4f{0.f, 0.f, 0.f, 0.f};
-        if constexpr (GATED) su4[rr] = *reinterpret_cast<const v4f*>(a_w_scale + half_n + e_n_safe);
+        if constexpr (GATED) su4[rr] = *reinterpret_cast<const v4f*>(a_w_scale + half_n + e_n_safe[rr]);
         bw2[rr] = make_uint2(0, 0); bu2[rr] = make_uint2(0, 0);
         if (a_bias) {
-            bw2[rr] = *reinterpret_cast<const uint2*>(a_bias + e_n_safe);
-            if constexpr (GATED) bu2[rr] = *reinterpret_cast<const uint2*>(a_bias + half_n + e_n_safe);
+            bw2[rr] = *reinterpret_cast<const uint2*>(a_bias + e_n_safe[rr]);
+            if constexpr (GATED) bu2[rr] = *reinterpret_cast<const uint2*>(a_bias + half_n + e_n_safe[rr]);
         }
     }
 
@@ -243,28 +257,51 @@ __global__ __launch_bounds__(FQ_THREADS) void gemm_fp8_fusedq_kernel(
             if (a_res.residual != nullptr && e_live[rr]) {
                 res2[rr] = *reinterpret_cast<const uint2*>(a_res.residual + (int64_t)e_m[rr] * a_res.ld_res + e_n[rr]);
                 gate2[rr] = *reinterpret_cast<const uint2*>(
-                    a_res.gate + (int64_t)(e_m[rr] / a_res.gate_group) * a_res.ld_gate + e_n[rr]);
+                    a_res.gate + (int64_t)gate_row_of(e_m[rr], a_res.gate_group) * a_res.ld_gate + e_n[rr]);
             }
         }
     }
 
     // ---- 1d. codes into the staging slice, in the layout the copies would have produced -----------
+    // (all reciprocals are fetched before the first conversion, and the choice between the two
+    // division forms is made once for the workgroup's rows, not per block of four rows)
+    float r_of[MB][4], s_of[MB][4];
 #pragma unroll
     for (int mb = 0; mb < MB; ++mb)
 #pragma unroll
         for (int i = 0; i < 4; ++i) {
-            if (4 * i >= rows_in_block(mb)) continue;
-            const int r16 = 4 * i + xr;
-            RowDivisor dv;
-            dv.s = fq_bpermute(s_row, mb * 16 + r16);
-            dv.r = fq_bpermute(r_row, mb * 16 + r16);
-            dv.fast = !any_slow;
-            const int at = r16 * 128 + (((xc >> 1) ^ ((r16 >> 1) & 7)) << 4) + (xc & 1) * 8;
-#pragma unroll
-            for (int j = 0; j < KPW; ++j)
-                *reinterpret_cast<uint2*>(my_stage + j * (BLOCKS * 2048) + (NT + mb) * 2048 + at) =
-                    encode8<QUANT_ACT_DYNAMIC>(fq_as_uint4(xv[j][mb][i]), dv);
+            r_of[mb][i] = 1.0f; s_of[mb][i] = 1.0f;
+            if (4 * i < rows_in_block(mb)) r_of[mb][i] = fq_bpermute(r_row, mb * 16 + 4 * i + xr);
         }
+    auto write_codes = [&](auto fast_tag) {
+        constexpr bool FAST = decltype(fast_tag)::value;
+#pragma unroll
+        for (int mb = 0; mb < MB; ++mb)
+#pragma unroll
+            for (int i = 0; i < 4; ++i) {
+                if (4 * i >= rows_in_block(mb)) continue;
+                const int r16 = 4 * i + xr;
+                RowDivisor dv;
+                dv.s = s_of[mb][i];
+                dv.r = r_of[mb][i];
+                dv.fast = FAST;
+                const int at = r16 * 128 + (((xc >> 1) ^ ((r16 >> 1) & 7)) << 4) + (xc & 1) * 8;
+#pragma unroll
+                for (int j = 0; j < KPW; ++j)
+                    *reinterpret_cast<uint2*>(my_stage + j * (BLOCKS * 2048) + (NT + mb) * 2048 + at) =
+                        encode8<QUANT_ACT_DYNAMIC>(fq_as_uint4(xv[j][mb][i]), dv);
+            }
+    };
+    if (!any_slow) {
+        write_codes(std::true_type{});
+    } else {
+#pragma unroll
+        for (int mb = 0; mb < MB; ++mb)
+#pragma unroll
+            for (int i = 0; i < 4; ++i)
+                if (4 * i < rows_in_block(mb)) s_of[mb][i] = fq_bpermute(s_row, mb * 16 + 4 * i + xr);
+        write_codes(std::false_type{});
+    }
     wait_copies<0>();   // the weights (and everything else this wavefront asked for)
 
     // ---- 2. MFMA over this wavefront's K steps -------------------------------------------------------
