@@ -129,7 +129,7 @@ int phyai_fp8_gemm(const void *xq, const float *x_scale, int x_scale_is_scalar,
  * GEMM above, as one call.  Replaces TorchKernel._fp8_per_channel
  * (layers/linear/backends/torch.py:155-176) end to end.
  *
- * Up to 64 token rows, K <= 2048 (a multiple of 128), with x and its row stride 16-byte
+ * Up to 128 token rows, K <= 2048 (a multiple of 128), with x and its row stride 16-byte
  * aligned and a grid that fits the chip at once, this is ONE kernel: every workgroup
  * quantizes the token rows it multiplies (same codes, same scales, same output bits as
  * the two launches) and the workspace is not touched.  Otherwise the quantizer writes

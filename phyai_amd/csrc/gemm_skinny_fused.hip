@@ -59,9 +59,9 @@ __device__ __forceinline__ v8i fq_join(v4i lo, v4i hi) {
     f[4] = hi[0]; f[5] = hi[1]; f[6] = hi[2]; f[7] = hi[3];
     return f;
 }
-// m / group for the token rows of this kernel (0 <= m < 64, 1 <= group <= 64) without the integer
-// division sequence: (m + 0.5) / group is at least 0.5 / 64 away from an integer, and the float
-// product with the hardware reciprocal is off by less than 64.5 * 2^-22.
+// m / group for the token rows of this kernel (0 <= m < 128, 1 <= group <= 128) without the integer
+// division sequence: (m + 0.5) / group is at least 0.5 / 128 away from an integer, and the float
+// product with the hardware reciprocal is off by less than 128.5 * 2^-22.
 __device__ __forceinline__ int gate_row_of(int m, int group) {
     return group == 1 ? m : (int)(((float)m + 0.5f) * __builtin_amdgcn_rcpf((float)group));
 }
@@ -400,12 +400,15 @@ static bool fq_fits(int rows, int nt, int kpw) {
 // bf16 rows it has weights for: measured 7.7 us against 6.6 us for quantizer + GEMM at 50 x 1024 x 4096.
 // (The kernels with four K steps per wavefront stay compiled: the plan can be forced for tests.)
 static const int kFusedMaxK = 2048;
+// Up to 128 token rows the kernel is level with or ahead of quantizer + GEMM as long as a workgroup
+// converts 16 rows or fewer (measured at M = 64 ... 256 on the expert shapes: 32-row workgroups lose).
+static const int kFusedMaxM = 128;
 static const int kFusedShapes[][2] = {{8, 2}, {8, 4}, {16, 1}, {16, 2}, {16, 4}, {16, 8}, {32, 2}, {32, 4}, {64, 2}};
 
 FusedPlan fused_plan(int M, int N, int K, int epilogue, int64_t ldo) {
     FusedPlan pl = {0, 0, 0, 0, 0};
     if (const char* e = tuning_env("PHYAI_FP8_FUSED")) { if (atoi(e) == 0) return pl; }
-    if (M < 1 || M > 64 || K % 128 != 0 || K > 4096 || ldo % 4 != 0) return pl;
+    if (M < 1 || M > kFusedMaxM || K % 128 != 0 || K > 4096 || ldo % 4 != 0) return pl;
     const bool gated = epi_is_gated(epilogue);
     const int cols = gated ? N / 2 : N;
     if (cols % 8 != 0) return pl;
@@ -427,7 +430,7 @@ FusedPlan fused_plan(int M, int N, int K, int epilogue, int64_t ldo) {
         if (forced_rows && (rows != forced_rows || nt != forced_nt)) continue;
         const int tiles = fq_ceil_div(cols, per_tile * nt), msplit = fq_ceil_div(M, rows);
         if (!forced_rows) {
-            if (rows > 16 && rows >= 2 * M) continue;                           // token blocks that do not exist
+            if (rows > 16 && (rows >= 2 * M || M > 64)) continue;              // blocks that do not exist; see kFusedMaxM
             if ((int64_t)tiles * msplit > 256) continue;
         }
         const double conv = (double)rows * K * 5.5 / 64.0;                      // cycles of VALU per workgroup

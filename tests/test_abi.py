@@ -117,7 +117,7 @@ def test_kernel_selection_for_the_benchmark_shapes(monkeypatch):
 
 def test_whole_linear_selection_one_launch_or_two(monkeypatch):
     """phyai_fp8_linear runs one kernel that quantizes its own token rows where that was measured
-    faster (up to 64 rows, K <= 2048, a grid of at most 256 workgroups), and quantizer + GEMM
+    faster (up to 128 rows, K <= 2048, a grid of at most 256 workgroups), and quantizer + GEMM
     elsewhere.  Host only."""
     from phyai_amd import ops
 
@@ -131,7 +131,9 @@ def test_whole_linear_selection_one_launch_or_two(monkeypatch):
     assert d(1, 2048, 2048) == "one launch: small-m rows=8 nt=2 kpw=2 grid=64x1"
     assert d(50, 1024, 4096) == "quantizer + small-m nt=1 mb=1 kpw=4 rounds=1"       # K too long for the LDS
     assert d(50, 12288, 2048).startswith("quantizer + small-m")                       # more than one round of workgroups
-    assert d(65, 1024, 1024).startswith("quantizer + small-m")
+    assert d(100, 2560, 1024) == "one launch: small-m rows=16 nt=8 kpw=1 grid=20x7"   # up to 128 rows, 16 per workgroup
+    assert d(100, 8192, 1024, "geglu_tanh").startswith("quantizer + small-m")          # 16-row workgroups would need two rounds
+    assert d(129, 1024, 1024).startswith("quantizer + small-m")
     assert d(50, 1024, 1040).startswith("quantizer + ")                               # K not a multiple of 128
     assert d(816, 2048, 2048) == "quantizer + tile 128x64 depth=4 splits=1 tiles=224"
     monkeypatch.setenv("PHYAI_FP8_FUSED", "0")

@@ -4,7 +4,7 @@ own activation rows (reference quant/fp8.py:150-155) in front of the fp8 GEMM
 codes, scales and outputs are pinned against the oracle elsewhere.
 
 Every workgroup shape the kernel exists in is forced in turn; the automatic choice is checked
-against the oracle as well, since for M <= 64 it is what `fp8_linear` now runs.
+against the oracle as well, since for M <= 128 it is what `fp8_linear` now runs.
 """
 
 from __future__ import annotations
@@ -54,6 +54,7 @@ CASES = [
     (1, 256, 128, None), (7, 272, 512, "gelu"), (16, 1024, 1024, "swiglu"), (33, 528, 2048, "gelu_tanh"),
     (64, 2048, 4096, "geglu_erf"), (50, 4096, 1024, None), (23, 144, 384, None), (9, 64, 3072, None),
     (64, 288, 256, "geglu_tanh"), (17, 48, 1152, None),
+    (100, 2560, 1024, None), (128, 1024, 2048, None), (77, 528, 512, "gelu"), (90, 1056, 1024, "geglu_tanh"),
 ]
 
 
@@ -102,7 +103,7 @@ def test_every_workgroup_shape_equals_two_launches_bit_for_bit(dev, monkeypatch,
 
 
 @pytest.mark.parametrize("M,N,K,epi", [(50, 4096, 1024, None), (50, 8192, 1024, "geglu_tanh"), (50, 1024, 2048, None),
-                                       (1, 2560, 1024, None), (64, 1024, 1024, "gelu_tanh")])
+                                       (1, 2560, 1024, None), (64, 1024, 1024, "gelu_tanh"), (100, 1024, 2048, None)])
 def test_automatic_choice_is_the_one_launch_kernel_and_matches_the_oracle(dev, M, N, K, epi):
     from oracle import ref
     ops = _ops()
