@@ -552,17 +552,17 @@ def sweep(dev):
 
 
 def probe(dev, layers, M, shapes=EXPERT_SET):
-    """Counter probe: per shape one GEMM launch per layer (distinct weight sets, so the weights
-    come from HBM), then a 64 MiB device-to-device copy whose traffic is known (64 MiB read,
-    64 MiB written) to calibrate the counters."""
+    """Counter probe: per shape one launch per layer of the kernel that reads the weights (the whole
+    linear where it is one kernel, else the GEMM on ready codes; distinct weight sets, so the
+    weights come from HBM), then a 64 MiB device-to-device copy whose traffic is known (64 MiB
+    read, 64 MiB written) to calibrate the counters."""
     from phyai_amd import ops
 
     for name, N, K, epi in shapes:
         pre = [(ops.fp8_quant_rowwise(layer[name]["x"]), layer[name]) for layer in layers]
         torch.cuda.synchronize()
         for (xq, xs), t in pre:
-            ops.fp8_gemm(xq, xs, t["w"], t["ws"], None, epilogue=t["epi"], out=t["out"],
-                         stream_weights=t.get("stream", False))
+            weight_kernel_launch(xq, xs, t)
         torch.cuda.synchronize()
     src = torch.empty(64 << 20, dtype=torch.uint8, device=dev).fill_(1)
     dst = torch.empty_like(src)
@@ -811,9 +811,13 @@ def main() -> int:
         del pl, pg
     if not args.no_extras:
         dl = decoder_layer_times(dev, layers, M, denoise_steps, max(20, args.steps // 4), 5)
+        lin = {name: (1 if one_launch(M, N, K, epi) else 2) for name, N, K, epi in EXPERT_SET}
         extra["expert_step_with_norms_and_residuals_us"] = {
             **dl, "note": "per denoise step, 18 layers: adaptive norm -> qkv, o -> gated residual, adaptive norm -> "
-                          "gate_up+GeGLU, down -> gated residual; separate = 12 kernels per layer, fused = 8"}
+                          "gate_up+GeGLU, down -> gated residual; kernels per layer: separate = "
+                          f"{4 + sum(lin.values())} (2 norms, 2 addcmul, the four linears), fused = "
+                          f"{4 + lin['o'] + lin['down']} (2 norm+quantizer, qkv and gate_up GEMMs on their codes, o and down "
+                          "with the gated residual in the epilogue)"}
         extra["torch_reference_path_us"] = {
             "expert_step": torch_reference_times(dev, layers, EXPERT_SET, denoise_steps, max(10, args.steps // 10), 3),
             "note": "same linears through the reference's own arithmetic on this GPU: torch-op quantizer + "
