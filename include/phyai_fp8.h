@@ -226,7 +226,7 @@ int phyai_fp8_describe_plan(int64_t M, int64_t N, int64_t K, int epilogue, char 
 
 /*
  * The same for phyai_fp8_linear (bf16 activations in, dense rows): either
- *   "one launch: small-m rows=16 nt=4 kpw=1 grid=40x4"     the kernel that quantizes its own token rows
+ *   "one launch: small-m rows=8 nt=5 kpw=1 grid=32x7"      the kernel that quantizes its own token rows
  * or "quantizer + " followed by what phyai_fp8_describe_plan reports.  Host only.
  */
 int phyai_fp8_describe_linear_plan(int64_t M, int64_t N, int64_t K, int epilogue, char *buf, size_t n);

@@ -403,7 +403,7 @@ static const int kFusedMaxK = 2048;
 // Up to 128 token rows the kernel is level with or ahead of quantizer + GEMM as long as a workgroup
 // converts 16 rows or fewer (measured at M = 64 ... 256 on the expert shapes: 32-row workgroups lose).
 static const int kFusedMaxM = 128;
-static const int kFusedShapes[][2] = {{8, 2}, {8, 4}, {16, 1}, {16, 2}, {16, 4}, {16, 8}, {32, 2}, {32, 4}, {64, 2}};
+static const int kFusedShapes[][2] = {{8, 2}, {8, 4}, {8, 5}, {8, 6}, {8, 8}, {16, 1}, {16, 2}, {16, 4}, {16, 8}, {32, 2}, {32, 4}, {64, 2}};
 
 FusedPlan fused_plan(int M, int N, int K, int epilogue, int64_t ldo) {
     FusedPlan pl = {0, 0, 0, 0, 0};
@@ -419,7 +419,8 @@ FusedPlan fused_plan(int M, int N, int K, int epilogue, int64_t ldo) {
     // operand blocks it pulls through its vector cache.  Only grids that fit the 256 CUs at once are
     // taken: with a second round of workgroups the repeated conversions cost more than the quantizer's
     // launch (measured at 12288 x 2048 and 32768 x 2048: up to 3 x slower at M = 50), and the ranking
-    // below agrees with the measured order of the shapes at 50 x {2560, 8192} x 1024 and 50 x 1024 x 2048.
+    // below agrees with the measured order of the shapes at 50 x {1024, 2560, 4096, 8192} x 1024, 16 x 2560 x 1024
+    // and 50 x 1024 x 2048.
     double best = 1e30;
     int forced_rows = 0, forced_nt = 0;
     if (const char* e = tuning_env("PHYAI_FP8_FUSED_PLAN")) sscanf(e, "%d,%d", &forced_rows, &forced_nt);
@@ -435,7 +436,10 @@ FusedPlan fused_plan(int M, int N, int K, int epilogue, int64_t ldo) {
         }
         const double conv = (double)rows * K * 5.5 / 64.0;                      // cycles of VALU per workgroup
         const double pull = (double)(nt * 16 + rows * 2) * K / 50.0;           // bytes through the vector cache
-        const double cost = conv + pull;
+        // workgroups that share a weight tile sit on one XCD (and fetch the tile from HBM once) only when
+        // the tile count is a multiple of 8: 27 tiles instead of 32 made qkv 1.6 x slower
+        const double spread = (msplit > 1 && tiles % 8 != 0) ? 1.6 : 1.0;
+        const double cost = (conv + pull) * spread;
         if (cost < best) { best = cost; pl.rows = rows; pl.nt = nt; pl.tiles = tiles; pl.msplit = msplit; }
     }
     pl.kpw = pl.rows ? kpw : 0;
@@ -474,6 +478,9 @@ static int fq_launch_epi(const GemmProblem& g, const FusedPlan& pl, hipStream_t 
     switch (pl.rows * 100 + pl.nt) {
     case 802: return fq_launch_kpw<8, 2, EPI>(g, pl, st);
     case 804: return fq_launch_kpw<8, 4, EPI>(g, pl, st);
+    case 805: return fq_launch_kpw<8, 5, EPI>(g, pl, st);
+    case 806: return fq_launch_kpw<8, 6, EPI>(g, pl, st);
+    case 808: return fq_launch_kpw<8, 8, EPI>(g, pl, st);
     case 1601: return fq_launch_kpw<16, 1, EPI>(g, pl, st);
     case 1602: return fq_launch_kpw<16, 2, EPI>(g, pl, st);
     case 1604: return fq_launch_kpw<16, 4, EPI>(g, pl, st);

@@ -124,7 +124,7 @@ def test_whole_linear_selection_one_launch_or_two(monkeypatch):
     for var in ("PHYAI_FP8_FUSED", "PHYAI_FP8_FUSED_PLAN", "PHYAI_FP8_SKINNY_PLAN", "PHYAI_FP8_BIG"):
         monkeypatch.delenv(var, raising=False)
     d = ops.describe_linear_plan
-    assert d(50, 2560, 1024) == "one launch: small-m rows=16 nt=4 kpw=1 grid=40x4"
+    assert d(50, 2560, 1024) == "one launch: small-m rows=8 nt=5 kpw=1 grid=32x7"      # half the conversions of 16 x 4
     assert d(50, 1024, 2048) == "one launch: small-m rows=8 nt=2 kpw=2 grid=32x7"
     assert d(50, 8192, 1024, "geglu_tanh") == "one launch: small-m rows=16 nt=8 kpw=1 grid=64x4"
     assert d(50, 4096, 1024) == "one launch: small-m rows=16 nt=4 kpw=1 grid=64x4"
