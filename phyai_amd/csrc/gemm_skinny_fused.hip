@@ -87,17 +87,27 @@ __global__ __launch_bounds__(FQ_THREADS) void gemm_fp8_fusedq_kernel(
     constexpr bool GATED = epi_is_gated(EPI);
     constexpr int MB = (ROWS + 15) / 16;              // 16-row token blocks (the last one may be half used)
     constexpr int COLS_PER_TILE = GATED ? 8 : 16;
-    constexpr int BLOCKS = NT + MB;
+    // One K step of staging: NT weight blocks of 2 KB (16 rows x 128 bytes) and the codes of the token
+    // rows; an 8-row workgroup keeps only the 1 KB of its 8 rows (the MFMA's other 8 columns re-read them).
+    constexpr int XB = ROWS == 8 ? 1024 : 2048;
+    constexpr int STEP_BYTES = NT * 2048 + MB * XB;
     constexpr int RED_PER_WAVE = NT * MB * kWave * (int)sizeof(v4f);
-    constexpr int STAGE_PER_WAVE = KPW * BLOCKS * 2048;
+    constexpr int STAGE_PER_WAVE = KPW * STEP_BYTES;
     constexpr int PER_WAVE = STAGE_PER_WAVE > RED_PER_WAVE ? STAGE_PER_WAVE : RED_PER_WAVE;
+    // The table of row maxima (one word per wavefront and row) has its own 2 KB unless the staging
+    // leaves no room: then it lies over the first wavefront's code block of K step 0, which nobody
+    // writes before a second barrier has seen every wavefront read the table.
+    constexpr int TBL_ROWS = ROWS < 64 ? ROWS : 64;
+    constexpr bool TBL_ALIASED = FQ_WAVES * PER_WAVE + FQ_WAVES * 64 * 4 > 160 * 1024;
+    static_assert(!TBL_ALIASED || FQ_WAVES * TBL_ROWS * 4 <= XB, "aliased table does not fit a code block");
     static_assert(ROWS == 8 || ROWS % 16 == 0, "token rows per workgroup");
-    static_assert(FQ_WAVES * PER_WAVE + FQ_WAVES * 64 * 4 <= 160 * 1024, "staging does not fit the LDS");
+    static_assert(FQ_WAVES * PER_WAVE + (TBL_ALIASED ? 0 : FQ_WAVES * 64 * 4) <= 160 * 1024, "staging does not fit the LDS");
     constexpr int ROLE_ROUNDS = (NT * MB + FQ_WAVES - 1) / FQ_WAVES;
     auto rows_in_block = [](int mb) constexpr { return ROWS - 16 * mb < 16 ? ROWS - 16 * mb : 16; };
 
     __shared__ __attribute__((aligned(1024))) uint8_t smem[FQ_WAVES * PER_WAVE];
-    __shared__ uint32_t amax_tbl[FQ_WAVES][64];
+    __shared__ uint32_t amax_own[TBL_ALIASED ? 1 : FQ_WAVES * 64];
+    uint32_t* amax_tbl = TBL_ALIASED ? reinterpret_cast<uint32_t*>(smem + NT * 2048) : amax_own;   // [wavefront][TBL_ROWS]
     auto red = [&](int w, int nt, int mb, int l) -> v4f& {
         return reinterpret_cast<v4f*>(smem + w * PER_WAVE)[(nt * MB + mb) * kWave + l];
     };
@@ -163,7 +173,7 @@ __global__ __launch_bounds__(FQ_THREADS) void gemm_fp8_fusedq_kernel(
     for (int j = 0; j < KPW; ++j) {
         const int s = __builtin_amdgcn_readfirstlane(j * FQ_WAVES + wave);
         const int s_safe = s < total_steps ? s : total_steps - 1;
-        const uint32_t dst = lds_wave + j * (BLOCKS * 2048);
+        const uint32_t dst = lds_wave + j * STEP_BYTES;
 #pragma unroll
         for (int nt = 0; nt < NT; ++nt)
 #pragma unroll
@@ -212,7 +222,7 @@ __global__ __launch_bounds__(FQ_THREADS) void gemm_fp8_fusedq_kernel(
             o = dpp_move_u32<0x4E>(v);  v = o > v ? o : v;
             o = dpp_move_u32<0x141>(v); v = o > v ? o : v;
             o = dpp_move_u32<0x140>(v); v = o > v ? o : v;
-            if (xc == 0) amax_tbl[wave][mb * 16 + 4 * i + xr] = v;
+            if (xc == 0) amax_tbl[wave * TBL_ROWS + mb * 16 + 4 * i + xr] = v;
         }
     __syncthreads();
     // ---- the column operands of the epilogue: requested here, off the path from the row loads to the
@@ -235,14 +245,15 @@ __global__ __launch_bounds__(FQ_THREADS) void gemm_fp8_fusedq_kernel(
     float s_row = 1.0f, r_row = 1.0f;
     bool slow_row = false;
     if (lane < ROWS) {
-        uint32_t a = amax_tbl[0][lane];
+        uint32_t a = amax_tbl[lane];
 #pragma unroll
-        for (int w = 1; w < FQ_WAVES; ++w) a = amax_tbl[w][lane] > a ? amax_tbl[w][lane] : a;
+        for (int w = 1; w < FQ_WAVES; ++w) a = amax_tbl[w * TBL_ROWS + lane] > a ? amax_tbl[w * TBL_ROWS + lane] : a;
         s_row = scale_from_amax_bits<QUANT_ACT_DYNAMIC>(a);
         r_row = biased_reciprocal(s_row);
         slow_row = (__float_as_uint(s_row) & 0x7FFFFFFFu) >= 0x7F800000u;   // an Inf or NaN in the row
     }
     const bool any_slow = __builtin_amdgcn_ballot_w64(slow_row) != 0;       // wavefront-uniform
+    if constexpr (TBL_ALIASED) __syncthreads();   // the table lies where codes go next: everyone has read it
     float sa[ROLE_ROUNDS];
 #pragma unroll
     for (int rr = 0; rr < ROLE_ROUNDS; ++rr) sa[rr] = fq_bpermute(s_row, (e_mb[rr] * 16 + l16) & 63);
@@ -288,7 +299,7 @@ __global__ __launch_bounds__(FQ_THREADS) void gemm_fp8_fusedq_kernel(
                 const int at = r16 * 128 + (((xc >> 1) ^ ((r16 >> 1) & 7)) << 4) + (xc & 1) * 8;
 #pragma unroll
                 for (int j = 0; j < KPW; ++j)
-                    *reinterpret_cast<uint2*>(my_stage + j * (BLOCKS * 2048) + (NT + mb) * 2048 + at) =
+                    *reinterpret_cast<uint2*>(my_stage + j * STEP_BYTES + NT * 2048 + mb * XB + at) =
                         encode8<QUANT_ACT_DYNAMIC>(fq_as_uint4(xv[j][mb][i]), dv);
             }
     };
@@ -312,16 +323,19 @@ __global__ __launch_bounds__(FQ_THREADS) void gemm_fp8_fusedq_kernel(
         for (int mb = 0; mb < MB; ++mb) acc[nt][mb] = v4f{0.f, 0.f, 0.f, 0.f};
     const int swz = (l16 >> 1) & 7;
     const int rd_lo = l16 * 128 + ((q ^ swz) << 4), rd_hi = l16 * 128 + (((4 + q) ^ swz) << 4);
+    // token-row operand: an 8-row block is read twice over (columns 8 .. 15 of the product are not stored)
+    const int xl = ROWS == 8 ? (l16 & 7) : l16, xswz = (xl >> 1) & 7;
+    const int xrd_lo = xl * 128 + ((q ^ xswz) << 4), xrd_hi = xl * 128 + (((4 + q) ^ xswz) << 4);
 #pragma unroll
     for (int j = 0; j < KPW; ++j) {
         const int s = __builtin_amdgcn_readfirstlane(j * FQ_WAVES + wave);
         if (s < total_steps) {
-            const uint8_t* blk = my_stage + j * (BLOCKS * 2048);
+            const uint8_t* blk = my_stage + j * STEP_BYTES;
             v8i xb[MB];
 #pragma unroll
             for (int mb = 0; mb < MB; ++mb)
-                xb[mb] = fq_join(*reinterpret_cast<const v4i*>(blk + (NT + mb) * 2048 + rd_lo),
-                                 *reinterpret_cast<const v4i*>(blk + (NT + mb) * 2048 + rd_hi));
+                xb[mb] = fq_join(*reinterpret_cast<const v4i*>(blk + NT * 2048 + mb * XB + xrd_lo),
+                                 *reinterpret_cast<const v4i*>(blk + NT * 2048 + mb * XB + xrd_hi));
 #pragma unroll
             for (int nt = 0; nt < NT; ++nt) {
                 const v8i a = fq_join(*reinterpret_cast<const v4i*>(blk + nt * 2048 + rd_lo),
@@ -389,10 +403,15 @@ __global__ __launch_bounds__(FQ_THREADS) void gemm_fp8_fusedq_kernel(
 
 static int fq_ceil_div(int a, int b) { return (a + b - 1) / b; }
 
-static bool fq_fits(int rows, int nt, int kpw) {
+// LDS of a workgroup shape, as the kernel lays it out (the table of row maxima has its own 2 KB unless
+// only the staging fits, see the kernel).
+static constexpr bool fq_fits(int rows, int nt, int kpw) {
     const int mb = (rows + 15) / 16;
-    const int stage = kpw * (nt + mb) * 2048, redb = nt * mb * 1024;
-    return FQ_WAVES * (stage > redb ? stage : redb) + FQ_WAVES * 64 * 4 <= 160 * 1024;
+    const int xb = rows == 8 ? 1024 : 2048;
+    const int stage = kpw * (nt * 2048 + mb * xb), redb = nt * mb * 1024;
+    const int waves = FQ_WAVES * (stage > redb ? stage : redb);
+    if (waves + FQ_WAVES * 64 * 4 <= 160 * 1024) return true;
+    return waves <= 160 * 1024 && FQ_WAVES * (rows < 64 ? rows : 64) * 4 <= xb;
 }
 
 // Shapes that exist as kernels: (rows, nt) below, with kpw = 1, 2 or 4 as K asks.
@@ -448,7 +467,7 @@ FusedPlan fused_plan(int M, int N, int K, int epilogue, int64_t ldo) {
 
 template <int ROWS, int NT, int KPW, int EPI>
 static int fq_launch_one(const GemmProblem& g, const FusedPlan& pl, hipStream_t st) {
-    if constexpr (FQ_WAVES * (KPW * (NT + (ROWS + 15) / 16) * 2048) + FQ_WAVES * 256 > 160 * 1024) {
+    if constexpr (!fq_fits(ROWS, NT, KPW)) {
         return -2;
     } else {
         if (g.stream_weights)
