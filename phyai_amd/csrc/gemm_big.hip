@@ -183,7 +183,18 @@ void gemm_fp8_big_kernel(
     const int l32 = lane & 31, h = lane >> 5;
     const int half_n = p.N / 2;
     BigTile tile_id;
-    if (p.by_rows) {   // an XCD takes tile rows: bands of tile columns, 8 neighbouring tile rows per 8 ids
+    int split_z = SPLIT ? (int)blockIdx.z : 0, n_splits = SPLIT ? (int)gridDim.z : 1;
+    if (SPLIT && p.by_rows == 2) {
+        // Split-K with an XCD per K range: XCD x (= id % 8) works on K range x % S of the tile
+        // columns of group x / S, all tile rows.  The workgroups of an XCD then march along the same
+        // K range together: its L2 fetches that range of the activation rows once, not all of K.
+        n_splits = p.band;   // the split count rides in `band`, which this order does not use
+        const int x = blockIdx.x & 7, r = blockIdx.x >> 3, groups = 8 / n_splits;
+        const int cols = (p.n_tiles + groups - 1) / groups;
+        split_z = x % n_splits;
+        tile_id.n = (x / n_splits) * cols + r % cols;
+        tile_id.m = r / cols;
+    } else if (p.by_rows) {   // an XCD takes tile rows: bands of tile columns, 8 neighbouring tile rows per 8 ids
         const BigTile t = big_tile_of(blockIdx.x, p.n_tiles, p.m_tiles, p.band);
         tile_id.m = t.n; tile_id.n = t.m;
     } else {
@@ -218,7 +229,7 @@ void gemm_fp8_big_kernel(
         }
         boff[i] = (uint32_t)rb * (uint32_t)p.K + (((lane & 7) ^ big_swizzle(jj)) << 4);
     }
-    const int k_begin = SPLIT ? blockIdx.z * p.k_per_split : 0;
+    const int k_begin = SPLIT ? split_z * p.k_per_split : 0;
     const uint32_t lds_base = (uint32_t)(uintptr_t)lds;
     const uint32_t wave_a = __builtin_amdgcn_readfirstlane(lds_base + wave * (CA * 1024));
     const uint32_t wave_b = __builtin_amdgcn_readfirstlane(lds_base + BM * BIG_BK + wave * (CB * 1024));
@@ -348,14 +359,14 @@ void gemm_fp8_big_kernel(
     // that outside its accumulators.
     if constexpr (SPLIT) {
         constexpr int FRAG = TM * TN * 16, CHUNK = 32;
-        const int S = gridDim.z;
+        const int S = n_splits;
         const int tile = tile_id.m * p.n_tiles + tile_id.n;
 #pragma unroll
         for (int c = 0; c < TM * TN / 2; ++c) {
             float frag[CHUNK];
 #pragma unroll
             for (int r = 0; r < 32; ++r) frag[r] = acc[(2 * c) / TN][(2 * c) % TN + r / 16][r % 16];
-            splitk_publish_part<FRAG, 256, CHUNK>(p.partials, tile, S, blockIdx.z, c * CHUNK, frag);
+            splitk_publish_part<FRAG, 256, CHUNK>(p.partials, tile, S, split_z, c * CHUNK, frag);
         }
         wait_own_stores();
         // splitk_arrive opens with a barrier, after which nobody reads operands any more: a word
@@ -607,6 +618,7 @@ static void big_launch(BigArgs a, const GemmProblem& g, int splits, hipStream_t 
     // projection) that is eight copies of the larger operand; then the roles are exchanged.
     // Estimated bytes from HBM: the operand an XCD does not own is read once per XCD (up to 8
     // times), the other once per band.
+    double chosen_bytes = 0.0;
     {
         const double a_bytes = (double)g.M * g.K, b_bytes = (double)g.N * g.K;
         const int band_c = 4, band_r = 4;
@@ -621,6 +633,7 @@ static void big_launch(BigArgs a, const GemmProblem& g, int splits, hipStream_t 
         const int rounds_r = big_ceil_div(big_max_tiles_per_xcd(a.n_tiles, a.m_tiles, 4), slots);
         if (rounds_c != rounds_r) a.by_rows = rounds_r < rounds_c;
         if (const char* e = tuning_env("PHYAI_FP8_BY_ROWS")) a.by_rows = atoi(e) != 0;
+        chosen_bytes = a.by_rows ? by_rows : by_cols;
     }
     // bands of 4 tile rows; a grid of up to 8 tile rows whose activation rows still fit an XCD's
     // L2 beside the weight stream is one band, so that the weights come from HBM once
@@ -628,7 +641,23 @@ static void big_launch(BigArgs a, const GemmProblem& g, int splits, hipStream_t 
     if (!a.by_rows && a.m_tiles <= 8 && (int64_t)a.m_tiles * BM * (g.K < 4096 ? g.K : 4096) <= (5 << 19)) a.band = a.m_tiles;
     if (const char* e = tuning_env("PHYAI_FP8_BAND")) { const int b = atoi(e); if (b >= 1 && b <= 16) a.band = b; }
     const int outer = a.by_rows ? a.n_tiles : a.m_tiles, inner = a.by_rows ? a.m_tiles : a.n_tiles;
-    const dim3 grid(big_grid_ids(outer, inner, a.band), 1, splits);
+    dim3 grid(big_grid_ids(outer, inner, a.band), 1, splits);
+    // Split along K: an XCD per K range (see the kernel).  Every XCD then fetches 1 / splits of the
+    // activation codes instead of all of them, and the weights of its tile columns once.  Taken when
+    // that is the smaller estimate and the tile columns divide evenly among the 8 / splits groups
+    // (816 x 2048 x 16384, K split in two: 155 -> 87 MB fetched; the time is the same to within 1 %,
+    // the kernel being bound by its LDS traffic, so this saves HBM bandwidth, not microseconds).
+    if (splits == 2 || splits == 4 || splits == 8) {
+        const int groups = 8 / splits, cols = big_ceil_div(a.n_tiles, groups);
+        const double by_k = (double)g.M * g.K * 8.0 / splits + (double)g.N * g.K;
+        bool xcd_k = cols * groups == a.n_tiles && by_k < 0.8 * chosen_bytes;
+        if (const char* e = tuning_env("PHYAI_FP8_XCD_SPLIT")) xcd_k = atoi(e) != 0;
+        if (xcd_k) {
+            a.by_rows = 2;
+            a.band = splits;
+            grid = dim3(8 * cols * a.m_tiles, 1, 1);
+        }
+    }
 #define PHYAI_BIG_ARGS a.a, a.b, a.K, a.M, a.N, a.m_tiles, a.n_tiles, a.band, a.by_rows, a.k_per_split, a.a_scale, \
                        a.b_scale, a.bias, a.out, a.ldo, a.a_scale_scalar, a.partials, a.counters, a.res
     if (splits > 1) {

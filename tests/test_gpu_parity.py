@@ -594,6 +594,36 @@ def test_split_k_many_runs_one_result(dev, monkeypatch, force, shape):
         assert torch.equal(_as_bits(o), _as_bits(first)), f"launch {i} differs from the first"
 
 
+@pytest.mark.parametrize("M,N,K,tile,splits", [(816, 2048, 16384, "", ""), (816, 2048, 8192, "128", "2"), (300, 1024, 4096, "128", "4"),
+                                               (300, 2048, 4096, "128", "8"), (520, 2048, 4096, "256", "2"), (300, 768, 4096, "128", "4")])
+def test_split_k_with_an_xcd_per_k_range_gives_the_same_bits(dev, monkeypatch, M, N, K, tile, splits):
+    """Split-K launches can hand every XCD one K range (its L2 then fetches that range of the activation
+    codes once) instead of whole tile columns; the tiles, the K ranges and the order in which the partial
+    sums are added are the same, so the output must be equal bit for bit.  Includes a tile-column count
+    that does not divide among the groups (768 / 128 = 6 columns in 2 groups of 4 K ranges: padding ids)."""
+    ops = _ops()
+    if tile:
+        monkeypatch.setenv("PHYAI_FP8_BIG", tile)
+        monkeypatch.setenv("PHYAI_FP8_BIG_SPLITS", splits)
+    x, wq, ws, b = _problem(M, N, K, seed=M + N)
+    xq, xs = ops.fp8_quant_rowwise(x.to(dev))
+    wd, sd, bd = wq.to(dev), ws.to(dev), b.to(dev)
+    assert "splits=" in ops.describe_plan(M, N, K) and "splits=1" not in ops.describe_plan(M, N, K)
+    outs = {}
+    for order in ("0", "1"):
+        monkeypatch.setenv("PHYAI_FP8_XCD_SPLIT", order)
+        outs[order] = ops.fp8_gemm(xq, xs, wd, sd, bd)
+        again = ops.fp8_gemm(xq, xs, wd, sd, bd)
+        torch.cuda.synchronize()
+        assert torch.equal(_as_bits(outs[order]), _as_bits(again))
+    assert torch.equal(_as_bits(outs["0"]), _as_bits(outs["1"]))
+    monkeypatch.delenv("PHYAI_FP8_XCD_SPLIT")
+    assert torch.equal(_as_bits(ops.fp8_gemm(xq, xs, wd, sd, bd)), _as_bits(outs["0"]))   # the automatic choice
+    assert_close_to_ref(outs["1"], ref.gemm_f32(*ref.quant_rowwise(x), wq, ws, b), "split-K, an XCD per K range")
+    for w in ops._workspaces.values():
+        assert int(w[: ops.WORKSPACE_HEADER_BYTES].max().item()) == 0
+
+
 def test_two_streams_run_split_k_linears_concurrently(dev, monkeypatch):
     """Each (device, stream) pair has its own workspace (split-K counters and partials, code
     staging), so linears issued on two streams at once must give the serial results bit for bit."""
