@@ -89,7 +89,7 @@ __global__ __launch_bounds__(FQ_THREADS) void gemm_fp8_fusedq_kernel(
     constexpr int COLS_PER_TILE = GATED ? 8 : 16;
     // One K step of staging: NT weight blocks of 2 KB (16 rows x 128 bytes) and the codes of the token
     // rows; an 8-row workgroup keeps only the 1 KB of its 8 rows (the MFMA's other 8 columns re-read them).
-    constexpr int XB = ROWS == 8 ? 1024 : 2048;
+    constexpr int XB = ROWS < 16 ? ROWS * 128 : 2048;
     constexpr int STEP_BYTES = NT * 2048 + MB * XB;
     constexpr int RED_PER_WAVE = NT * MB * kWave * (int)sizeof(v4f);
     constexpr int STAGE_PER_WAVE = KPW * STEP_BYTES;
@@ -100,7 +100,7 @@ __global__ __launch_bounds__(FQ_THREADS) void gemm_fp8_fusedq_kernel(
     constexpr int TBL_ROWS = ROWS < 64 ? ROWS : 64;
     constexpr bool TBL_ALIASED = FQ_WAVES * PER_WAVE + FQ_WAVES * 64 * 4 > 160 * 1024;
     static_assert(!TBL_ALIASED || FQ_WAVES * TBL_ROWS * 4 <= XB, "aliased table does not fit a code block");
-    static_assert(ROWS == 8 || ROWS % 16 == 0, "token rows per workgroup");
+    static_assert(ROWS == 8 || ROWS % 16 == 0, "token rows per workgroup");   // (4-row workgroups were measured: slower)
     static_assert(FQ_WAVES * PER_WAVE + (TBL_ALIASED ? 0 : FQ_WAVES * 64 * 4) <= 160 * 1024, "staging does not fit the LDS");
     constexpr int ROLE_ROUNDS = (NT * MB + FQ_WAVES - 1) / FQ_WAVES;
     auto rows_in_block = [](int mb) constexpr { return ROWS - 16 * mb < 16 ? ROWS - 16 * mb : 16; };
@@ -324,7 +324,7 @@ __global__ __launch_bounds__(FQ_THREADS) void gemm_fp8_fusedq_kernel(
     const int swz = (l16 >> 1) & 7;
     const int rd_lo = l16 * 128 + ((q ^ swz) << 4), rd_hi = l16 * 128 + (((4 + q) ^ swz) << 4);
     // token-row operand: an 8-row block is read twice over (columns 8 .. 15 of the product are not stored)
-    const int xl = ROWS == 8 ? (l16 & 7) : l16, xswz = (xl >> 1) & 7;
+    const int xl = ROWS < 16 ? (l16 & (ROWS - 1)) : l16, xswz = (xl >> 1) & 7;
     const int xrd_lo = xl * 128 + ((q ^ xswz) << 4), xrd_hi = xl * 128 + (((4 + q) ^ xswz) << 4);
 #pragma unroll
     for (int j = 0; j < KPW; ++j) {
@@ -407,7 +407,7 @@ static int fq_ceil_div(int a, int b) { return (a + b - 1) / b; }
 // only the staging fits, see the kernel).
 static constexpr bool fq_fits(int rows, int nt, int kpw) {
     const int mb = (rows + 15) / 16;
-    const int xb = rows == 8 ? 1024 : 2048;
+    const int xb = rows < 16 ? rows * 128 : 2048;
     const int stage = kpw * (nt * 2048 + mb * xb), redb = nt * mb * 1024;
     const int waves = FQ_WAVES * (stage > redb ? stage : redb);
     if (waves + FQ_WAVES * 64 * 4 <= 160 * 1024) return true;
