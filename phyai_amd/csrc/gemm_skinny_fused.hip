@@ -422,7 +422,7 @@ static const int kFusedMaxK = 2048;
 // Up to 128 token rows the kernel is level with or ahead of quantizer + GEMM as long as a workgroup
 // converts 16 rows or fewer (measured at M = 64 ... 256 on the expert shapes: 32-row workgroups lose).
 static const int kFusedMaxM = 128;
-static const int kFusedShapes[][2] = {{8, 2}, {8, 4}, {8, 5}, {8, 6}, {8, 8}, {16, 1}, {16, 2}, {16, 4}, {16, 8}, {32, 2}, {32, 4}, {64, 2}};
+static const int kFusedShapes[][2] = {{8, 2}, {8, 4}, {8, 5}, {8, 8}, {16, 1}, {16, 2}, {16, 4}, {16, 8}, {32, 2}, {32, 4}};
 
 FusedPlan fused_plan(int M, int N, int K, int epilogue, int64_t ldo) {
     FusedPlan pl = {0, 0, 0, 0, 0};
@@ -498,7 +498,6 @@ static int fq_launch_epi(const GemmProblem& g, const FusedPlan& pl, hipStream_t 
     case 802: return fq_launch_kpw<8, 2, EPI>(g, pl, st);
     case 804: return fq_launch_kpw<8, 4, EPI>(g, pl, st);
     case 805: return fq_launch_kpw<8, 5, EPI>(g, pl, st);
-    case 806: return fq_launch_kpw<8, 6, EPI>(g, pl, st);
     case 808: return fq_launch_kpw<8, 8, EPI>(g, pl, st);
     case 1601: return fq_launch_kpw<16, 1, EPI>(g, pl, st);
     case 1602: return fq_launch_kpw<16, 2, EPI>(g, pl, st);
@@ -506,7 +505,6 @@ static int fq_launch_epi(const GemmProblem& g, const FusedPlan& pl, hipStream_t 
     case 1608: return fq_launch_kpw<16, 8, EPI>(g, pl, st);
     case 3202: return fq_launch_kpw<32, 2, EPI>(g, pl, st);
     case 3204: return fq_launch_kpw<32, 4, EPI>(g, pl, st);
-    case 6402: return fq_launch_kpw<64, 2, EPI>(g, pl, st);
     default: return -2;
     }
 }
