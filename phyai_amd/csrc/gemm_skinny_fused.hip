@@ -69,7 +69,7 @@ __device__ __forceinline__ float fq_bpermute(float v, int src_lane) {
     return __uint_as_float((uint32_t)__builtin_amdgcn_ds_bpermute(src_lane << 2, (int)__float_as_uint(v)));
 }
 
-// ROWS: token rows per workgroup (8, 16, 32, 64; grid.y workgroups cover M); NT: 16-row weight tiles
+// ROWS: token rows per workgroup (8, 16 or 32; grid.y workgroups cover M); NT: 16-row weight tiles
 // per workgroup; KPW: K steps per wavefront (K <= 128 * 8 * KPW, one round).
 //
 // Between the row loads and the wait for them the code is straight-line on purpose: the loaded
@@ -81,9 +81,8 @@ __device__ __forceinline__ float fq_bpermute(float v, int src_lane) {
 template <int ROWS, int NT, int KPW, int EPI, bool STREAM>
 __global__ __launch_bounds__(FQ_THREADS) void gemm_fp8_fusedq_kernel(
     const uint8_t* __restrict__ a_w, const uint8_t* __restrict__ a_x, const float* __restrict__ a_w_scale,
-    const uint16_t* __restrict__ a_bias, int a_K, int a_N, int a_m_flags, int a_ldx_bytes, uint16_t* __restrict__ a_out,
+    const uint16_t* __restrict__ a_bias, int a_K, int a_N, int a_M, int a_ldx_bytes, uint16_t* __restrict__ a_out,
     int64_t a_ldo, const ResidualArgs a_res) {
-    const int a_M = a_m_flags & 0x0FFFFFFF;
     constexpr bool GATED = epi_is_gated(EPI);
     constexpr int MB = (ROWS + 15) / 16;              // 16-row token blocks (the last one may be half used)
     constexpr int COLS_PER_TILE = GATED ? 8 : 16;

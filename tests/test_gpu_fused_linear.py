@@ -170,3 +170,38 @@ def test_graph_replay_of_the_one_launch_kernel(dev):
         gr.replay()
         torch.cuda.synchronize()
         assert _same(out, want), f"replay with seed {seed}"
+
+
+def test_random_shapes_equal_two_launches_bit_for_bit(dev, monkeypatch):
+    """150 seeded random problems the automatic choice serves with the one-launch kernel (M up to 128,
+    every epilogue, with and without bias, streamed weights or not, tiny and outlier rows)."""
+    import random
+
+    ops = _ops()
+    rnd = random.Random(7)
+    epis = [None, "gelu", "gelu_tanh", "geglu_tanh", "geglu_erf", "swiglu"]
+    ran = 0
+    for it in range(150):
+        M = rnd.choice([1, 2, 3, 5, 7, 8, 9, 15, 16, 17, 31, 33, 47, 50, 63, 64, 65, 77, 96, 100, 127, 128])
+        K = 128 * rnd.randint(1, 16)
+        epi = rnd.choice(epis)
+        N = (32 if epi in ("geglu_tanh", "geglu_erf", "swiglu") else 16) * rnd.randint(1, 96)
+        monkeypatch.setenv("PHYAI_FP8_FUSED", "1")
+        desc = ops.describe_linear_plan(M, N, K, epi)
+        if not desc.startswith("one launch"):
+            continue
+        ran += 1
+        x = seeded((M, K), seed=it)
+        if it % 5 == 0:
+            x[M // 2] *= 1e-20
+        if it % 7 == 0:
+            x[0, K // 2] = 1000.0
+        xd = x.to(dev)
+        wq, ws = ops.fp8_weight_quant(seeded((N, K), seed=1000 + it, scale=0.02).to(dev))
+        b = seeded((N,), seed=2000 + it, scale=0.01).to(dev) if it % 2 else None
+        got = ops.fp8_linear(xd, wq, ws, b, epilogue=epi, stream_weights=it % 3 == 0)
+        monkeypatch.setenv("PHYAI_FP8_FUSED", "0")
+        want = ops.fp8_linear(xd, wq, ws, b, epilogue=epi)
+        torch.cuda.synchronize()
+        assert _same(got, want), f"case {it}: {M}x{N}x{K} {epi} ({desc}): {int((_bits(got) != _bits(want)).sum())} outputs differ"
+    assert ran >= 100
