@@ -156,6 +156,18 @@ __device__ __forceinline__ float apply_act(float v) {
     else return v;
 }
 
+// Round an fp32 value through bf16 (the reference materialises the GEMM output
+// as a bf16 tensor before the activation kernel reads it).  The hardware convert rounds to nearest
+// even like f32_to_bf16_bits; the two differ only in the bits of a NaN (the convert keeps sign and
+// payload, the software form returns 0x7FC0).  All GEMM epilogues use the convert.
+__device__ __forceinline__ float round_bf16(float v) { return __uint_as_float(pack_bf16x2(v, 0.0f) << 16); }
+// Two values at once: three instructions instead of four.
+__device__ __forceinline__ void round_bf16_pair(float& a, float& b) {
+    const uint32_t p = pack_bf16x2(a, b);
+    a = __uint_as_float(p << 16);
+    b = __uint_as_float(p & 0xFFFF0000u);
+}
+
 // residual + y * gate on four consecutive columns; y is the linear's bf16 output.  The product of
 // two bf16 values is exact in fp32, so this equals torch.addcmul's single rounding whether or
 // not the multiply and the add are contracted.
@@ -165,11 +177,7 @@ __device__ __forceinline__ void addcmul4(float* y, uint2 res, uint2 gate) {
     const float g[4] = {bf16_bits_to_f32(gate.x & 0xFFFFu), __uint_as_float(gate.x & 0xFFFF0000u),
                         bf16_bits_to_f32(gate.y & 0xFFFFu), __uint_as_float(gate.y & 0xFFFF0000u)};
 #pragma unroll
-    for (int e = 0; e < 4; ++e) y[e] = r[e] + bf16_bits_to_f32(f32_to_bf16_bits(y[e])) * g[e];
+    for (int e = 0; e < 4; ++e) y[e] = r[e] + round_bf16(y[e]) * g[e];
 }
-
-// Round an fp32 value through bf16 (the reference materialises the GEMM output
-// as a bf16 tensor before the activation kernel reads it).
-__device__ __forceinline__ float round_bf16(float v) { return bf16_bits_to_f32(f32_to_bf16_bits(v)); }
 
 }  // namespace phyai

@@ -342,7 +342,6 @@ __global__ __launch_bounds__(SK_THREADS) void gemm_fp8_skinny_kernel(
                               bf16_bits_to_f32(bw2[rr].y & 0xFFFFu), bf16_bits_to_f32(bw2[rr].y >> 16)};
         const float buf[4] = {bf16_bits_to_f32(bu2[rr].x & 0xFFFFu), bf16_bits_to_f32(bu2[rr].x >> 16),
                               bf16_bits_to_f32(bu2[rr].y & 0xFFFFu), bf16_bits_to_f32(bu2[rr].y >> 16)};
-        uint32_t o[4];
         float vf[4];
 #pragma unroll
         for (int r = 0; r < 4; ++r) {
@@ -358,11 +357,9 @@ __global__ __launch_bounds__(SK_THREADS) void gemm_fp8_skinny_kernel(
         if constexpr (EPI == EPI_NONE) {
             if (p.res.residual != nullptr) addcmul4(vf, res2[rr], gate2[rr]);
         }
-#pragma unroll
-        for (int r = 0; r < 4; ++r) o[r] = f32_to_bf16_bits(vf[r]);
         if (e_live[rr])
             *reinterpret_cast<uint2*>(p.out + (int64_t)e_m[rr] * p.ldo + e_n[rr]) =
-                make_uint2(o[0] | (o[1] << 16), o[2] | (o[3] << 16));
+                make_uint2(pack_bf16x2(vf[0], vf[1]), pack_bf16x2(vf[2], vf[3]));
     }
 }
 

@@ -157,8 +157,11 @@ __global__ __launch_bounds__(FQ_THREADS) void gemm_fp8_fusedq_kernel(
         for (int nt = 0; nt < NT; ++nt) {
             int wr;
             if constexpr (GATED) {
-                const int g = col0 + nt * 8 + (r16 & 7);
-                wr = (r16 < 8 ? 0 : half_n) + (g < half_n ? g : half_n - 1);
+                // rows 4p .. 4p+3 of a gated tile: gate columns 2p, 2p+1, then up columns 2p, 2p+1, so
+                // that an MFMA lane (which owns four consecutive tile rows) holds both halves of two
+                // output columns and all 64 lanes take part in the epilogue
+                const int g = col0 + nt * 8 + 2 * (r16 >> 2) + (r16 & 1);
+                wr = ((r16 & 2) ? half_n : 0) + (g < half_n ? g : half_n - 1);
             } else {
                 const int r = col0 + nt * 16 + r16;
                 wr = r < N ? r : N - 1;
@@ -191,10 +194,10 @@ __global__ __launch_bounds__(FQ_THREADS) void gemm_fp8_fusedq_kernel(
         const int role = rr * FQ_WAVES + wave;
         e_mb[rr] = role % MB;
         e_nt[rr] = role / MB;
-        e_role[rr] = (e_nt[rr] < NT) && (!GATED || q < 2);
+        e_role[rr] = e_nt[rr] < NT;
         const int r_in = e_mb[rr] * 16 + l16;                 // token row within the workgroup
         e_m[rr] = m_base + r_in;
-        e_n[rr] = col0 + (e_nt[rr] < NT ? e_nt[rr] : 0) * COLS_PER_TILE + 4 * q;
+        e_n[rr] = col0 + (e_nt[rr] < NT ? e_nt[rr] : 0) * COLS_PER_TILE + (GATED ? 2 : 4) * q;
         e_live[rr] = e_role[rr] && r_in < ROWS && e_m[rr] < M && e_n[rr] < n_out_total;
         e_n_safe[rr] = e_live[rr] ? e_n[rr] : 0;
     }
@@ -230,13 +233,20 @@ __global__ __launch_bounds__(FQ_THREADS) void gemm_fp8_fusedq_kernel(
     uint2 bw2[ROLE_ROUNDS], bu2[ROLE_ROUNDS];
 #pragma unroll
     for (int rr = 0; rr < ROLE_ROUNDS; ++rr) {
-        sw4[rr] = *reinterpret_cast<const v4f*>(a_w_scale + e_n_safe[rr]);
         su4[rr] = v4f{0.f, 0.f, 0.f, 0.f};
-        if constexpr (GATED) su4[rr] = *reinterpret_cast<const v4f*>(a_w_scale + half_n + e_n_safe[rr]);
         bw2[rr] = make_uint2(0, 0); bu2[rr] = make_uint2(0, 0);
-        if (a_bias) {
-            bw2[rr] = *reinterpret_cast<const uint2*>(a_bias + e_n_safe[rr]);
-            if constexpr (GATED) bu2[rr] = *reinterpret_cast<const uint2*>(a_bias + half_n + e_n_safe[rr]);
+        if constexpr (GATED) {   // two output columns per lane: two scales and two bias values of each half
+            const float2 sg = *reinterpret_cast<const float2*>(a_w_scale + e_n_safe[rr]);
+            const float2 su = *reinterpret_cast<const float2*>(a_w_scale + half_n + e_n_safe[rr]);
+            sw4[rr] = v4f{sg.x, sg.y, 0.f, 0.f};
+            su4[rr] = v4f{su.x, su.y, 0.f, 0.f};
+            if (a_bias) {
+                bw2[rr].x = *reinterpret_cast<const uint32_t*>(a_bias + e_n_safe[rr]);
+                bu2[rr].x = *reinterpret_cast<const uint32_t*>(a_bias + half_n + e_n_safe[rr]);
+            }
+        } else {
+            sw4[rr] = *reinterpret_cast<const v4f*>(a_w_scale + e_n_safe[rr]);
+            if (a_bias) bw2[rr] = *reinterpret_cast<const uint2*>(a_bias + e_n_safe[rr]);
         }
     }
 
@@ -360,41 +370,39 @@ __global__ __launch_bounds__(FQ_THREADS) void gemm_fp8_fusedq_kernel(
         v4f g = red(0, e_nt[rr], e_mb[rr], lane);
 #pragma unroll
         for (int w = 1; w < FQ_WAVES; ++w) g += red(w, e_nt[rr], e_mb[rr], lane);
-        v4f u = v4f{0.f, 0.f, 0.f, 0.f};
-        if constexpr (GATED) {
-            const int from = ((lane + 32) & 63) << 2;      // the up half of a gated tile sits 32 lanes further on
-#pragma unroll
-            for (int r = 0; r < 4; ++r)
-                u[r] = __uint_as_float((uint32_t)__builtin_amdgcn_ds_bpermute(from, (int)__float_as_uint(g[r])));
-        }
         if (!e_role[rr]) continue;
 
         // ---- 4. epilogue (the arithmetic of gemm_skinny.hip, operation for operation) --------------
         const float bwf[4] = {bf16_bits_to_f32(bw2[rr].x & 0xFFFFu), bf16_bits_to_f32(bw2[rr].x >> 16),
                               bf16_bits_to_f32(bw2[rr].y & 0xFFFFu), bf16_bits_to_f32(bw2[rr].y >> 16)};
-        const float buf[4] = {bf16_bits_to_f32(bu2[rr].x & 0xFFFFu), bf16_bits_to_f32(bu2[rr].x >> 16),
-                              bf16_bits_to_f32(bu2[rr].y & 0xFFFFu), bf16_bits_to_f32(bu2[rr].y >> 16)};
-        uint32_t o[4];
-        float vf[4];
+        if constexpr (GATED) {
+            // g[0], g[1]: gate sums of this lane's two columns; g[2], g[3]: their up sums
+            const float buf[2] = {bf16_bits_to_f32(bu2[rr].x & 0xFFFFu), bf16_bits_to_f32(bu2[rr].x >> 16)};
+            float vf[2];
 #pragma unroll
-        for (int r = 0; r < 4; ++r) {
-            float v = __builtin_fmaf(g[r], sa[rr] * sw4[rr][r], bwf[r]);
-            if constexpr (GATED) {
-                const float up = __builtin_fmaf(u[r], sa[rr] * su4[rr][r], buf[r]);
-                v = apply_act<EPI>(round_bf16(v)) * round_bf16(up);
-            } else if constexpr (EPI != EPI_NONE) {
-                v = apply_act<EPI>(round_bf16(v));
+            for (int r = 0; r < 2; ++r) {
+                float v = __builtin_fmaf(g[r], sa[rr] * sw4[rr][r], bwf[r]);
+                float up = __builtin_fmaf(g[2 + r], sa[rr] * su4[rr][r], buf[r]);
+                round_bf16_pair(v, up);
+                vf[r] = apply_act<EPI>(v) * up;
             }
-            vf[r] = v;
-        }
-        if constexpr (EPI == EPI_NONE) {
-            if (a_res.residual != nullptr) addcmul4(vf, res2[rr], gate2[rr]);
-        }
+            if (e_live[rr])
+                *reinterpret_cast<uint32_t*>(a_out + (int64_t)e_m[rr] * a_ldo + e_n[rr]) = pack_bf16x2(vf[0], vf[1]);
+        } else {
+            float vf[4];
 #pragma unroll
-        for (int r = 0; r < 4; ++r) o[r] = f32_to_bf16_bits(vf[r]);
-        if (e_live[rr])
-            *reinterpret_cast<uint2*>(a_out + (int64_t)e_m[rr] * a_ldo + e_n[rr]) =
-                make_uint2(o[0] | (o[1] << 16), o[2] | (o[3] << 16));
+            for (int r = 0; r < 4; ++r) {
+                float v = __builtin_fmaf(g[r], sa[rr] * sw4[rr][r], bwf[r]);
+                if constexpr (EPI != EPI_NONE) v = apply_act<EPI>(round_bf16(v));
+                vf[r] = v;
+            }
+            if constexpr (EPI == EPI_NONE) {
+                if (a_res.residual != nullptr) addcmul4(vf, res2[rr], gate2[rr]);
+            }
+            if (e_live[rr])
+                *reinterpret_cast<uint2*>(a_out + (int64_t)e_m[rr] * a_ldo + e_n[rr]) =
+                    make_uint2(pack_bf16x2(vf[0], vf[1]), pack_bf16x2(vf[2], vf[3]));
+        }
     }
 }
 

@@ -241,7 +241,7 @@ __global__ __launch_bounds__(256) void gemm_fp8_tile_kernel(const TileArgs p) {
                                 round_bf16(v) *
                                     bf16_bits_to_f32(p.res.gate[(int64_t)(m / p.res.gate_group) * p.res.ld_gate + n_out]);
                     }
-                    p.out[(int64_t)m * p.ldo + n_out] = (uint16_t)f32_to_bf16_bits(v);
+                    p.out[(int64_t)m * p.ldo + n_out] = (uint16_t)(pack_bf16x2(v, 0.0f) & 0xFFFFu);
                 }
             }
         }
