@@ -135,18 +135,25 @@ __global__ __launch_bounds__(SK_THREADS) void gemm_fp8_skinny_kernel(
         const int role = rr * SK_WAVES + (tid >> 6);
         e_mb[rr] = role % MB;
         e_nt[rr] = role / MB;
-        e_role[rr] = (e_nt[rr] < NT) && (!GATED || e_q < 2);
+        e_role[rr] = e_nt[rr] < NT;
         e_m[rr] = m_base + e_mb[rr] * 16 + (e_lane & 15);
-        e_n[rr] = col0 + (e_nt[rr] < NT ? e_nt[rr] : 0) * COLS_PER_TILE + 4 * e_q;
+        e_n[rr] = col0 + (e_nt[rr] < NT ? e_nt[rr] : 0) * COLS_PER_TILE + (GATED ? 2 : 4) * e_q;
         e_live[rr] = e_role[rr] && e_m[rr] < p.M && e_n[rr] < n_out_total;
         const int e_n_safe = e_live[rr] ? e_n[rr] : 0;
-        sw4[rr] = *reinterpret_cast<const v4f*>(p.w_scale + e_n_safe);
         su4[rr] = v4f{0.f, 0.f, 0.f, 0.f};
-        if constexpr (GATED) su4[rr] = *reinterpret_cast<const v4f*>(p.w_scale + half_n + e_n_safe);
         bw2[rr] = make_uint2(0, 0); bu2[rr] = make_uint2(0, 0);
-        if (p.bias) {
-            bw2[rr] = *reinterpret_cast<const uint2*>(p.bias + e_n_safe);
-            if constexpr (GATED) bu2[rr] = *reinterpret_cast<const uint2*>(p.bias + half_n + e_n_safe);
+        if constexpr (GATED) {   // two output columns per lane: two scales and two bias values of each half
+            const float2 sg = *reinterpret_cast<const float2*>(p.w_scale + e_n_safe);
+            const float2 su = *reinterpret_cast<const float2*>(p.w_scale + half_n + e_n_safe);
+            sw4[rr] = v4f{sg.x, sg.y, 0.f, 0.f};
+            su4[rr] = v4f{su.x, su.y, 0.f, 0.f};
+            if (p.bias) {
+                bw2[rr].x = *reinterpret_cast<const uint32_t*>(p.bias + e_n_safe);
+                bu2[rr].x = *reinterpret_cast<const uint32_t*>(p.bias + half_n + e_n_safe);
+            }
+        } else {
+            sw4[rr] = *reinterpret_cast<const v4f*>(p.w_scale + e_n_safe);
+            if (p.bias) bw2[rr] = *reinterpret_cast<const uint2*>(p.bias + e_n_safe);
         }
         sa[rr] = p.x_scale[(p.x_scale_scalar || !e_live[rr]) ? 0 : e_m[rr]];
     }
@@ -172,8 +179,11 @@ __global__ __launch_bounds__(SK_THREADS) void gemm_fp8_skinny_kernel(
     // weight row of operand row r16 (0..15) of tile nt, token row of operand row r16 of block mb
     auto w_row = [&](int nt, int r16) -> int {
         if constexpr (GATED) {
-            const int g = col0 + nt * 8 + (r16 & 7);
-            return (r16 < 8 ? 0 : half_n) + (g < half_n ? g : half_n - 1);
+            // rows 4p .. 4p+3 of a gated tile: gate columns 2p, 2p+1, then up columns 2p, 2p+1, so that
+            // an MFMA lane (which owns four consecutive tile rows) holds both halves of two output
+            // columns: no exchange between lanes, and all 64 lanes take part in the epilogue
+            const int g = col0 + nt * 8 + 2 * (r16 >> 2) + (r16 & 1);
+            return ((r16 & 2) ? half_n : 0) + (g < half_n ? g : half_n - 1);
         } else {
             const int r = col0 + nt * 16 + r16;
             return r < p.N ? r : p.N - 1;
@@ -325,41 +335,39 @@ __global__ __launch_bounds__(SK_THREADS) void gemm_fp8_skinny_kernel(
         v4f g = red(0, e_nt[rr], e_mb[rr], e_lane);
 #pragma unroll
         for (int w = 1; w < SK_WAVES; ++w) g += red(w, e_nt[rr], e_mb[rr], e_lane);
-        v4f u = v4f{0.f, 0.f, 0.f, 0.f};
-        if constexpr (GATED) {
-            // The up half of a gated tile sits 32 lanes further on.  Every lane has just added up its
-            // own slot, so the upper half of the wavefront hands its sums down instead of the lower
-            // half reading eight more partials each.
-            const int from = ((e_lane + 32) & 63) << 2;
-#pragma unroll
-            for (int r = 0; r < 4; ++r)
-                u[r] = __uint_as_float((uint32_t)__builtin_amdgcn_ds_bpermute(from, (int)__float_as_uint(g[r])));
-        }
         if (!e_role[rr]) continue;
 
         // ---- 4. epilogue --------------------------------------------------------------------
         const float bwf[4] = {bf16_bits_to_f32(bw2[rr].x & 0xFFFFu), bf16_bits_to_f32(bw2[rr].x >> 16),
                               bf16_bits_to_f32(bw2[rr].y & 0xFFFFu), bf16_bits_to_f32(bw2[rr].y >> 16)};
-        const float buf[4] = {bf16_bits_to_f32(bu2[rr].x & 0xFFFFu), bf16_bits_to_f32(bu2[rr].x >> 16),
-                              bf16_bits_to_f32(bu2[rr].y & 0xFFFFu), bf16_bits_to_f32(bu2[rr].y >> 16)};
-        float vf[4];
+        if constexpr (GATED) {
+            // g[0], g[1]: gate sums of this lane's two columns; g[2], g[3]: their up sums
+            const float buf[2] = {bf16_bits_to_f32(bu2[rr].x & 0xFFFFu), bf16_bits_to_f32(bu2[rr].x >> 16)};
+            float vf[2];
 #pragma unroll
-        for (int r = 0; r < 4; ++r) {
-            float v = __builtin_fmaf(g[r], sa[rr] * sw4[rr][r], bwf[r]);   // one rounding, like the tile kernels
-            if constexpr (GATED) {
-                const float up = __builtin_fmaf(u[r], sa[rr] * su4[rr][r], buf[r]);
-                v = apply_act<EPI>(round_bf16(v)) * round_bf16(up);
-            } else if constexpr (EPI != EPI_NONE) {
-                v = apply_act<EPI>(round_bf16(v));
+            for (int r = 0; r < 2; ++r) {
+                float v = __builtin_fmaf(g[r], sa[rr] * sw4[rr][r], bwf[r]);   // one rounding, like the tile kernels
+                float up = __builtin_fmaf(g[2 + r], sa[rr] * su4[rr][r], buf[r]);
+                round_bf16_pair(v, up);
+                vf[r] = apply_act<EPI>(v) * up;
             }
-            vf[r] = v;
+            if (e_live[rr])
+                *reinterpret_cast<uint32_t*>(p.out + (int64_t)e_m[rr] * p.ldo + e_n[rr]) = pack_bf16x2(vf[0], vf[1]);
+        } else {
+            float vf[4];
+#pragma unroll
+            for (int r = 0; r < 4; ++r) {
+                float v = __builtin_fmaf(g[r], sa[rr] * sw4[rr][r], bwf[r]);   // one rounding, like the tile kernels
+                if constexpr (EPI != EPI_NONE) v = apply_act<EPI>(round_bf16(v));
+                vf[r] = v;
+            }
+            if constexpr (EPI == EPI_NONE) {
+                if (p.res.residual != nullptr) addcmul4(vf, res2[rr], gate2[rr]);
+            }
+            if (e_live[rr])
+                *reinterpret_cast<uint2*>(p.out + (int64_t)e_m[rr] * p.ldo + e_n[rr]) =
+                    make_uint2(pack_bf16x2(vf[0], vf[1]), pack_bf16x2(vf[2], vf[3]));
         }
-        if constexpr (EPI == EPI_NONE) {
-            if (p.res.residual != nullptr) addcmul4(vf, res2[rr], gate2[rr]);
-        }
-        if (e_live[rr])
-            *reinterpret_cast<uint2*>(p.out + (int64_t)e_m[rr] * p.ldo + e_n[rr]) =
-                make_uint2(pack_bf16x2(vf[0], vf[1]), pack_bf16x2(vf[2], vf[3]));
     }
 }
 
