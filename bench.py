@@ -453,11 +453,13 @@ def gemm_only_times(dev, layers, shapes, M, reps=8, iters=30):
     return out
 
 
-def gemm_only_layer_time(dev, layers, shapes, reps=8, iters=30):
+def gemm_only_layer_time(dev, layers, shapes, reps=8, iters=30, ready_codes=False):
     """Average duration of one layer's weight-reading kernels in the order and under the cache conditions
     of the benchmark: a graph holding only those launches, all shapes of a layer, layer
     after layer (the whole 311 MB of weights per pass, so no matrix is cache-warm by accident; a
-    graph of one shape alone holds 47-151 MB, which fits the 256 MB Infinity Cache)."""
+    graph of one shape alone holds 47-151 MB, which fits the 256 MB Infinity Cache).
+    ready_codes: every shape as the GEMM on codes the quantizer left (what this figure measured
+    before a linear could be one kernel)."""
     from phyai_amd import ops
     from phyai_amd.runtime import HipGraph
 
@@ -471,7 +473,11 @@ def gemm_only_layer_time(dev, layers, shapes, reps=8, iters=30):
     def fn():
         for _ in range(reps):
             for xq, xs, t in pre:
-                weight_kernel_launch(xq, xs, t)
+                if ready_codes:
+                    ops.fp8_gemm(xq, xs, t["w"], t["ws"], None, epilogue=t["epi"], out=t["out"],
+                                 stream_weights=t.get("stream", False))
+                else:
+                    weight_kernel_launch(xq, xs, t)
 
     g = HipGraph()
     g.capture(fn, {})
@@ -745,11 +751,18 @@ def main() -> int:
                 "in a graph of those launches only that walks all 18 layers (311 MB of weights per pass); per_shape "
                 "times come from graphs of one shape alone, whose 47-151 MB of weights fit the Infinity Cache",
         "plans": {name: ops_plan(M, N, K, epi) for name, N, K, epi in EXPERT_SET},
+        "gemm_on_ready_codes": None,
         "per_shape": {name: {"us": round(per_launch_us[name], 3),
                              "GB/s": round(algorithmic_bytes(M, N, K, epi) / per_launch_us[name] / 1e3, 1)}
                       for name, N, K, epi in EXPERT_SET},
         "whole_path_frac": round(layer_bytes * n_layers / (value_us * 1e-6) / 1e9 / HBM_PEAK_GBS, 4),
     }
+    if not args.no_extras:
+        codes_us = gemm_only_layer_time(dev, layers, EXPERT_SET, ready_codes=True)
+        roofline["gemm_on_ready_codes"] = {
+            "us_per_layer": round(codes_us, 3), "frac": round(layer_bytes / (codes_us * 1e-6) / 1e9 / HBM_PEAK_GBS, 4),
+            "note": "the four GEMM launches of a layer on codes and scales the quantizer left (phyai_fp8_gemm): what "
+                    "`frac` measured before a linear could be one kernel; the quantization is not in this figure"}
     # (profiler sessions pass --no-extras: then only the benchmark's own kernels run)
     measured = None if args.no_extras else hardware_probe(dev)
     if measured is not None:
