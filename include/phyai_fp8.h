@@ -31,7 +31,7 @@
 extern "C" {
 #endif
 
-#define PHYAI_FP8_ABI_VERSION 7
+#define PHYAI_FP8_ABI_VERSION 8
 
 enum {
     PHYAI_FP8_OK = 0,
@@ -64,9 +64,18 @@ enum {
  * kernel (what phyai_fp8_describe_plan reports as "small-m"), ignored by the tile kernels, whose
  * workgroups share weight rows through L2; results are bit-identical with and without it.  The
  * reference has no counterpart (its GEMM is a library call, linear/backends/torch.py:168-175).
+ *
+ * W_OPERAND_ORDER / W_OPERAND_GATED: `w` is not row-major [N, K] but in MFMA operand order, as
+ * phyai_fp8_weight_to_operand_order() wrote it (plain form for the first flag, the fused gate | up
+ * form for the second).  Every kernel accepts both layouts and gives bit-identical results; the
+ * kernels whose weight blocks are private to a wavefront then load them straight into registers
+ * instead of staging them through LDS.  A gated epilogue needs W_OPERAND_GATED, any other epilogue
+ * W_OPERAND_ORDER; a mismatch is refused with PHYAI_FP8_EINVAL.  K must be a multiple of 128.
  */
 #define PHYAI_FP8_EPILOGUE_MASK 0xFF
 #define PHYAI_FP8_FLAG_STREAM_WEIGHTS 0x100
+#define PHYAI_FP8_FLAG_W_OPERAND_ORDER 0x200
+#define PHYAI_FP8_FLAG_W_OPERAND_GATED 0x600
 
 int phyai_fp8_abi_version(void);
 const char *phyai_fp8_last_error(void);
@@ -98,6 +107,22 @@ int phyai_fp8_quant_static(const void *x, int64_t M, int64_t K, int64_t ldx,
  */
 int phyai_fp8_weight_quant_rowwise(const void *w, int64_t N, int64_t K, int64_t ldw,
                                    void *wq, float *w_scale, void *stream);
+
+/*
+ * Re-lays a row-major fp8 weight matrix w[N, K] into MFMA operand order, out of place (out: N * K
+ * bytes, 16-byte aligned, must not overlap w).  Units of 16 rows x 128 bytes of K are stored
+ * K step after K step, and inside a unit the 16-byte chunk c of row r sits at (c * 16 + r) * 16:
+ * the sixteen lanes of a wavefront that want the same 16 bytes of K of sixteen neighbouring rows read
+ * 256 contiguous bytes.  gated != 0: w is a fused gate | up matrix (gate = rows [0, N/2)); unit u
+ * then holds gate columns 8 u .. 8 u + 7 and the up columns that pair with them, row 4 p + 2 t + b of
+ * the unit being row t * N/2 + 8 u + 2 p + b of w, so that an MFMA lane ends up with gate and up of
+ * the same output columns.  Needs K % 128 == 0 and N % 16 == 0 (N % 32 == 0 when gated).
+ * This is the work the reference leaves to WeightSpec.process_after_loading
+ * (layers/quant/base.py:55-70, layers/quant/fp8.py:127-135: "re-lay weights after loading");
+ * pass the result to the GEMM entry points with PHYAI_FP8_FLAG_W_OPERAND_ORDER / _GATED.
+ */
+int phyai_fp8_weight_to_operand_order(const void *w, int64_t N, int64_t K, int gated, void *out,
+                                      void *stream);
 
 /*
  * Bytes of workspace phyai_fp8_linear / phyai_fp8_gemm need for this shape.
@@ -132,9 +157,9 @@ int phyai_fp8_gemm(const void *xq, const float *x_scale, int x_scale_is_scalar,
  * Up to 128 token rows, K <= 2048 (a multiple of 128), with x and its row stride 16-byte
  * aligned and a grid that fits the chip at once, this is ONE kernel: every workgroup
  * quantizes the token rows it multiplies (same codes, same scales, same output bits as
- * the two launches) and the workspace is not touched.  Otherwise the quantizer writes
- * codes and scales into the workspace and a GEMM kernel follows.
- * phyai_fp8_describe_linear_plan tells which.
+ * the two launches) and the workspace is not touched: such a call may pass workspace = NULL.
+ * Otherwise the quantizer writes codes and scales into the workspace and a GEMM kernel follows
+ * (PHYAI_FP8_EWORKSPACE without one).  phyai_fp8_describe_linear_plan tells which.
  */
 int phyai_fp8_linear(const void *x, int64_t ldx, const void *w, const float *w_scale,
                      const void *bias, void *out, int64_t ldo, int64_t M, int64_t N,
@@ -148,19 +173,20 @@ int phyai_fp8_linear(const void *x, int64_t ldx, const void *w, const float *w_s
  * tensors (models/pi05/modeling_pi05.py:822-826,835: `h = torch.addcmul(residual, out, gate)`
  * after o_proj and after the MLP's down_proj).  residual: [M, N] bf16, row stride ld_res;
  * gate: [gate_rows, N] bf16, row stride ld_gate, M a multiple of gate_rows and g = M / gate_rows
- * (the gate of an adaptive norm has one row per modulation row).  No activation epilogue.
- * out may alias residual.
+ * (the gate of an adaptive norm has one row per modulation row).  No activation epilogue;
+ * flags: PHYAI_FP8_FLAG_* bits (STREAM_WEIGHTS, W_OPERAND_ORDER) or 0.  out may alias residual.
  */
 int phyai_fp8_gemm_addcmul(const void *xq, const float *x_scale, int x_scale_is_scalar,
                            const void *w, const float *w_scale, const void *bias,
                            const void *residual, int64_t ld_res, const void *gate, int64_t ld_gate,
                            int64_t gate_rows, void *out, int64_t ldo, int64_t M, int64_t N,
-                           int64_t K, void *workspace, size_t workspace_bytes, void *stream);
+                           int64_t K, int flags, void *workspace, size_t workspace_bytes,
+                           void *stream);
 int phyai_fp8_linear_addcmul(const void *x, int64_t ldx, const void *w, const float *w_scale,
                              const void *bias, const void *residual, int64_t ld_res,
                              const void *gate, int64_t ld_gate, int64_t gate_rows, void *out,
-                             int64_t ldo, int64_t M, int64_t N, int64_t K, void *workspace,
-                             size_t workspace_bytes, void *stream);
+                             int64_t ldo, int64_t M, int64_t N, int64_t K, int flags,
+                             void *workspace, size_t workspace_bytes, void *stream);
 
 /*
  * phyai_fp8_linear for callers that cannot allocate device memory or hand over a workspace: code

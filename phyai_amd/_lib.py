@@ -13,7 +13,7 @@ import subprocess
 _PKG = os.path.dirname(os.path.abspath(__file__))
 LIB_PATH = os.path.join(_PKG, "lib", "libphyai_fp8.so")
 CSRC_DIR = os.path.join(_PKG, "csrc")
-ABI_VERSION = 7
+ABI_VERSION = 8
 
 # name -> (restype, argtypes); mirrors include/phyai_fp8.h one to one.
 _i64, _vp, _int, _sz = ctypes.c_int64, ctypes.c_void_p, ctypes.c_int, ctypes.c_size_t
@@ -23,14 +23,15 @@ SIGNATURES: dict[str, tuple[object, list[object]]] = {
     "phyai_fp8_quant_rowwise": (_int, [_vp, _i64, _i64, _i64, _vp, _vp, _vp]),
     "phyai_fp8_quant_static": (_int, [_vp, _i64, _i64, _i64, _vp, _vp, _vp]),
     "phyai_fp8_weight_quant_rowwise": (_int, [_vp, _i64, _i64, _i64, _vp, _vp, _vp]),
+    "phyai_fp8_weight_to_operand_order": (_int, [_vp, _i64, _i64, _int, _vp, _vp]),
     "phyai_fp8_linear_workspace_bytes": (_sz, [_i64, _i64, _i64, _int]),
     "phyai_fp8_gemm": (_int, [_vp, _vp, _int, _vp, _vp, _vp, _vp, _i64, _i64, _i64, _i64, _int, _vp, _sz, _vp]),
     "phyai_fp8_linear": (_int, [_vp, _i64, _vp, _vp, _vp, _vp, _i64, _i64, _i64, _i64, _int, _vp, _sz, _vp]),
     "phyai_fp8_linear_static": (_int, [_vp, _i64, _vp, _vp, _vp, _vp, _i64, _i64, _i64, _i64, _int, _vp]),
     "phyai_fp8_gemm_addcmul": (_int, [_vp, _vp, _int, _vp, _vp, _vp, _vp, _i64, _vp, _i64, _i64, _vp, _i64, _i64, _i64,
-                                      _i64, _vp, _sz, _vp]),
+                                      _i64, _int, _vp, _sz, _vp]),
     "phyai_fp8_linear_addcmul": (_int, [_vp, _i64, _vp, _vp, _vp, _vp, _i64, _vp, _i64, _i64, _vp, _i64, _i64, _i64,
-                                        _i64, _vp, _sz, _vp]),
+                                        _i64, _int, _vp, _sz, _vp]),
     "phyai_fp8_rmsnorm_quant": (_int, [_vp, _i64, _vp, _int, _i64, _i64, ctypes.c_float, _vp, _i64, _vp, _vp, _vp]),
     "phyai_fp8_adarmsnorm_quant": (_int, [_vp, _i64, _vp, _i64, _i64, _i64, _i64, ctypes.c_float, _vp, _i64, _vp,
                                           _i64, _vp, _vp, _vp]),

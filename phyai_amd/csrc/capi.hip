@@ -9,6 +9,7 @@
 #include "../../include/phyai_fp8.h"
 #include "fp8_device.h"
 #include "launch.h"
+#include "weight_layout.h"
 
 // Scratch of phyai_fp8_linear_static: one array per GPU, part of the loaded code object (zero when
 // the module is loaded), held until the process ends.  The name is only a handle on the host; the
@@ -142,6 +143,23 @@ int phyai_fp8_weight_quant_rowwise(const void* w, int64_t N, int64_t K, int64_t 
     return check_launch("phyai_fp8_weight_quant_rowwise");
 }
 
+int phyai_fp8_weight_to_operand_order(const void* w, int64_t N, int64_t K, int gated, void* out, void* stream) {
+    const char* fn = "phyai_fp8_weight_to_operand_order";
+    if (N < 0 || K <= 0) return fail(PHYAI_FP8_EINVAL, "%s: bad shape N=%lld K=%lld", fn, (long long)N, (long long)K);
+    if (N == 0) return PHYAI_FP8_OK;
+    if (!w || !out) return fail(PHYAI_FP8_EINVAL, "%s: null pointer", fn);
+    if (K % 128 != 0 || N % (gated ? 32 : 16) != 0)
+        return fail(PHYAI_FP8_EUNSUPPORTED, "%s: needs K %% 128 == 0 and N %% %d == 0, got N=%lld K=%lld", fn, gated ? 32 : 16,
+                    (long long)N, (long long)K);
+    if (!aligned(w, 16) || !aligned(out, 16)) return fail(PHYAI_FP8_EINVAL, "%s: w and out must be 16-byte aligned", fn);
+    if (N * K >= kMaxElems) return fail(PHYAI_FP8_EUNSUPPORTED, "%s: matrix larger than 2^31 elements", fn);
+    const uintptr_t a = reinterpret_cast<uintptr_t>(w), b = reinterpret_cast<uintptr_t>(out), n = (uintptr_t)(N * K);
+    if (a < b + n && b < a + n) return fail(PHYAI_FP8_EINVAL, "%s: out overlaps w (the re-lay is not in place)", fn);
+    if (phyai::launch_weight_to_operand_order(w, N, K, gated ? 1 : 0, out, static_cast<hipStream_t>(stream)) != 0)
+        return fail(PHYAI_FP8_EUNSUPPORTED, "%s: matrix too large", fn);
+    return check_launch(fn);
+}
+
 size_t phyai_fp8_linear_workspace_bytes(int64_t M, int64_t N, int64_t K, int epilogue) {
     return carve(M, N, K, epilogue & PHYAI_FP8_EPILOGUE_MASK).total;
 }
@@ -177,8 +195,21 @@ int prepare_gemm(const char* fn, const void* xq, const float* x_scale, int x_sca
         return fail(PHYAI_FP8_EINVAL, "%s: bad shape M=%lld N=%lld K=%lld", fn, (long long)M, (long long)N, (long long)K);
     const int flags = flagged_epilogue & ~PHYAI_FP8_EPILOGUE_MASK;
     const int epilogue = flagged_epilogue & PHYAI_FP8_EPILOGUE_MASK;
-    if (flags & ~PHYAI_FP8_FLAG_STREAM_WEIGHTS) return fail(PHYAI_FP8_EINVAL, "%s: unknown flag bits 0x%x", fn, flags);
+    if (flags & ~(PHYAI_FP8_FLAG_STREAM_WEIGHTS | PHYAI_FP8_FLAG_W_OPERAND_GATED))
+        return fail(PHYAI_FP8_EINVAL, "%s: unknown flag bits 0x%x", fn, flags);
     if (int rc = check_epilogue(epilogue, N)) return rc;
+    int layout = phyai::W_ROW_MAJOR;
+    if (flags & PHYAI_FP8_FLAG_W_OPERAND_GATED) {
+        const bool gated_w = (flags & PHYAI_FP8_FLAG_W_OPERAND_GATED) == PHYAI_FP8_FLAG_W_OPERAND_GATED;
+        if (!(flags & PHYAI_FP8_FLAG_W_OPERAND_ORDER))
+            return fail(PHYAI_FP8_EINVAL, "%s: flag bits 0x%x name no weight layout", fn, flags);
+        if (gated_w != phyai::epi_is_gated(epilogue))
+            return fail(PHYAI_FP8_EINVAL, "%s: a gated epilogue needs weights in the gated operand order and any other "
+                        "epilogue the plain one (epilogue %d, flags 0x%x)", fn, epilogue, flags);
+        if (K % 128 != 0)
+            return fail(PHYAI_FP8_EUNSUPPORTED, "%s: weights in operand order need K %% 128 == 0, got K=%lld", fn, (long long)K);
+        layout = gated_w ? phyai::W_OPERAND_GATED : phyai::W_OPERAND_PLAIN;
+    }
     if (K % 16 != 0 || N % 16 != 0)
         return fail(PHYAI_FP8_EUNSUPPORTED, "%s: K=%lld and N=%lld must be multiples of 16", fn, (long long)K, (long long)N);
     if (int rc = check_residual(fn, res, M, N, epilogue)) return rc;
@@ -204,6 +235,7 @@ int prepare_gemm(const char* fn, const void* xq, const float* x_scale, int x_sca
     g.ldo = ldo;
     g.epilogue = epilogue;
     g.stream_weights = (flags & PHYAI_FP8_FLAG_STREAM_WEIGHTS) ? 1 : 0;
+    g.weight_layout = layout;
     g.workspace = workspace;
     g.workspace_bytes = workspace_bytes;
     g.gate_group = 1;
@@ -267,9 +299,19 @@ int run_linear(const char* fn, const void* x, int64_t ldx, const void* w, const 
         return fail(PHYAI_FP8_EINVAL, "%s: bad shape M=%lld N=%lld K=%lld", fn, (long long)M, (long long)N, (long long)K);
     if (M == 0) return PHYAI_FP8_OK;
     const LinearCarve c = carve(M, N, K, epilogue & PHYAI_FP8_EPILOGUE_MASK);
-    if (!workspace || workspace_bytes < c.total)
+    if (!workspace || workspace_bytes < c.total) {
+        // The kernel that quantizes its own rows touches neither staged codes nor GEMM scratch: a call
+        // that it serves needs no workspace at all (x stands in for the code and scale pointers, which
+        // are never dereferenced then).
+        phyai::GemmProblem g;
+        if (x && check_quant_args(fn, x, M, K, ldx, x) == 0 &&
+            prepare_gemm(fn, x, static_cast<const float*>(x), 0, w, w_scale, bias, res, out, ldo, M, N, K, epilogue, nullptr,
+                         0, &g, x, ldx) == 0 &&
+            phyai::gemm_quantizes_itself(g))
+            return launch_prepared(fn, g, stream);
         return fail(PHYAI_FP8_EWORKSPACE, "%s: workspace of %zu bytes is too small, need %zu", fn,
                     workspace ? workspace_bytes : (size_t)0, c.total);
+    }
     if (!aligned(workspace, 256)) return fail(PHYAI_FP8_EINVAL, "%s: workspace must be 256-byte aligned", fn);
     uint8_t* ws = static_cast<uint8_t*>(workspace);
     return run_linear_at(fn, x, ldx, w, w_scale, bias, res, out, ldo, M, N, K, epilogue, ws + c.xq_off,
@@ -288,12 +330,13 @@ int phyai_fp8_gemm(const void* xq, const float* x_scale, int x_scale_is_scalar, 
 int phyai_fp8_gemm_addcmul(const void* xq, const float* x_scale, int x_scale_is_scalar, const void* w,
                            const float* w_scale, const void* bias, const void* residual, int64_t ld_res,
                            const void* gate, int64_t ld_gate, int64_t gate_rows, void* out, int64_t ldo,
-                           int64_t M, int64_t N, int64_t K, void* workspace, size_t workspace_bytes,
+                           int64_t M, int64_t N, int64_t K, int flags, void* workspace, size_t workspace_bytes,
                            void* stream) {
     if (!residual || !gate) return fail(PHYAI_FP8_EINVAL, "phyai_fp8_gemm_addcmul: null residual or gate");
+    if (flags & PHYAI_FP8_EPILOGUE_MASK) return fail(PHYAI_FP8_EINVAL, "phyai_fp8_gemm_addcmul: flags 0x%x carry an epilogue", flags);
     const ResidualSpec r = {residual, ld_res, gate, ld_gate, gate_rows};
     return run_gemm("phyai_fp8_gemm_addcmul", xq, x_scale, x_scale_is_scalar, w, w_scale, bias, r, out, ldo, M, N,
-                    K, PHYAI_FP8_EPI_NONE, workspace, workspace_bytes, stream);
+                    K, PHYAI_FP8_EPI_NONE | flags, workspace, workspace_bytes, stream);
 }
 
 int phyai_fp8_linear(const void* x, int64_t ldx, const void* w, const float* w_scale,
@@ -306,11 +349,12 @@ int phyai_fp8_linear(const void* x, int64_t ldx, const void* w, const float* w_s
 int phyai_fp8_linear_addcmul(const void* x, int64_t ldx, const void* w, const float* w_scale,
                              const void* bias, const void* residual, int64_t ld_res, const void* gate,
                              int64_t ld_gate, int64_t gate_rows, void* out, int64_t ldo, int64_t M,
-                             int64_t N, int64_t K, void* workspace, size_t workspace_bytes, void* stream) {
+                             int64_t N, int64_t K, int flags, void* workspace, size_t workspace_bytes, void* stream) {
     if (!residual || !gate) return fail(PHYAI_FP8_EINVAL, "phyai_fp8_linear_addcmul: null residual or gate");
+    if (flags & PHYAI_FP8_EPILOGUE_MASK) return fail(PHYAI_FP8_EINVAL, "phyai_fp8_linear_addcmul: flags 0x%x carry an epilogue", flags);
     const ResidualSpec r = {residual, ld_res, gate, ld_gate, gate_rows};
     return run_linear("phyai_fp8_linear_addcmul", x, ldx, w, w_scale, bias, r, out, ldo, M, N, K,
-                      PHYAI_FP8_EPI_NONE, workspace, workspace_bytes, stream);
+                      PHYAI_FP8_EPI_NONE | flags, workspace, workspace_bytes, stream);
 }
 
 int phyai_fp8_linear_static(const void* x, int64_t ldx, const void* w, const float* w_scale, const void* bias,

@@ -46,6 +46,7 @@
 #include "launch.h"
 #include "tuning.h"
 #include "splitk.h"
+#include "weight_layout.h"
 #include <stdlib.h>
 
 namespace phyai {
@@ -69,6 +70,7 @@ struct BigArgs {
     int m_tiles, n_tiles;            // tile grid; the launch is 1-D over it (see big_tile_of)
     int band;                        // tile rows per band of that order
     int by_rows;                     // the order with the roles of tile rows and columns exchanged
+    int operand_w;                   // weights in MFMA operand order (weight_layout.h)
     ResidualArgs res;
 };
 
@@ -162,7 +164,9 @@ void gemm_fp8_big_kernel(
     p.a = a_a; p.b = a_b; p.a_scale = a_a_scale; p.b_scale = a_b_scale; p.bias = a_bias; p.out = a_out;
     p.ldo = a_ldo; p.M = a_M; p.N = a_N; p.K = a_K; p.a_scale_scalar = a_a_scale_scalar;
     p.k_per_split = a_k_per_split; p.partials = a_partials; p.counters = a_counters;
-    p.m_tiles = a_m_tiles; p.n_tiles = a_n_tiles; p.band = a_band; p.by_rows = a_by_rows; p.res = a_res;
+    // a_by_rows = tile order | weights in operand order << 4
+    p.m_tiles = a_m_tiles; p.n_tiles = a_n_tiles; p.band = a_band; p.by_rows = a_by_rows & 15; p.res = a_res;
+    p.operand_w = __builtin_amdgcn_readfirstlane(a_by_rows >> 4);
     constexpr bool GATED = epi_is_gated(EPI);
     static_assert(WGM * WGN == 4, "four wavefronts per workgroup");
     constexpr int BM = WGM * 32 * TM, BN = WGN * 32 * TN;   // workgroup tile
@@ -218,18 +222,23 @@ void gemm_fp8_big_kernel(
     for (int i = 0; i < CB; ++i) {
         const int jj = (wave * CB + i) * 8 + (lane >> 3);         // column of the output tile
         int rb;
+        uint32_t ob;   // the row's place in operand order
         if constexpr (GATED) {
             const int w_ = jj / WN, j = jj % WN;
             int g = n0 + w_ * (WN / 2) + (j % (WN / 2));
             g = g < half_n ? g : half_n - 1;
             rb = (j / (WN / 2)) * half_n + g;
+            ob = operand_offset_gated((uint32_t)g, (uint32_t)(j / (WN / 2)), (uint32_t)p.K);
         } else {
             rb = n0 + jj;
             rb = rb < p.N ? rb : p.N - 1;
+            ob = operand_offset_plain((uint32_t)rb, (uint32_t)p.K);
         }
-        boff[i] = (uint32_t)rb * (uint32_t)p.K + (((lane & 7) ^ big_swizzle(jj)) << 4);
+        const uint32_t chunk = (uint32_t)((lane & 7) ^ big_swizzle(jj));
+        boff[i] = p.operand_w ? ob + chunk * kOperandChunkBytes : (uint32_t)rb * (uint32_t)p.K + (chunk << 4);
     }
     const int k_begin = SPLIT ? split_z * p.k_per_split : 0;
+    const int b_step_shift = p.operand_w ? 4 : 0;   // a K step of operand-order weights is 2 KB away, not 128 bytes
     const uint32_t lds_base = (uint32_t)(uintptr_t)lds;
     const uint32_t wave_a = __builtin_amdgcn_readfirstlane(lds_base + wave * (CA * 1024));
     const uint32_t wave_b = __builtin_amdgcn_readfirstlane(lds_base + BM * BIG_BK + wave * (CB * 1024));
@@ -238,7 +247,7 @@ void gemm_fp8_big_kernel(
         const int k = k_begin + d * BIG_BK;
         const uint32_t stage_off = (d % DEPTH) * STAGE_BYTES;
         if (c < CA) copy16_to_lds(p.a + k, aoff[c], wave_a + stage_off + c * 1024);
-        else copy16_to_lds(p.b + k, boff[c - CA], wave_b + stage_off + (c - CA) * 1024);
+        else copy16_to_lds(p.b + ((size_t)k << b_step_shift), boff[c - CA], wave_b + stage_off + (c - CA) * 1024);
     };
 
     v16f acc[TM][TN];
@@ -658,7 +667,7 @@ static void big_launch(BigArgs a, const GemmProblem& g, int splits, hipStream_t 
             grid = dim3(8 * cols * a.m_tiles, 1, 1);
         }
     }
-#define PHYAI_BIG_ARGS a.a, a.b, a.K, a.M, a.N, a.m_tiles, a.n_tiles, a.band, a.by_rows, a.k_per_split, a.a_scale, \
+#define PHYAI_BIG_ARGS a.a, a.b, a.K, a.M, a.N, a.m_tiles, a.n_tiles, a.band, a.by_rows | (a.operand_w << 4), a.k_per_split, a.a_scale, \
                        a.b_scale, a.bias, a.out, a.ldo, a.a_scale_scalar, a.partials, a.counters, a.res
     if (splits > 1) {
         if constexpr (TM == TN && (TM == 4 || DEPTH == 4))
@@ -690,6 +699,7 @@ int launch_gemm_big(const GemmProblem& g, const BigPlan& pl, hipStream_t st) {
     a.out = g.out; a.ldo = g.ldo; a.M = g.M; a.N = g.N; a.K = g.K;
     a.a_scale_scalar = g.x_scale_is_scalar;
     a.res = residual_of(g);
+    a.operand_w = g.weight_layout != W_ROW_MAJOR;
     a.k_per_split = g.K / pl.splits;
     a.counters = static_cast<int*>(g.workspace);
     a.partials = g.workspace ? reinterpret_cast<float*>(static_cast<uint8_t*>(g.workspace) + kGemmHeaderBytes) : nullptr;

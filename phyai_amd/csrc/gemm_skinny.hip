@@ -35,6 +35,7 @@
 #include "fp8_device.h"
 #include "launch.h"
 #include "tuning.h"
+#include "weight_layout.h"
 #include <stdio.h>
 #include <stdlib.h>
 
@@ -52,6 +53,7 @@ struct SkinnyArgs {
     int x_scale_scalar;
     int rounds;  // K steps are consumed in rounds of SK_WAVES * KPW
     int stream_w;  // weights with non-temporal loads
+    int operand_w; // weights in MFMA operand order (weight_layout.h; the gated form for gated epilogues)
     ResidualArgs res;
 };
 
@@ -86,7 +88,8 @@ __global__ __launch_bounds__(SK_THREADS) void gemm_fp8_skinny_kernel(
     const float* __restrict__ a_w_scale, const uint16_t* __restrict__ a_bias, int a_K, int a_N, int a_m_flags,
     uint16_t* __restrict__ a_out, int64_t a_ldo, const ResidualArgs a_res) {
     // 13 preloaded dwords: everything the operand requests and the early epilogue loads need.
-    // a_m_flags = M | stream_weights << 29 | x_scale_is_scalar << 30; the rounds follow from K.
+    // a_m_flags = M | operand-order weights << 28 | stream_weights << 29 | x_scale_is_scalar << 30; the
+    // rounds follow from K.
     SkinnyArgs p;
     p.xq = a_xq; p.w = a_w; p.x_scale = a_x_scale; p.w_scale = a_w_scale; p.bias = a_bias; p.out = a_out;
     p.ldo = a_ldo; p.M = a_m_flags & 0x0FFFFFFF; p.N = a_N; p.K = a_K; p.x_scale_scalar = (a_m_flags >> 30) & 1;
@@ -94,6 +97,16 @@ __global__ __launch_bounds__(SK_THREADS) void gemm_fp8_skinny_kernel(
     // others from the Infinity Cache (STAGED form only; the hint is ignored otherwise)
     const bool stream_w = __builtin_amdgcn_readfirstlane((a_m_flags >> 29) & 1) != 0;
     (void)stream_w;
+    // Weights in operand order: tile nt of this workgroup is unit blockIdx.x * NT + nt of the matrix (for
+    // gated epilogues the gated order is exactly the row order of a gated tile); a K step is 2 KB away
+    // instead of 128 bytes, a 16-byte chunk 256 bytes instead of 16.
+    const bool operand_w = __builtin_amdgcn_readfirstlane((a_m_flags >> 28) & 1) != 0;
+    const int w_step_shift = operand_w ? 11 : 7;
+    const uint32_t w_units = (uint32_t)a_N >> 4;
+    auto w_unit = [&](int nt) -> uint32_t {
+        const uint32_t u = blockIdx.x * NT + nt;
+        return u < w_units ? u : w_units - 1;
+    };
     p.rounds = (((a_K >> 7) + SK_WAVES - 1) / SK_WAVES + KPW - 1) / KPW;
     p.res = a_res;
     constexpr bool GATED = epi_is_gated(EPI);
@@ -203,7 +216,10 @@ __global__ __launch_bounds__(SK_THREADS) void gemm_fp8_skinny_kernel(
     if constexpr (!STAGED) {
         const uint8_t* wrow[NT];
 #pragma unroll
-        for (int nt = 0; nt < NT; ++nt) wrow[nt] = p.w + (size_t)w_row(nt, l16) * p.K + q * 16;
+        for (int nt = 0; nt < NT; ++nt)
+            wrow[nt] = operand_w ? p.w + operand_row_offset(w_unit(nt), l16, p.K) + q * kOperandChunkBytes
+                                 : p.w + (size_t)w_row(nt, l16) * p.K + q * 16;
+        const int w_hi = operand_w ? 4 * (int)kOperandChunkBytes : 64;   // chunk 4 + q
         const uint8_t* xrow[MB];
 #pragma unroll
         for (int mb = 0; mb < MB; ++mb) xrow[mb] = p.xq + (size_t)x_row(mb, l16) * p.K + q * 16;
@@ -217,10 +233,11 @@ __global__ __launch_bounds__(SK_THREADS) void gemm_fp8_skinny_kernel(
                 const int s = (rnd * KPW + j) * SK_WAVES + wave;  // wave-uniform
                 live[j] = s < total_steps;
                 const int off = (live[j] ? s : total_steps - 1) << 7;
+                const int woff_s = (live[j] ? s : total_steps - 1) << w_step_shift;
 #pragma unroll
                 for (int nt = 0; nt < NT; ++nt) {
-                    wlo[j][nt] = *reinterpret_cast<const v4i*>(wrow[nt] + off);
-                    whi[j][nt] = *reinterpret_cast<const v4i*>(wrow[nt] + off + 64);
+                    wlo[j][nt] = *reinterpret_cast<const v4i*>(wrow[nt] + woff_s);
+                    whi[j][nt] = *reinterpret_cast<const v4i*>(wrow[nt] + woff_s + w_hi);
                 }
 #pragma unroll
                 for (int mb = 0; mb < MB; ++mb) {
@@ -256,7 +273,9 @@ __global__ __launch_bounds__(SK_THREADS) void gemm_fp8_skinny_kernel(
 #pragma unroll
             // rows and K are below 2^24 and their product below 2^32 (checked by the launcher): the
             // 24-bit multiply is a full-rate instruction, the general one is not
-            for (int nt = 0; nt < NT; ++nt) woff[nt][hf] = __umul24((uint32_t)w_row(nt, r16), (uint32_t)p.K) + chunk;
+            for (int nt = 0; nt < NT; ++nt)
+                woff[nt][hf] = operand_w ? operand_row_offset(w_unit(nt), r16, p.K) + (chunk << 4)
+                                         : __umul24((uint32_t)w_row(nt, r16), (uint32_t)p.K) + chunk;
 #pragma unroll
             for (int mb = 0; mb < MB; ++mb) xoff[mb][hf] = __umul24((uint32_t)x_row(mb, r16), (uint32_t)p.K) + chunk;
         }
@@ -279,13 +298,13 @@ __global__ __launch_bounds__(SK_THREADS) void gemm_fp8_skinny_kernel(
                         for (int nt = 0; nt < NT; ++nt)
 #pragma unroll
                             for (int hf = 0; hf < 2; ++hf)
-                                copy16_to_lds_nt(p.w + ((size_t)s << 7), woff[nt][hf], dst + (nt * 2 + hf) * 1024);
+                                copy16_to_lds_nt(p.w + ((size_t)s << w_step_shift), woff[nt][hf], dst + (nt * 2 + hf) * 1024);
                     } else {
 #pragma unroll
                         for (int nt = 0; nt < NT; ++nt)
 #pragma unroll
                             for (int hf = 0; hf < 2; ++hf)
-                                copy16_to_lds(p.w + ((size_t)s << 7), woff[nt][hf], dst + (nt * 2 + hf) * 1024);
+                                copy16_to_lds(p.w + ((size_t)s << w_step_shift), woff[nt][hf], dst + (nt * 2 + hf) * 1024);
                     }
 #pragma unroll
                     for (int mb = 0; mb < MB; ++mb)
@@ -451,13 +470,13 @@ static void sk_launch_one(const SkinnyArgs& a, const dim3& grid, hipStream_t st)
     if constexpr (fits) {
         if (want && a.K * (int64_t)(a.N > a.M ? a.N : a.M) < ((int64_t)1 << 32) && a.K < (1 << 24) && a.N < (1 << 24)) {
             hipLaunchKernelGGL((gemm_fp8_skinny_kernel<MB, NT, KPW, EPI, true>), grid, dim3(SK_THREADS), 0, st,
-                               a.w, a.xq, a.x_scale, a.w_scale, a.bias, a.K, a.N, a.M | (a.x_scale_scalar ? 1 << 30 : 0) | (a.stream_w ? 1 << 29 : 0),
+                               a.w, a.xq, a.x_scale, a.w_scale, a.bias, a.K, a.N, a.M | (a.x_scale_scalar ? 1 << 30 : 0) | (a.stream_w ? 1 << 29 : 0) | (a.operand_w ? 1 << 28 : 0),
                                a.out, a.ldo, a.res);
             return;
         }
     }
     hipLaunchKernelGGL((gemm_fp8_skinny_kernel<MB, NT, KPW, EPI, false>), grid, dim3(SK_THREADS), 0, st,
-                       a.w, a.xq, a.x_scale, a.w_scale, a.bias, a.K, a.N, a.M | (a.x_scale_scalar ? 1 << 30 : 0) | (a.stream_w ? 1 << 29 : 0),
+                       a.w, a.xq, a.x_scale, a.w_scale, a.bias, a.K, a.N, a.M | (a.x_scale_scalar ? 1 << 30 : 0) | (a.stream_w ? 1 << 29 : 0) | (a.operand_w ? 1 << 28 : 0),
                        a.out, a.ldo, a.res);
 }
 
@@ -501,6 +520,7 @@ int launch_gemm_skinny(const GemmProblem& g, const SkinnyPlan& pl, hipStream_t s
     a.x_scale_scalar = g.x_scale_is_scalar;
     a.rounds = pl.rounds;
     a.stream_w = g.stream_weights;
+    a.operand_w = g.weight_layout != W_ROW_MAJOR;
     a.res = residual_of(g);
     switch (g.epilogue) {
     case EPI_NONE: return sk_launch_epi<EPI_NONE>(a, pl, st);

@@ -29,6 +29,7 @@
 
 #include "quant_device.h"
 #include "tuning.h"
+#include "weight_layout.h"
 #include <stdio.h>
 
 namespace phyai {
@@ -113,7 +114,12 @@ __global__ __launch_bounds__(FQ_THREADS) void gemm_fp8_fusedq_kernel(
 
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     const int l16 = lane & 15, q = lane >> 4;
-    const int M = a_M, N = a_N, K = a_K;
+    // a_M = M | weights in MFMA operand order << 28 (weight_layout.h; gemm_skinny.hip reads them the same way)
+    const int M = a_M & 0x0FFFFFFF, N = a_N, K = a_K;
+    // (selected with masks and shifts, not with conditions: the code between the row loads and their
+    // wait must stay free of branches, see below)
+    const uint32_t om = 0u - (uint32_t)__builtin_amdgcn_readfirstlane((a_M >> 28) & 1);   // all ones: operand order
+    const int w_step_shift = 7 + (int)(om & 4);
     const int half_n = N / 2;
     const int n_out_total = GATED ? half_n : N;
     const int col0 = blockIdx.x * (COLS_PER_TILE * NT);
@@ -173,7 +179,11 @@ __global__ __launch_bounds__(FQ_THREADS) void gemm_fp8_fusedq_kernel(
                 const int r = col0 + nt * 16 + r16;
                 wr = r < N ? r : N - 1;
             }
-            woff[nt][hf] = __umul24((uint32_t)wr, (uint32_t)K) + chunk;
+            // row-major: wr * K + 16 * chunk index; operand order: unit * 16 K + 16 * r16 + 256 * chunk index
+            const uint32_t w_units = (uint32_t)N >> 4, wu = blockIdx.x * NT + nt;
+            const uint32_t unit = wu < w_units ? wu : w_units - 1;
+            const uint32_t row = (uint32_t)wr + ((unit - (uint32_t)wr) & om);
+            woff[nt][hf] = __umul24(row, (uint32_t)K << (om & 4)) + (((uint32_t)r16 << 4) & om) + (chunk << (om & 4));
         }
     }
     const uint32_t lds_wave = __builtin_amdgcn_readfirstlane((uint32_t)(uintptr_t)smem + wave * PER_WAVE);
@@ -187,8 +197,8 @@ __global__ __launch_bounds__(FQ_THREADS) void gemm_fp8_fusedq_kernel(
         for (int nt = 0; nt < NT; ++nt)
 #pragma unroll
             for (int hf = 0; hf < 2; ++hf) {
-                if constexpr (STREAM) copy16_to_lds_nt(a_w + ((size_t)s_safe << 7), woff[nt][hf], dst + (nt * 2 + hf) * 1024);
-                else copy16_to_lds(a_w + ((size_t)s_safe << 7), woff[nt][hf], dst + (nt * 2 + hf) * 1024);
+                if constexpr (STREAM) copy16_to_lds_nt(a_w + ((size_t)s_safe << w_step_shift), woff[nt][hf], dst + (nt * 2 + hf) * 1024);
+                else copy16_to_lds(a_w + ((size_t)s_safe << w_step_shift), woff[nt][hf], dst + (nt * 2 + hf) * 1024);
             }
     }
 
@@ -486,11 +496,11 @@ static int fq_launch_one(const GemmProblem& g, const FusedPlan& pl, hipStream_t 
     } else {
         if (g.stream_weights)
             hipLaunchKernelGGL((gemm_fp8_fusedq_kernel<ROWS, NT, KPW, EPI, true>), dim3(pl.tiles, pl.msplit), dim3(FQ_THREADS), 0, st,
-                               g.w, reinterpret_cast<const uint8_t*>(g.x_bf16), g.w_scale, g.bias, g.K, g.N, g.M,
+                               g.w, reinterpret_cast<const uint8_t*>(g.x_bf16), g.w_scale, g.bias, g.K, g.N, g.M | (g.weight_layout != W_ROW_MAJOR ? 1 << 28 : 0),
                                (int)(g.ldx * 2), g.out, g.ldo, residual_of(g));
         else
             hipLaunchKernelGGL((gemm_fp8_fusedq_kernel<ROWS, NT, KPW, EPI, false>), dim3(pl.tiles, pl.msplit), dim3(FQ_THREADS), 0, st,
-                               g.w, reinterpret_cast<const uint8_t*>(g.x_bf16), g.w_scale, g.bias, g.K, g.N, g.M,
+                               g.w, reinterpret_cast<const uint8_t*>(g.x_bf16), g.w_scale, g.bias, g.K, g.N, g.M | (g.weight_layout != W_ROW_MAJOR ? 1 << 28 : 0),
                                (int)(g.ldx * 2), g.out, g.ldo, residual_of(g));
         return 0;
     }

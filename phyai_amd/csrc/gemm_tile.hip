@@ -27,6 +27,7 @@
 #include "launch.h"
 #include "tuning.h"
 #include "splitk.h"
+#include "weight_layout.h"
 #include <stdio.h>
 #include <stdlib.h>
 
@@ -47,6 +48,7 @@ struct TileArgs {
     int M, N, K;
     int a_scale_scalar;
     int k_tiles_per_split;  // in BK slabs
+    int operand_w;          // weights in MFMA operand order (weight_layout.h; needs K % 128 == 0)
     ResidualArgs res;
 };
 
@@ -105,9 +107,11 @@ __global__ __launch_bounds__(256) void gemm_fp8_tile_kernel(const TileArgs p) {
             int g = n0 + w_ * (WN / 2) + j % (WN / 2);
             g = g < half_n ? g : half_n - 1;
             r = up * half_n + g;
+            if (p.operand_w) { b_off[i] = (int)operand_offset_gated((uint32_t)g, (uint32_t)up, (uint32_t)p.K); continue; }
         } else {
             r = n0 + jj;
             r = r < p.N ? r : p.N - 1;
+            if (p.operand_w) { b_off[i] = (int)operand_offset_plain((uint32_t)r, (uint32_t)p.K); continue; }
         }
         b_off[i] = r * p.K;
     }
@@ -121,12 +125,14 @@ __global__ __launch_bounds__(256) void gemm_fp8_tile_kernel(const TileArgs p) {
     auto load_global = [&](int slab) {
         const int k = k_begin + slab * BK + lchunk * 16;
         const bool ok = k < k_end;
+        // operand order: the K step is 2 KB away and the chunk 256 bytes (K is a multiple of 128 then)
+        const uint32_t kb = p.operand_w ? ((uint32_t)(k >> 7) << 11) + (uint32_t)lchunk * kOperandChunkBytes : (uint32_t)k;
 #pragma unroll
         for (int i = 0; i < PA; ++i)
             ra[i] = ok ? *reinterpret_cast<const uint4*>(p.a + a_off[i] + k) : make_uint4(0, 0, 0, 0);
 #pragma unroll
         for (int i = 0; i < PB; ++i)
-            rb[i] = ok ? *reinterpret_cast<const uint4*>(p.b + b_off[i] + k) : make_uint4(0, 0, 0, 0);
+            rb[i] = ok ? *reinterpret_cast<const uint4*>(p.b + (uint32_t)b_off[i] + kb) : make_uint4(0, 0, 0, 0);
     };
     auto store_lds = [&](int buf) {
         uint8_t* base = lds + buf * TILE_BYTES;
@@ -465,6 +471,7 @@ int launch_gemm(const GemmProblem& g, hipStream_t st) {
     a.out = g.out; a.ldo = g.ldo; a.M = g.M; a.N = g.N; a.K = g.K;
     a.a_scale_scalar = g.x_scale_is_scalar;
     a.res = residual_of(g);
+    a.operand_w = g.weight_layout != W_ROW_MAJOR;
     a.counters = static_cast<int*>(g.workspace);
     a.partials = g.workspace ? reinterpret_cast<float*>(static_cast<uint8_t*>(g.workspace) + kHeaderBytes) : nullptr;
     const int slabs = ceil_div(g.K, BK);

@@ -14,6 +14,8 @@ int launch_weight_quant(const void* w, int64_t N, int64_t K, int64_t ldw, void* 
 int launch_quant_static(const void* x, int64_t M, int64_t K, int64_t ldx, const float* input_scale,
                         void* xq, hipStream_t st);
 int launch_debug_cast(const float* v, int64_t n, void* codes, hipStream_t st);
+// Row-major fp8 weights -> MFMA operand order (weight_layout.hip); gated: the fused gate | up form.
+int launch_weight_to_operand_order(const void* w, int64_t N, int64_t K, int gated, void* out, hipStream_t st);
 // fp8 MFMA issue-rate probe (probe_kernels.hip): out holds 2 x workgroups 64-bit counters.
 int launch_mfma_rate(int workgroups, int iters, unsigned long long* out, float* sink, hipStream_t st);
 
@@ -64,6 +66,9 @@ struct GemmProblem {
     // then never written; null for the GEMM entry points.
     const uint16_t* x_bf16;
     int64_t ldx;
+    // Layout of w (weight_layout.h): 0 row-major [N, K]; 1 MFMA operand order; 2 operand order of a fused
+    // gate | up matrix (gated epilogues only).
+    int weight_layout;
 };
 
 // What the kernels need of the above, by value.

@@ -53,6 +53,8 @@ class HipFp8Kernel:
         # set by phyai_amd.cache_plan.plan_weight_streaming on the layers whose weights should
         # pass the Infinity Cache by
         stream = bool(getattr(layer, "stream_weights", False))
+        # set by Fp8Spec.process_after_loading when it re-laid the weight in MFMA operand order
+        layout = getattr(layer, "weight_layout", None)
         spec_id = layer.spec.spec_id
         if isinstance(x, ActivationView):
             # already quantized per token by the producer (a norm with the quantizer fused in)
@@ -60,14 +62,15 @@ class HipFp8Kernel:
                 raise RuntimeError(f"HipFp8Kernel: pre-quantized activations need per-token scales and an "
                                    f"fp8_per_channel layer, got spec_id={spec_id!r}, granularity={x.granularity}")
             return ops.fp8_gemm(x.x, x.x_scale, layer.weight, layer.weight_scale, bias, epilogue=epilogue,
-                                residual=residual, gate=gate, stream_weights=stream)
+                                residual=residual, gate=gate, stream_weights=stream, weight_layout=layout)
         if spec_id == "fp8_per_channel":
             return ops.fp8_linear(x, layer.weight, layer.weight_scale, bias, epilogue=epilogue,
-                                  residual=residual, gate=gate, stream_weights=stream)
+                                  residual=residual, gate=gate, stream_weights=stream, weight_layout=layout)
         if spec_id == "fp8_per_tensor":
             act = layer.spec.quantize_activation(x, layer)
             return ops.fp8_gemm(act.x, layer.input_scale, layer.weight, layer.weight_scale, bias,
-                                epilogue=epilogue, residual=residual, gate=gate, stream_weights=stream)
+                                epilogue=epilogue, residual=residual, gate=gate, stream_weights=stream,
+                                weight_layout=layout)
         raise RuntimeError(f"HipFp8Kernel got unhandled spec_id={spec_id!r}")
 
 

@@ -89,6 +89,8 @@ class DenseMLP(nn.Module):
             self.down_proj = RowParallelLinear(
                 intermediate_size, hidden_size, input_is_parallel=True, reduce_results=True, spec=spec_out,
                 prefix=child("down_proj"), **common)
+            # a spec that re-lays weights after loading should pair gate and up rows for the epilogue
+            self.gate_up_proj.gated_pairs = bool(fuse_activation)
         else:
             self._unfused_act = _plain_act(activation)
             self._epilogue = _PLAIN_EPILOGUE[self.activation]
@@ -102,6 +104,9 @@ class DenseMLP(nn.Module):
         second = self.down_proj if self.gated else self.fc2
         if self.fuse_activation and first.supports_fused_epilogue(x):
             h = first.forward_fused(x, self._epilogue)
+        elif getattr(first, "weight_layout", None) == "operand_gated":
+            raise RuntimeError("DenseMLP: gate_up_proj holds its weight in the gated operand order, which only the "
+                               "fused activation epilogue can read, and the fused path is not available for this input")
         else:
             h, _ = first(x)
             h = self._unfused_act(h)

@@ -34,6 +34,9 @@ EPILOGUES = {
 
 WORKSPACE_HEADER_BYTES = 16384
 FLAG_STREAM_WEIGHTS = 0x100   # OR-ed into the epilogue argument of the C entry points
+FLAG_W_OPERAND_ORDER = 0x200  # weight in MFMA operand order (fp8_weight_to_operand_order), plain form
+FLAG_W_OPERAND_GATED = 0x600  # ... the form of a fused gate | up matrix (gated epilogues only)
+WEIGHT_LAYOUTS = {None: 0, "row_major": 0, "operand": FLAG_W_OPERAND_ORDER, "operand_gated": FLAG_W_OPERAND_GATED}
 
 
 def _err(op: str, msg: str) -> RuntimeError:
@@ -347,6 +350,45 @@ def fp8_weight_quant(w: torch.Tensor, *, out: torch.Tensor | None = None,
     return out, scale_out
 
 
+def fp8_weight_to_operand_order(w: torch.Tensor, *, gated: bool = False, out: torch.Tensor | None = None) -> torch.Tensor:
+    """Re-lay fp8 weights ``w[N, K]`` (row-major) into MFMA operand order: same shape and dtype, the
+    bytes in the order the kernels' lanes read them (units of 16 rows x 128 bytes of K, the 16 x 8
+    matrix of 16-byte chunks of a unit transposed).  ``gated``: ``w`` is a fused gate | up matrix and
+    the result is for gated epilogues only.  Pass the result to :func:`fp8_gemm` / :func:`fp8_linear`
+    with ``weight_layout="operand"`` (``"operand_gated"``).  Out of place.
+
+    This is what ``Fp8Spec.process_after_loading`` runs once per layer (the reference's hook for
+    "re-lay weights after loading", ``layers/quant/base.py:55-70``)."""
+    op = "fp8_weight_to_operand_order"
+    if not (isinstance(w, torch.Tensor) and w.is_cuda and w.dim() == 2 and w.is_contiguous()
+            and w.dtype in (torch.float8_e4m3fn, torch.uint8)):
+        raise _err(op, "w must be a contiguous 2-D float8_e4m3fn GPU tensor (N, K)")
+    N, K = w.shape
+    if K % 128 != 0 or N % (32 if gated else 16) != 0:
+        raise _err(op, f"needs K % 128 == 0 and N % {32 if gated else 16} == 0, got N={N}, K={K}")
+    if out is None:
+        out = torch.empty_like(w)
+    elif not (isinstance(out, torch.Tensor) and out.shape == w.shape and out.dtype == w.dtype and out.device == w.device
+              and out.is_contiguous()):
+        raise _err(op, "out must be a contiguous tensor shaped and typed like w")
+    if N == 0:
+        return out
+    rc = _lib.load().phyai_fp8_weight_to_operand_order(w.data_ptr(), N, K, 1 if gated else 0, out.data_ptr(), _stream_ptr())
+    _lib.check(rc, op)
+    return out
+
+
+def _layout_flag(op: str, weight_layout, epi: int) -> int:
+    try:
+        flag = WEIGHT_LAYOUTS[weight_layout]
+    except (KeyError, TypeError):
+        raise _err(op, f"unknown weight_layout {weight_layout!r}; expected one of {sorted(k for k in WEIGHT_LAYOUTS if k)}") from None
+    if flag and (flag == FLAG_W_OPERAND_GATED) != (epi in _GATED):
+        raise _err(op, f"weight_layout={weight_layout!r} does not go with epilogue {epi}: a gated epilogue needs "
+                       "'operand_gated', any other epilogue 'operand'")
+    return flag
+
+
 # ---- GEMM / linear --------------------------------------------------------------
 
 def _check_weight(op: str, weight: torch.Tensor, weight_scale: torch.Tensor, K: int) -> tuple[int, int]:
@@ -411,8 +453,11 @@ def _check_addcmul(op: str, residual, gate, lead: tuple[int, ...], M: int, N: in
 def fp8_gemm(xq: torch.Tensor, x_scale: torch.Tensor, weight: torch.Tensor, weight_scale: torch.Tensor,
              bias: torch.Tensor | None = None, *, epilogue=None, out: torch.Tensor | None = None,
              residual: torch.Tensor | None = None, gate: torch.Tensor | None = None,
-             stream_weights: bool = False) -> torch.Tensor:
+             stream_weights: bool = False, weight_layout: str | None = None) -> torch.Tensor:
     """``bf16(act((xq @ weight.T) * x_scale * weight_scale + bias))`` on quantized inputs.
+
+    ``weight_layout``: ``"operand"`` / ``"operand_gated"`` when ``weight`` went through
+    :func:`fp8_weight_to_operand_order`; same result as with the row-major matrix.
 
     ``stream_weights``: read the weights past the caches (see :mod:`phyai_amd.cache_plan`);
     same result, honoured by the weight-streaming kernel (small M) without a gated residual.
@@ -441,6 +486,7 @@ def fp8_gemm(xq: torch.Tensor, x_scale: torch.Tensor, weight: torch.Tensor, weig
         raise _err(op, f"x_scale must be float32 with 1 or {M} elements")
     scalar = 1 if (xs.numel() == 1 and M != 1) else 0
     bias_ptr = _check_bias(op, bias, N)
+    flags = _layout_flag(op, weight_layout, epi) | (FLAG_STREAM_WEIGHTS if stream_weights else 0)
     n_out = N // 2 if epi in _GATED else N
     r2, g2 = _check_addcmul(op, residual, gate, tuple(xq.shape[:-1]), M, N, epi, xq.device)
     out = _out_for(op, tuple(xq.shape[:-1]), n_out, out, xq.device)
@@ -451,12 +497,11 @@ def fp8_gemm(xq: torch.Tensor, x_scale: torch.Tensor, weight: torch.Tensor, weig
         rc = _lib.load().phyai_fp8_gemm_addcmul(
             x2.data_ptr(), xs.data_ptr(), scalar, weight.data_ptr(), weight_scale.data_ptr(), bias_ptr,
             r2.data_ptr(), r2.stride(0) if M > 1 else N, g2.data_ptr(), g2.stride(0) if g2.shape[0] > 1 else N,
-            g2.shape[0], out.data_ptr(), n_out, M, N, K, ws.data_ptr(), ws.numel(), _stream_ptr())
+            g2.shape[0], out.data_ptr(), n_out, M, N, K, flags, ws.data_ptr(), ws.numel(), _stream_ptr())
     else:
         rc = _lib.load().phyai_fp8_gemm(x2.data_ptr(), xs.data_ptr(), scalar, weight.data_ptr(),
                                          weight_scale.data_ptr(), bias_ptr, out.data_ptr(), n_out, M, N, K,
-                                         epi | (FLAG_STREAM_WEIGHTS if stream_weights else 0),
-                                         ws.data_ptr(), ws.numel(), _stream_ptr())
+                                         epi | flags, ws.data_ptr(), ws.numel(), _stream_ptr())
     _lib.check(rc, op)
     return out
 
@@ -464,11 +509,11 @@ def fp8_gemm(xq: torch.Tensor, x_scale: torch.Tensor, weight: torch.Tensor, weig
 def fp8_linear(x: torch.Tensor, weight: torch.Tensor, weight_scale: torch.Tensor,
                bias: torch.Tensor | None = None, *, epilogue=None, out: torch.Tensor | None = None,
                residual: torch.Tensor | None = None, gate: torch.Tensor | None = None,
-               stream_weights: bool = False) -> torch.Tensor:
+               stream_weights: bool = False, weight_layout: str | None = None) -> torch.Tensor:
     """The whole W8A8 linear on bf16 ``x[..., K]``: per-token quantization, fp8 MFMA
     GEMM, per-channel dequantization, bias and optional activation, bf16 out.
 
-    ``stream_weights``: as for :func:`fp8_gemm`.
+    ``stream_weights``, ``weight_layout``: as for :func:`fp8_gemm`.
 
     Replaces ``TorchKernel._fp8_per_channel`` (reference
     ``layers/linear/backends/torch.py:155-176``) and, with a gated ``epilogue``,
@@ -483,6 +528,7 @@ def fp8_linear(x: torch.Tensor, weight: torch.Tensor, weight_scale: torch.Tensor
     if epi in _GATED and N % 32 != 0:
         raise _err(op, f"gated epilogue needs N % 32 == 0, got {N}")
     bias_ptr = _check_bias(op, bias, N)
+    flags = _layout_flag(op, weight_layout, epi) | (FLAG_STREAM_WEIGHTS if stream_weights else 0)
     n_out = N // 2 if epi in _GATED else N
     r2, g2 = _check_addcmul(op, residual, gate, tuple(x.shape[:-1]), M, N, epi, x.device)
     out = _out_for(op, tuple(x.shape[:-1]), n_out, out, x.device)
@@ -493,12 +539,11 @@ def fp8_linear(x: torch.Tensor, weight: torch.Tensor, weight_scale: torch.Tensor
         rc = _lib.load().phyai_fp8_linear_addcmul(
             x2.data_ptr(), x2.stride(0) if M > 1 else K, weight.data_ptr(), weight_scale.data_ptr(), bias_ptr,
             r2.data_ptr(), r2.stride(0) if M > 1 else N, g2.data_ptr(), g2.stride(0) if g2.shape[0] > 1 else N,
-            g2.shape[0], out.data_ptr(), n_out, M, N, K, ws.data_ptr(), ws.numel(), _stream_ptr())
+            g2.shape[0], out.data_ptr(), n_out, M, N, K, flags, ws.data_ptr(), ws.numel(), _stream_ptr())
     else:
         rc = _lib.load().phyai_fp8_linear(x2.data_ptr(), x2.stride(0) if M > 1 else K, weight.data_ptr(),
                                            weight_scale.data_ptr(), bias_ptr, out.data_ptr(), n_out, M, N, K,
-                                           epi | (FLAG_STREAM_WEIGHTS if stream_weights else 0),
-                                           ws.data_ptr(), ws.numel(), _stream_ptr())
+                                           epi | flags, ws.data_ptr(), ws.numel(), _stream_ptr())
     _lib.check(rc, op)
     return out
 

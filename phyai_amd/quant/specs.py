@@ -55,6 +55,11 @@ class Fp8Spec:
     block_shape: tuple[int, int] | None = None
     weight_dtype: torch.dtype = torch.float8_e4m3fn
     needs_act_quant: bool = True
+    # Re-lay the weight into MFMA operand order after loading (``process_after_loading``): same
+    # results, and the kernels whose weight blocks are private to a wavefront then load them straight
+    # into registers.  Off by default: the row-major ``[N, K]`` tensor is what checkpoints hold and
+    # what other code may read.
+    operand_order: bool = False
 
     def __post_init__(self) -> None:
         if self.granularity is Granularity.BLOCK and self.block_shape is None:
@@ -89,10 +94,35 @@ class Fp8Spec:
         layer.logical_widths = list(request.logical_widths)
 
     def process_after_loading(self, layer: nn.Module) -> None:
-        """Per-tensor scales become one value per output row (reference fp8.py:128-135)."""
-        if self.granularity is Granularity.PER_TENSOR:
+        """Per-tensor scales become one value per output row (reference fp8.py:128-135); with
+        ``operand_order`` the weight is re-laid for the MFMA (the use the reference's protocol names
+        for this hook, ``layers/quant/base.py:55-70``)."""
+        if self.granularity is Granularity.PER_TENSOR and layer.weight_scale.numel() == len(layer.logical_widths) \
+                and layer.weight_scale.numel() != layer.weight.shape[0]:
             widths = torch.tensor(layer.logical_widths, device=layer.weight_scale.device)
             layer.weight_scale = _frozen(torch.repeat_interleave(layer.weight_scale.detach(), widths).contiguous())
+        if self.operand_order and self.granularity is not Granularity.BLOCK:
+            self.to_operand_order_(layer)
+
+    def to_operand_order_(self, layer: nn.Module) -> bool:
+        """Re-lay ``layer.weight`` (row-major as loaded) in place; ``layer.weight_layout`` then says
+        ``"operand"`` or, for a layer marked ``gated_pairs`` (the fused gate | up projection of an MLP
+        whose activation runs in the GEMM epilogue), ``"operand_gated"``.  Returns False, leaving the
+        layer as it is, when the shape does not allow it or the weight lives on the CPU.  A layer that
+        already says so is left alone; whoever writes row-major bytes into the weight again (the
+        checkpoint loader, ``quantize_weight_``) clears ``weight_layout`` first."""
+        from phyai_amd import ops
+
+        w = layer.weight
+        if getattr(layer, "weight_layout", None):
+            return True
+        gated = bool(getattr(layer, "gated_pairs", False))
+        n, k = w.shape
+        if not w.is_cuda or k % 128 != 0 or n % (32 if gated else 16) != 0:
+            return False
+        w.data.copy_(ops.fp8_weight_to_operand_order(w.data, gated=gated))
+        layer.weight_layout = "operand_gated" if gated else "operand"
+        return True
 
     # -- activation quantization (reference fp8.py:137-157) ----------------------
     def quantize_activation(self, x: torch.Tensor, layer: nn.Module) -> ActivationView:
@@ -116,6 +146,7 @@ class Fp8Spec:
             raise RuntimeError("quantize_weight_ is defined for PER_CHANNEL only")
         if tuple(w_bf16.shape) != tuple(layer.weight.shape):
             raise ValueError(f"weight shape {tuple(w_bf16.shape)} != {tuple(layer.weight.shape)}")
+        layer.weight_layout = None   # row-major again until process_after_loading re-lays it
         ops.fp8_weight_quant(w_bf16.to(device=layer.weight.device, dtype=torch.bfloat16).contiguous(),
                              out=layer.weight.data, scale_out=layer.weight_scale.data)
 

@@ -172,6 +172,17 @@ def load_pretrained(model: nn.Module, source: "str | Path | Iterable[str | Path]
             (report.optional_missing if hf_key in optional else report.missing).append(hf_key)
     if strict and (report.missing or report.unexpected):
         raise RuntimeError(f"load_pretrained strict failure: {report.summary()}")
+    # A weight that an earlier post_load re-laid in MFMA operand order holds row-major bytes again
+    # once every tensor that feeds it was loaded; a reload of only some of them would mix the two.
+    for module in model.modules():
+        if getattr(module, "weight_layout", None):
+            keys = [k for k, _ in getattr(getattr(module, "weight", None), "hf_keys", None) or []]
+            hits = [k in seen for k in keys]
+            if keys and all(hits):
+                module.weight_layout = None
+            elif any(hits):
+                raise RuntimeError(f"load_pretrained: {type(module).__name__} holds its weight in operand order and the "
+                                   f"checkpoint reloads only part of it ({[k for k, h in zip(keys, hits) if h]})")
     for module in model.modules():
         post = getattr(module, "post_load", None)
         if callable(post):

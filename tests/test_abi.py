@@ -43,6 +43,7 @@ def test_workspace_query_and_argument_validation_without_gpu():
 
     lib = _lib.load()
     hdr = 16384
+    buf0 = (ctypes.c_char * 64)()
     assert lib.phyai_fp8_linear_workspace_bytes(50, 1024, 4096, 0) >= hdr + 50 * 4096
     assert lib.phyai_fp8_linear_workspace_bytes(0, 1024, 4096, 0) >= hdr
     # null pointers / bad shapes are rejected before anything is launched
@@ -54,8 +55,20 @@ def test_workspace_query_and_argument_validation_without_gpu():
     assert lib.phyai_fp8_gemm(None, None, 0, None, None, None, None, 64, 0, 64, 64, 0, None, 0, None) == 0
     # flag bits ride in the epilogue argument: the known one is accepted, others are not
     assert lib.phyai_fp8_gemm(None, None, 0, None, None, None, None, 64, 0, 64, 64, 0x100 | 1, None, 0, None) == 0
-    assert lib.phyai_fp8_gemm(None, None, 0, None, None, None, None, 64, 4, 64, 64, 0x200, None, 0, None) == -1
+    assert lib.phyai_fp8_gemm(None, None, 0, None, None, None, None, 64, 4, 64, 64, 0x800, None, 0, None) == -1
     assert b"flag" in lib.phyai_fp8_last_error()
+    # weight layout flags: operand order needs K % 128 == 0, the gated form goes with gated epilogues only
+    assert lib.phyai_fp8_gemm(None, None, 0, None, None, None, None, 64, 4, 64, 64, 0x200, None, 0, None) == -2
+    assert b"K % 128" in lib.phyai_fp8_last_error()
+    assert lib.phyai_fp8_gemm(None, None, 0, None, None, None, None, 64, 0, 64, 128, 0x200, None, 0, None) == 0
+    assert lib.phyai_fp8_gemm(None, None, 0, None, None, None, None, 64, 0, 64, 128, 0x600 | 1, None, 0, None) == 0
+    assert lib.phyai_fp8_gemm(None, None, 0, None, None, None, None, 64, 4, 64, 128, 0x600, None, 0, None) == -1
+    assert lib.phyai_fp8_gemm(None, None, 0, None, None, None, None, 64, 4, 64, 128, 0x200 | 1, None, 0, None) == -1
+    assert lib.phyai_fp8_gemm(None, None, 0, None, None, None, None, 64, 4, 64, 128, 0x400, None, 0, None) == -1
+    assert lib.phyai_fp8_weight_to_operand_order(None, 0, 128, 0, None, None) == 0
+    assert lib.phyai_fp8_weight_to_operand_order(None, 16, 128, 0, None, None) == -1
+    assert lib.phyai_fp8_weight_to_operand_order(None, 16, 128, 1, None, None) == -1   # null before the N % 32 check
+    assert lib.phyai_fp8_weight_to_operand_order(ctypes.addressof(buf0), 16, 64, 0, ctypes.addressof(buf0), None) == -2
     assert lib.phyai_fp8_linear_workspace_bytes(50, 1024, 4096, 0x100) == lib.phyai_fp8_linear_workspace_bytes(50, 1024, 4096, 0)
     buf = (ctypes.c_char * 64)()
     assert lib.phyai_fp8_linear(ctypes.addressof(buf), 64, None, None, None, None, 64, 4, 64, 64, 0, None, 0, None) == -3
