@@ -189,6 +189,36 @@ int phyai_fp8_linear_addcmul(const void *x, int64_t ldx, const void *w, const fl
                              void *workspace, size_t workspace_bytes, void *stream);
 
 /*
+ * The two projections of an MLP as one call: out = W2 . act(W1 . x), both W8A8 with per-token
+ * quantization of their input (x, then the activation's bf16 output h, which stays in the workspace).
+ * Replaces DenseMLP.forward (layers/mlp/dense_mlp.py:256-265: gate_up_proj / fc1, the activation
+ * launch, down_proj / fc2) for fp8 per-channel layers.  `epilogue` is the first projection's
+ * activation (any PHYAI_FP8_EPI_* but NONE): w1 is [N1, H] with N1 = 2 I for the gated ones (gate | up
+ * fused, dense_mlp.py:11-15) and N1 = I otherwise; w2 is [O, I].  flags1 / flags2: PHYAI_FP8_FLAG_* bits of
+ * the two weight matrices (layout, streaming).  residual / gate (both or neither; residual [M, O], gate
+ * [gate_rows, O]) put the decoder layer's addcmul behind the second projection as in
+ * phyai_fp8_linear_addcmul.  Same bits as phyai_fp8_linear (epilogue) followed by
+ * phyai_fp8_linear[_addcmul] on its output.
+ *
+ * What the one call buys: when both projections are served by the kernel that quantizes its own token
+ * rows (M <= 128, H <= 2048, I <= 4096, see phyai_fp8_describe_mlp_plan), the first one also leaves the
+ * |h| maximum of every token row per workgroup column in the workspace, and the second one starts its
+ * conversions from those instead of first passing over its rows - which is what makes one launch pay
+ * for a down projection with K = 4096.  Otherwise it is the two linears back to back.
+ * Workspace: phyai_fp8_mlp_workspace_bytes(), same rules as for phyai_fp8_linear.
+ */
+size_t phyai_fp8_mlp_workspace_bytes(int64_t M, int64_t H, int64_t I, int64_t O, int epilogue);
+int phyai_fp8_mlp(const void *x, int64_t ldx, const void *w1, const float *w1_scale, const void *bias1,
+                  int flags1, const void *w2, const float *w2_scale, const void *bias2, int flags2,
+                  const void *residual, int64_t ld_res, const void *gate, int64_t ld_gate,
+                  int64_t gate_rows, void *out, int64_t ldo, int64_t M, int64_t H, int64_t I,
+                  int64_t O, int epilogue, void *workspace, size_t workspace_bytes, void *stream);
+/* "row maxima handed over: <first> | <second>" or "<first> | <second>", each part as
+ * phyai_fp8_describe_linear_plan reports it (row-major weights; host only). */
+int phyai_fp8_describe_mlp_plan(int64_t M, int64_t H, int64_t I, int64_t O, int epilogue, char *buf,
+                                size_t n);
+
+/*
  * phyai_fp8_linear for callers that cannot allocate device memory or hand over a workspace: code
  * under HIP graph capture, tight serving loops, harnesses that forbid hipMalloc.  No counterpart
  * in the reference (its linear returns a tensor from torch's caching allocator,

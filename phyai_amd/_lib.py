@@ -27,6 +27,10 @@ SIGNATURES: dict[str, tuple[object, list[object]]] = {
     "phyai_fp8_linear_workspace_bytes": (_sz, [_i64, _i64, _i64, _int]),
     "phyai_fp8_gemm": (_int, [_vp, _vp, _int, _vp, _vp, _vp, _vp, _i64, _i64, _i64, _i64, _int, _vp, _sz, _vp]),
     "phyai_fp8_linear": (_int, [_vp, _i64, _vp, _vp, _vp, _vp, _i64, _i64, _i64, _i64, _int, _vp, _sz, _vp]),
+    "phyai_fp8_mlp_workspace_bytes": (_sz, [_i64, _i64, _i64, _i64, _int]),
+    "phyai_fp8_mlp": (_int, [_vp, _i64, _vp, _vp, _vp, _int, _vp, _vp, _vp, _int, _vp, _i64, _vp, _i64, _i64, _vp, _i64,
+                             _i64, _i64, _i64, _i64, _int, _vp, _sz, _vp]),
+    "phyai_fp8_describe_mlp_plan": (_int, [_i64, _i64, _i64, _i64, _int, ctypes.c_char_p, _sz]),
     "phyai_fp8_linear_static": (_int, [_vp, _i64, _vp, _vp, _vp, _vp, _i64, _i64, _i64, _i64, _int, _vp]),
     "phyai_fp8_gemm_addcmul": (_int, [_vp, _vp, _int, _vp, _vp, _vp, _vp, _i64, _vp, _i64, _i64, _vp, _i64, _i64, _i64,
                                       _i64, _int, _vp, _sz, _vp]),

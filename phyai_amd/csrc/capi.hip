@@ -357,6 +357,80 @@ int phyai_fp8_linear_addcmul(const void* x, int64_t ldx, const void* w, const fl
                       PHYAI_FP8_EPI_NONE | flags, workspace, workspace_bytes, stream);
 }
 
+namespace {
+// Workspace of phyai_fp8_mlp: [scratch of either linear][h: M x I bf16][row maxima: M x 64 x 16 bit].
+struct MlpCarve {
+    size_t linear_bytes, h_off, amax_off, total;
+    LinearCarve first, second;
+};
+MlpCarve mlp_carve(int64_t M, int64_t H, int64_t I, int64_t O, int epilogue) {
+    MlpCarve c;
+    const int64_t n1 = phyai::epi_is_gated(epilogue) ? 2 * I : I;
+    c.first = carve(M, n1, H, epilogue);
+    c.second = carve(M, O, I, PHYAI_FP8_EPI_NONE);
+    c.linear_bytes = c.first.total > c.second.total ? c.first.total : c.second.total;
+    c.h_off = c.linear_bytes;
+    c.amax_off = c.h_off + align_up((size_t)(M > 0 ? M : 0) * (size_t)(I > 0 ? I : 0) * 2, 256);
+    c.total = c.amax_off + align_up((size_t)(M > 0 ? M : 0) * phyai::kRowAmaxSlots * 2, 256);
+    return c;
+}
+}  // namespace
+
+size_t phyai_fp8_mlp_workspace_bytes(int64_t M, int64_t H, int64_t I, int64_t O, int epilogue) {
+    return mlp_carve(M, H, I, O, epilogue & PHYAI_FP8_EPILOGUE_MASK).total;
+}
+
+int phyai_fp8_mlp(const void* x, int64_t ldx, const void* w1, const float* w1_scale, const void* bias1, int flags1,
+                  const void* w2, const float* w2_scale, const void* bias2, int flags2, const void* residual,
+                  int64_t ld_res, const void* gate, int64_t ld_gate, int64_t gate_rows, void* out, int64_t ldo, int64_t M,
+                  int64_t H, int64_t I, int64_t O, int epilogue, void* workspace, size_t workspace_bytes, void* stream) {
+    const char* fn = "phyai_fp8_mlp";
+    if (M < 0 || H <= 0 || I <= 0 || O <= 0)
+        return fail(PHYAI_FP8_EINVAL, "%s: bad shape M=%lld H=%lld I=%lld O=%lld", fn, (long long)M, (long long)H, (long long)I, (long long)O);
+    if ((epilogue & ~PHYAI_FP8_EPILOGUE_MASK) || epilogue <= PHYAI_FP8_EPI_NONE || epilogue > PHYAI_FP8_EPI_GELU_ERF)
+        return fail(PHYAI_FP8_EINVAL, "%s: epilogue %d is not an activation", fn, epilogue);
+    if ((flags1 | flags2) & PHYAI_FP8_EPILOGUE_MASK) return fail(PHYAI_FP8_EINVAL, "%s: flags carry an epilogue", fn);
+    if ((residual == nullptr) != (gate == nullptr)) return fail(PHYAI_FP8_EINVAL, "%s: residual and gate go together", fn);
+    if (M == 0) return PHYAI_FP8_OK;
+    const MlpCarve c = mlp_carve(M, H, I, O, epilogue);
+    if (!workspace || workspace_bytes < c.total)
+        return fail(PHYAI_FP8_EWORKSPACE, "%s: workspace of %zu bytes is too small, need %zu", fn,
+                    workspace ? workspace_bytes : (size_t)0, c.total);
+    if (!aligned(workspace, 256)) return fail(PHYAI_FP8_EINVAL, "%s: workspace must be 256-byte aligned", fn);
+    uint8_t* ws = static_cast<uint8_t*>(workspace);
+    void* h = ws + c.h_off;
+    uint16_t* table = reinterpret_cast<uint16_t*>(ws + c.amax_off);
+    const int64_t n1 = phyai::epi_is_gated(epilogue) ? 2 * I : I;
+    const ResidualSpec res = {residual, ld_res, gate, ld_gate, gate_rows};
+    // both problems are validated before anything is enqueued
+    phyai::GemmProblem g1, g2;
+    if (int rc = check_quant_args(fn, x, M, H, ldx, ws + c.first.xq_off)) return rc;
+    if (int rc = prepare_gemm(fn, ws + c.first.xq_off, reinterpret_cast<float*>(ws + c.first.xs_off), 0, w1, w1_scale, bias1,
+                              ResidualSpec{}, h, I, M, n1, H, epilogue | flags1, workspace, c.first.gemm_bytes, &g1, x, ldx))
+        return rc;
+    if (int rc = prepare_gemm(fn, ws + c.second.xq_off, reinterpret_cast<float*>(ws + c.second.xs_off), 0, w2, w2_scale, bias2,
+                              res, out, ldo, M, O, I, PHYAI_FP8_EPI_NONE | flags2, workspace, c.second.gemm_bytes, &g2, h, I))
+        return rc;
+    const int slots = phyai::gemm_row_maxima_slots(g1);
+    if (slots > 0) {
+        g2.amax_in = table;
+        g2.amax_parts = slots;
+        if (phyai::gemm_takes_row_maxima(g2)) g1.amax_out = table;
+        else g2.amax_in = nullptr;
+    }
+    const hipStream_t st = static_cast<hipStream_t>(stream);
+    if (!phyai::gemm_quantizes_itself(g1)) {
+        phyai::launch_quant_rowwise(x, M, H, ldx, ws + c.first.xq_off, reinterpret_cast<float*>(ws + c.first.xs_off), st);
+        if (int rc = check_launch(fn)) return rc;
+    }
+    if (int rc = launch_prepared(fn, g1, stream)) return rc;
+    if (!phyai::gemm_quantizes_itself(g2)) {
+        phyai::launch_quant_rowwise(h, M, I, I, ws + c.second.xq_off, reinterpret_cast<float*>(ws + c.second.xs_off), st);
+        if (int rc = check_launch(fn)) return rc;
+    }
+    return launch_prepared(fn, g2, stream);
+}
+
 int phyai_fp8_linear_static(const void* x, int64_t ldx, const void* w, const float* w_scale, const void* bias,
                             void* out, int64_t ldo, int64_t M, int64_t N, int64_t K, int epilogue, void* stream) {
     const char* fn = "phyai_fp8_linear_static";
@@ -487,6 +561,23 @@ int phyai_fp8_describe_linear_plan(int64_t M, int64_t N, int64_t K, int epilogue
     if (K % 16 != 0 || N % 16 != 0)
         return fail(PHYAI_FP8_EUNSUPPORTED, "phyai_fp8_describe_linear_plan: K=%lld and N=%lld must be multiples of 16", (long long)K, (long long)N);
     const int len = phyai::describe_linear_plan((int)M, (int)N, (int)K, epilogue, buf, n);
+    buf[n - 1] = 0;
+    return len;
+}
+
+int phyai_fp8_describe_mlp_plan(int64_t M, int64_t H, int64_t I, int64_t O, int epilogue, char* buf, size_t n) {
+    const char* fn = "phyai_fp8_describe_mlp_plan";
+    if (!buf || n == 0) return fail(PHYAI_FP8_EINVAL, "%s: no buffer", fn);
+    buf[0] = 0;
+    if (M < 0 || H <= 0 || I <= 0 || O <= 0 || M >= kMaxElems || H >= kMaxElems || I >= kMaxElems || O >= kMaxElems)
+        return fail(PHYAI_FP8_EINVAL, "%s: bad shape", fn);
+    if (epilogue <= PHYAI_FP8_EPI_NONE || epilogue > PHYAI_FP8_EPI_GELU_ERF)
+        return fail(PHYAI_FP8_EINVAL, "%s: epilogue %d is not an activation", fn, epilogue);
+    const int64_t n1 = phyai::epi_is_gated(epilogue) ? 2 * I : I;
+    if (int rc = check_epilogue(epilogue, n1)) return rc;
+    if (H % 16 != 0 || I % 16 != 0 || O % 16 != 0)
+        return fail(PHYAI_FP8_EUNSUPPORTED, "%s: H, I and O must be multiples of 16", fn);
+    const int len = phyai::describe_mlp_plan((int)M, (int)H, (int)I, (int)O, epilogue, buf, n);
     buf[n - 1] = 0;
     return len;
 }

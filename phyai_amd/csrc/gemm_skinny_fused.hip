@@ -70,27 +70,47 @@ __device__ __forceinline__ float fq_bpermute(float v, int src_lane) {
     return __uint_as_float((uint32_t)__builtin_amdgcn_ds_bpermute(src_lane << 2, (int)__float_as_uint(v)));
 }
 
+// Row maxima handed from one linear to the next (the gate | up projection of an MLP to its down
+// projection): table[M][64] of bf16 bit patterns of |value| maxima, one slot per workgroup column of
+// the producer; the consumer takes the maximum over the first `parts` slots of a row.  Plain stores
+// and loads, no atomics, nothing to reset between calls.
+constexpr int kAmaxSlots = 64;   // slots (16-bit) per token row: 128 bytes
+struct AmaxOut {
+    uint16_t* table;   // null: do not produce
+};
+
 // ROWS: token rows per workgroup (8, 16 or 32; grid.y workgroups cover M); NT: 16-row weight tiles
 // per workgroup; KPW: K steps per wavefront (K <= 128 * 8 * KPW, one round).
 //
 // Between the row loads and the wait for them the code is straight-line on purpose: the loaded
 // registers are live behind the compiler's back, and any branch there lets it merge values with
-// copies that would read them too early.  Hence the weight copies are issued for every K step slot
-// (a slot past the end copies the last step again; it is never multiplied), which also keeps the
-// number of copies younger than the row loads a compile-time constant, and the cache policy of the
-// weight copies (STREAM: non-temporal) is a template parameter, not a run-time branch.
-template <int ROWS, int NT, int KPW, int EPI, bool STREAM>
+// copies that would read them too early.  Hence the weight requests are issued for every K step slot
+// (a slot past the end fetches the last step again; it is never multiplied), which also keeps the
+// number of requests younger than the row loads a compile-time constant, and the cache policy of the
+// weight requests (STREAM: non-temporal) is a template parameter, not a run-time branch.
+//
+// DIRECT: the weights are in MFMA operand order (weight_layout.h): lane i of a wavefront wants bytes
+// [16 i, 16 i + 16) and [1024 + 16 i, ...) of a 2 KB unit, so every request is 1 KB in a row and goes
+// straight into registers; LDS then holds only the activation codes.  Otherwise the weights are
+// row-major or in operand order and are staged through the wavefront's LDS slice.
+//
+// AMAX_IN: the row maxima come from the producer of the activations (AmaxOut of an earlier launch)
+// instead of being found here: no table of per-wavefront maxima, no barrier before the conversions.
+template <int ROWS, int NT, int KPW, int EPI, bool STREAM, bool DIRECT, bool AMAX_IN>
 __global__ __launch_bounds__(FQ_THREADS) void gemm_fp8_fusedq_kernel(
-    const uint8_t* __restrict__ a_w, const uint8_t* __restrict__ a_x, const float* __restrict__ a_w_scale,
-    const uint16_t* __restrict__ a_bias, int a_K, int a_N, int a_M, int a_ldx_bytes, uint16_t* __restrict__ a_out,
-    int64_t a_ldo, const ResidualArgs a_res) {
+    const uint8_t* __restrict__ a_w, const uint8_t* __restrict__ a_x, int a_K, int a_N, int a_M, int a_ldx_bytes,
+    const uint8_t* __restrict__ a_amax_in, int a_amax_parts, const float* __restrict__ a_w_scale,
+    const uint16_t* __restrict__ a_bias, uint16_t* __restrict__ a_out, int64_t a_ldo, const ResidualArgs a_res,
+    const AmaxOut a_amax_out) {
     constexpr bool GATED = epi_is_gated(EPI);
     constexpr int MB = (ROWS + 15) / 16;              // 16-row token blocks (the last one may be half used)
     constexpr int COLS_PER_TILE = GATED ? 8 : 16;
-    // One K step of staging: NT weight blocks of 2 KB (16 rows x 128 bytes) and the codes of the token
-    // rows; an 8-row workgroup keeps only the 1 KB of its 8 rows (the MFMA's other 8 columns re-read them).
+    // One K step of staging: NT weight blocks of 2 KB (16 rows x 128 bytes; none when they go straight to
+    // registers) and the codes of the token rows; an 8-row workgroup keeps only the 1 KB of its 8 rows
+    // (the MFMA's other 8 columns re-read them).
     constexpr int XB = ROWS < 16 ? ROWS * 128 : 2048;
-    constexpr int STEP_BYTES = NT * 2048 + MB * XB;
+    constexpr int WB = DIRECT ? 0 : NT * 2048;        // staged weight bytes per K step
+    constexpr int STEP_BYTES = WB + MB * XB;
     constexpr int RED_PER_WAVE = NT * MB * kWave * (int)sizeof(v4f);
     constexpr int STAGE_PER_WAVE = KPW * STEP_BYTES;
     constexpr int PER_WAVE = STAGE_PER_WAVE > RED_PER_WAVE ? STAGE_PER_WAVE : RED_PER_WAVE;
@@ -98,16 +118,21 @@ __global__ __launch_bounds__(FQ_THREADS) void gemm_fp8_fusedq_kernel(
     // leaves no room: then it lies over the first wavefront's code block of K step 0, which nobody
     // writes before a second barrier has seen every wavefront read the table.
     constexpr int TBL_ROWS = ROWS < 64 ? ROWS : 64;
-    constexpr bool TBL_ALIASED = FQ_WAVES * PER_WAVE + FQ_WAVES * 64 * 4 > 160 * 1024;
+    constexpr bool TBL_ALIASED = !AMAX_IN && FQ_WAVES * PER_WAVE + FQ_WAVES * 64 * 4 > 160 * 1024;
     static_assert(!TBL_ALIASED || FQ_WAVES * TBL_ROWS * 4 <= XB, "aliased table does not fit a code block");
     static_assert(ROWS == 8 || ROWS % 16 == 0, "token rows per workgroup");   // (4-row workgroups were measured: slower)
-    static_assert(FQ_WAVES * PER_WAVE + (TBL_ALIASED ? 0 : FQ_WAVES * 64 * 4) <= 160 * 1024, "staging does not fit the LDS");
+    static_assert(FQ_WAVES * PER_WAVE + ((TBL_ALIASED || AMAX_IN) ? 0 : FQ_WAVES * 64 * 4) <= 160 * 1024, "staging does not fit the LDS");
+    static_assert(!AMAX_IN || (ROWS <= 16 && EPI == EPI_NONE), "row maxima are handed to plain projections of up to 16 rows per workgroup");
     constexpr int ROLE_ROUNDS = (NT * MB + FQ_WAVES - 1) / FQ_WAVES;
+    constexpr int AL = AMAX_IN ? (ROWS + 7) / 8 : 0;  // loads of handed-over maxima per lane: 8 rows x 8 lanes x 16 bytes each
+    constexpr int YOUNGER = KPW * NT * 2;             // weight requests issued behind the row loads
     auto rows_in_block = [](int mb) constexpr { return ROWS - 16 * mb < 16 ? ROWS - 16 * mb : 16; };
 
     __shared__ __attribute__((aligned(1024))) uint8_t smem[FQ_WAVES * PER_WAVE];
-    __shared__ uint32_t amax_own[TBL_ALIASED ? 1 : FQ_WAVES * 64];
-    uint32_t* amax_tbl = TBL_ALIASED ? reinterpret_cast<uint32_t*>(smem + NT * 2048) : amax_own;   // [wavefront][TBL_ROWS]
+    __shared__ uint32_t amax_own[(TBL_ALIASED || AMAX_IN) ? 1 : FQ_WAVES * 64];
+    constexpr bool MAKES_AMAX = EPI != EPI_NONE;      // AmaxOut exists for the epilogues an MLP's first projection has
+    __shared__ uint32_t amax_made[MAKES_AMAX ? 64 : 1];   // AmaxOut: maxima of this workgroup's outputs per token row
+    uint32_t* amax_tbl = TBL_ALIASED ? reinterpret_cast<uint32_t*>(smem + WB) : amax_own;   // [wavefront][TBL_ROWS]
     auto red = [&](int w, int nt, int mb, int l) -> v4f& {
         return reinterpret_cast<v4f*>(smem + w * PER_WAVE)[(nt * MB + mb) * kWave + l];
     };
@@ -117,8 +142,8 @@ __global__ __launch_bounds__(FQ_THREADS) void gemm_fp8_fusedq_kernel(
     // a_M = M | weights in MFMA operand order << 28 (weight_layout.h; gemm_skinny.hip reads them the same way)
     const int M = a_M & 0x0FFFFFFF, N = a_N, K = a_K;
     // (selected with masks and shifts, not with conditions: the code between the row loads and their
-    // wait must stay free of branches, see below)
-    const uint32_t om = 0u - (uint32_t)__builtin_amdgcn_readfirstlane((a_M >> 28) & 1);   // all ones: operand order
+    // wait must stay free of branches, see above)
+    const uint32_t om = DIRECT ? ~0u : 0u - (uint32_t)__builtin_amdgcn_readfirstlane((a_M >> 28) & 1);   // all ones: operand order
     const int w_step_shift = 7 + (int)(om & 4);
     const int half_n = N / 2;
     const int n_out_total = GATED ? half_n : N;
@@ -127,9 +152,20 @@ __global__ __launch_bounds__(FQ_THREADS) void gemm_fp8_fusedq_kernel(
     const int m_base = blockIdx.y * ROWS;
 
     // ---- 1a. this wavefront's K steps of the activation rows, bf16, straight into registers --------
+    // (with AMAX_IN, in front of them, the maxima the producer left for this workgroup's rows: lane i
+    // takes 8 slots of row i / 8)
     // instruction i of block mb covers rows 4i .. 4i+3 of the block: 16 lanes per row, 16 bytes
     // (8 elements) per lane, 256 bytes = one K step per row.  Rows past M repeat row M - 1.
     const int xr = lane >> 4, xc = lane & 15;
+    v4i am[AL > 0 ? AL : 1];
+    if constexpr (AMAX_IN) {
+#pragma unroll
+        for (int a = 0; a < AL; ++a) {
+            int r = m_base + a * 8 + (lane >> 3);
+            r = r < M ? r : M - 1;
+            am[a] = fq_load16_async(a_amax_in, (uint32_t)r * (kAmaxSlots * 2) + (lane & 7) * 16);
+        }
+    }
     v4i xv[KPW][MB][4];
 #pragma unroll
     for (int j = 0; j < KPW; ++j) {
@@ -152,54 +188,77 @@ __global__ __launch_bounds__(FQ_THREADS) void gemm_fp8_fusedq_kernel(
                 }
             }
     }
-    // Every wavefront's row loads go out before any wavefront's weight copies: the CU's memory pipeline
+    // Every wavefront's row loads go out before any wavefront's weight requests: the CU's memory pipeline
     // serves requests in order, and a wavefront that starts late would otherwise queue its few row loads
-    // behind the 16 KB of copies of each earlier one - the rows, not the weights, are what the workgroup
+    // behind the 16 KB of weights of each earlier one - the rows, not the weights, are what the workgroup
     // waits for first.  (A bare barrier: nothing is awaited, only the order of issue is fixed.)  Measured:
     // o 2048 -> 1024 at M = 50 4.54 -> 4.32 us; with one K step per wavefront (K = 1024) the later start
-    // of the weight copies costs as much as the rows gain (gate_up 6.33 -> 6.41 us), so only K > 1024.
+    // of the weight requests costs as much as the rows gain (gate_up 6.33 -> 6.41 us), so only K > 1024.
     if constexpr (KPW >= 2) __builtin_amdgcn_s_barrier();
-    // ---- 1b. the weights of the same K steps, global -> LDS (as in gemm_skinny.hip) -----------------
-    const int c_row = lane >> 3, c_slot = lane & 7;
-    uint32_t woff[NT][2];
-#pragma unroll
-    for (int hf = 0; hf < 2; ++hf) {
-        const int r16 = hf * 8 + c_row;
-        const uint32_t chunk = (uint32_t)((c_slot ^ ((r16 >> 1) & 7)) << 4);
-#pragma unroll
-        for (int nt = 0; nt < NT; ++nt) {
-            int wr;
-            if constexpr (GATED) {
-                // rows 4p .. 4p+3 of a gated tile: gate columns 2p, 2p+1, then up columns 2p, 2p+1, so
-                // that an MFMA lane (which owns four consecutive tile rows) holds both halves of two
-                // output columns and all 64 lanes take part in the epilogue
-                const int g = col0 + nt * 8 + 2 * (r16 >> 2) + (r16 & 1);
-                wr = ((r16 & 2) ? half_n : 0) + (g < half_n ? g : half_n - 1);
-            } else {
-                const int r = col0 + nt * 16 + r16;
-                wr = r < N ? r : N - 1;
-            }
-            // row-major: wr * K + 16 * chunk index; operand order: unit * 16 K + 16 * r16 + 256 * chunk index
-            const uint32_t w_units = (uint32_t)N >> 4, wu = blockIdx.x * NT + nt;
-            const uint32_t unit = wu < w_units ? wu : w_units - 1;
-            const uint32_t row = (uint32_t)wr + ((unit - (uint32_t)wr) & om);
-            woff[nt][hf] = __umul24(row, (uint32_t)K << (om & 4)) + (((uint32_t)r16 << 4) & om) + (chunk << (om & 4));
-        }
-    }
+    // ---- 1b. the weights of the same K steps: into registers, or global -> LDS (as in gemm_skinny.hip) --
     const uint32_t lds_wave = __builtin_amdgcn_readfirstlane((uint32_t)(uintptr_t)smem + wave * PER_WAVE);
     uint8_t* my_stage = smem + wave * PER_WAVE;
+    v4i wlo[DIRECT ? KPW : 1][DIRECT ? NT : 1], whi[DIRECT ? KPW : 1][DIRECT ? NT : 1];
+    if constexpr (DIRECT) {
+        const uint32_t w_units = (uint32_t)N >> 4;
 #pragma unroll
-    for (int j = 0; j < KPW; ++j) {
-        const int s = __builtin_amdgcn_readfirstlane(j * FQ_WAVES + wave);
-        const int s_safe = s < total_steps ? s : total_steps - 1;
-        const uint32_t dst = lds_wave + j * STEP_BYTES;
+        for (int j = 0; j < KPW; ++j) {
+            const int s = __builtin_amdgcn_readfirstlane(j * FQ_WAVES + wave);
+            const uint32_t s_safe = s < total_steps ? s : total_steps - 1;
 #pragma unroll
-        for (int nt = 0; nt < NT; ++nt)
-#pragma unroll
-            for (int hf = 0; hf < 2; ++hf) {
-                if constexpr (STREAM) copy16_to_lds_nt(a_w + ((size_t)s_safe << w_step_shift), woff[nt][hf], dst + (nt * 2 + hf) * 1024);
-                else copy16_to_lds(a_w + ((size_t)s_safe << w_step_shift), woff[nt][hf], dst + (nt * 2 + hf) * 1024);
+            for (int nt = 0; nt < NT; ++nt) {
+                const uint32_t wu = blockIdx.x * NT + nt, unit = wu < w_units ? wu : w_units - 1;
+                // unit (unit, s_safe) of the matrix: 2 KB, lane i wants chunks i and 64 + i of it
+                const v4i* src = reinterpret_cast<const v4i*>(a_w + ((size_t)unit * (uint32_t)total_steps + s_safe) * kOperandStepBytes) + lane;
+                if constexpr (STREAM) {
+                    wlo[j][nt] = __builtin_nontemporal_load(src);
+                    whi[j][nt] = __builtin_nontemporal_load(src + 64);
+                } else {
+                    wlo[j][nt] = src[0];
+                    whi[j][nt] = src[64];
+                }
             }
+        }
+    } else {
+        const int c_row = lane >> 3, c_slot = lane & 7;
+        uint32_t woff[NT][2];
+#pragma unroll
+        for (int hf = 0; hf < 2; ++hf) {
+            const int r16 = hf * 8 + c_row;
+            const uint32_t chunk = (uint32_t)((c_slot ^ ((r16 >> 1) & 7)) << 4);
+#pragma unroll
+            for (int nt = 0; nt < NT; ++nt) {
+                int wr;
+                if constexpr (GATED) {
+                    // rows 4p .. 4p+3 of a gated tile: gate columns 2p, 2p+1, then up columns 2p, 2p+1, so
+                    // that an MFMA lane (which owns four consecutive tile rows) holds both halves of two
+                    // output columns and all 64 lanes take part in the epilogue
+                    const int g = col0 + nt * 8 + 2 * (r16 >> 2) + (r16 & 1);
+                    wr = ((r16 & 2) ? half_n : 0) + (g < half_n ? g : half_n - 1);
+                } else {
+                    const int r = col0 + nt * 16 + r16;
+                    wr = r < N ? r : N - 1;
+                }
+                // row-major: wr * K + 16 * chunk index; operand order: unit * 16 K + 16 * r16 + 256 * chunk index
+                const uint32_t w_units = (uint32_t)N >> 4, wu = blockIdx.x * NT + nt;
+                const uint32_t unit = wu < w_units ? wu : w_units - 1;
+                const uint32_t row = (uint32_t)wr + ((unit - (uint32_t)wr) & om);
+                woff[nt][hf] = __umul24(row, (uint32_t)K << (om & 4)) + (((uint32_t)r16 << 4) & om) + (chunk << (om & 4));
+            }
+        }
+#pragma unroll
+        for (int j = 0; j < KPW; ++j) {
+            const int s = __builtin_amdgcn_readfirstlane(j * FQ_WAVES + wave);
+            const int s_safe = s < total_steps ? s : total_steps - 1;
+            const uint32_t dst = lds_wave + j * STEP_BYTES;
+#pragma unroll
+            for (int nt = 0; nt < NT; ++nt)
+#pragma unroll
+                for (int hf = 0; hf < 2; ++hf) {
+                    if constexpr (STREAM) copy16_to_lds_nt(a_w + ((size_t)s_safe << w_step_shift), woff[nt][hf], dst + (nt * 2 + hf) * 1024);
+                    else copy16_to_lds(a_w + ((size_t)s_safe << w_step_shift), woff[nt][hf], dst + (nt * 2 + hf) * 1024);
+                }
+        }
     }
 
     // ---- epilogue roles: index arithmetic in the shadow of the row loads (no memory operation and no
@@ -218,32 +277,74 @@ __global__ __launch_bounds__(FQ_THREADS) void gemm_fp8_fusedq_kernel(
         e_live[rr] = e_role[rr] && r_in < ROWS && e_m[rr] < M && e_n[rr] < n_out_total;
         e_n_safe[rr] = e_live[rr] ? e_n[rr] : 0;
     }
+    // which of a lane's 8 handed-over slots exist (slot index < parts), as masks over its four words
+    uint32_t am_mask[4] = {0, 0, 0, 0};
+    if constexpr (AMAX_IN) {
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+            const int e0 = 8 * (lane & 7) + 2 * i;
+            am_mask[i] = (e0 < a_amax_parts ? 0x7FFFu : 0u) | (e0 + 1 < a_amax_parts ? 0x7FFF0000u : 0u);
+        }
+    }
 
-    // ---- 1c. row maxima of this wavefront's K steps (the weight copies stay in flight) -------------
-    // exactly KPW * NT * 2 copies are younger than the row loads
+    // ---- 1c. the row loads have landed (the weight requests stay in flight) ----------------------------
+    // exactly YOUNGER requests are younger than the row loads
+    if constexpr (AMAX_IN) {
+#pragma unroll
+        for (int a = 0; a < AL; ++a) fq_landed<YOUNGER>(am[a]);
+    }
 #pragma unroll
     for (int j = 0; j < KPW; ++j)
 #pragma unroll
         for (int mb = 0; mb < MB; ++mb)
 #pragma unroll
             for (int i = 0; i < 4; ++i)
-                if (4 * i < rows_in_block(mb)) fq_landed<KPW * NT * 2>(xv[j][mb][i]);
+                if (4 * i < rows_in_block(mb)) fq_landed<YOUNGER>(xv[j][mb][i]);
+
+    // ---- row scales: lane l holds the scale of "its" row and the reciprocal ----------------------------
+    // own maxima: lane l <-> row l, every wavefront derives all scales from the table; handed-over maxima:
+    // lanes 8 r .. 8 r + 7 of register set a <-> row 8 a + r
+    constexpr int SETS = AMAX_IN ? AL : 1;
+    float s_row[SETS], r_row[SETS];
+    bool slow_row = false;
+    if constexpr (AMAX_IN) {
 #pragma unroll
-    for (int mb = 0; mb < MB; ++mb)
-#pragma unroll
-        for (int i = 0; i < 4; ++i) {
-            if (4 * i >= rows_in_block(mb)) continue;
+        for (int a = 0; a < AL; ++a) {
+            const uint4 w4 = fq_as_uint4(am[a]);
             uint32_t m2 = 0;
-#pragma unroll
-            for (int j = 0; j < KPW; ++j) m2 = absmax8_pk(fq_as_uint4(xv[j][mb][i]), m2);
+            m2 = absmax8_pk(make_uint4(w4.x & am_mask[0], w4.y & am_mask[1], w4.z & am_mask[2], w4.w & am_mask[3]), m2);
             uint32_t v = absmax_finish(m2), o;
-            o = dpp_move_u32<0xB1>(v);  v = o > v ? o : v;      // the 16 lanes of a row
+            o = dpp_move_u32<0xB1>(v);  v = o > v ? o : v;      // the 8 lanes of a row
             o = dpp_move_u32<0x4E>(v);  v = o > v ? o : v;
             o = dpp_move_u32<0x141>(v); v = o > v ? o : v;
-            o = dpp_move_u32<0x140>(v); v = o > v ? o : v;
-            if (xc == 0) amax_tbl[wave * TBL_ROWS + mb * 16 + 4 * i + xr] = v;
+            s_row[a] = scale_from_amax_bits<QUANT_ACT_DYNAMIC>(v);
+            r_row[a] = biased_reciprocal(s_row[a]);
+            slow_row = slow_row || (__float_as_uint(s_row[a]) & 0x7FFFFFFFu) >= 0x7F800000u;
         }
-    __syncthreads();
+    } else {
+        // the maxima of this wavefront's K steps, one word per row into the table
+#pragma unroll
+        for (int mb = 0; mb < MB; ++mb)
+#pragma unroll
+            for (int i = 0; i < 4; ++i) {
+                if (4 * i >= rows_in_block(mb)) continue;
+                uint32_t m2 = 0;
+#pragma unroll
+                for (int j = 0; j < KPW; ++j) m2 = absmax8_pk(fq_as_uint4(xv[j][mb][i]), m2);
+                uint32_t v = absmax_finish(m2), o;
+                o = dpp_move_u32<0xB1>(v);  v = o > v ? o : v;      // the 16 lanes of a row
+                o = dpp_move_u32<0x4E>(v);  v = o > v ? o : v;
+                o = dpp_move_u32<0x141>(v); v = o > v ? o : v;
+                o = dpp_move_u32<0x140>(v); v = o > v ? o : v;
+                if (xc == 0) amax_tbl[wave * TBL_ROWS + mb * 16 + 4 * i + xr] = v;
+            }
+        __syncthreads();
+    }
+    if constexpr (MAKES_AMAX) {
+        // AmaxOut: the table the epilogue folds its outputs into starts at zero (ordered before the
+        // epilogue by the barrier in front of the reduction)
+        if (a_amax_out.table != nullptr && tid < 64) amax_made[tid] = 0u;
+    }
     // ---- the column operands of the epilogue: requested here, off the path from the row loads to the
     // row maxima, and hidden behind the conversions ------------------------------------------------------
     v4f sw4[ROLE_ROUNDS], su4[ROLE_ROUNDS];
@@ -267,22 +368,38 @@ __global__ __launch_bounds__(FQ_THREADS) void gemm_fp8_fusedq_kernel(
         }
     }
 
-    // every wavefront derives all scales: lane l holds row l's scale and its reciprocal
-    float s_row = 1.0f, r_row = 1.0f;
-    bool slow_row = false;
-    if (lane < ROWS) {
-        uint32_t a = amax_tbl[lane];
+    if constexpr (!AMAX_IN) {
+        s_row[0] = 1.0f; r_row[0] = 1.0f;
+        if (lane < ROWS) {
+            uint32_t a = amax_tbl[lane];
 #pragma unroll
-        for (int w = 1; w < FQ_WAVES; ++w) a = amax_tbl[w * TBL_ROWS + lane] > a ? amax_tbl[w * TBL_ROWS + lane] : a;
-        s_row = scale_from_amax_bits<QUANT_ACT_DYNAMIC>(a);
-        r_row = biased_reciprocal(s_row);
-        slow_row = (__float_as_uint(s_row) & 0x7FFFFFFFu) >= 0x7F800000u;   // an Inf or NaN in the row
+            for (int w = 1; w < FQ_WAVES; ++w) a = amax_tbl[w * TBL_ROWS + lane] > a ? amax_tbl[w * TBL_ROWS + lane] : a;
+            s_row[0] = scale_from_amax_bits<QUANT_ACT_DYNAMIC>(a);
+            r_row[0] = biased_reciprocal(s_row[0]);
+            slow_row = (__float_as_uint(s_row[0]) & 0x7FFFFFFFu) >= 0x7F800000u;   // an Inf or NaN in the row
+        }
     }
     const bool any_slow = __builtin_amdgcn_ballot_w64(slow_row) != 0;       // wavefront-uniform
     if constexpr (TBL_ALIASED) __syncthreads();   // the table lies where codes go next: everyone has read it
+    // value of `v` (s_row or r_row) for row R of the workgroup, R's register set known at compile time
+    auto of_row = [&](const float* v, int set, int r_in_set) -> float {
+        if constexpr (AMAX_IN) return fq_bpermute(v[set], 8 * r_in_set);
+        else return fq_bpermute(v[0], set * 8 + r_in_set);
+    };
     float sa[ROLE_ROUNDS];
 #pragma unroll
-    for (int rr = 0; rr < ROLE_ROUNDS; ++rr) sa[rr] = fq_bpermute(s_row, (e_mb[rr] * 16 + l16) & 63);
+    for (int rr = 0; rr < ROLE_ROUNDS; ++rr) {
+        if constexpr (AMAX_IN) {   // one 16-row block: rows 0 .. 7 in set 0, 8 .. 15 in set 1 (an 8-row block repeats itself)
+            const float lo = of_row(s_row, 0, l16 & 7);
+            sa[rr] = lo;
+            if constexpr (AL > 1) {
+                const float hi = of_row(s_row, 1, l16 & 7);
+                sa[rr] = (l16 & 8) ? hi : lo;
+            }
+        } else {
+            sa[rr] = fq_bpermute(s_row[0], (e_mb[rr] * 16 + l16) & 63);
+        }
+    }
 
     // gated residual: requested now, behind the row loads whose wait counted instructions
     uint2 res2[ROLE_ROUNDS], gate2[ROLE_ROUNDS];
@@ -308,7 +425,8 @@ __global__ __launch_bounds__(FQ_THREADS) void gemm_fp8_fusedq_kernel(
 #pragma unroll
         for (int i = 0; i < 4; ++i) {
             r_of[mb][i] = 1.0f; s_of[mb][i] = 1.0f;
-            if (4 * i < rows_in_block(mb)) r_of[mb][i] = fq_bpermute(r_row, mb * 16 + 4 * i + xr);
+            // row mb * 16 + 4 i + xr: set 2 mb + i / 2, row 4 (i % 2) + xr of the set
+            if (4 * i < rows_in_block(mb)) r_of[mb][i] = of_row(r_row, 2 * mb + (i >> 1), 4 * (i & 1) + xr);
         }
     auto write_codes = [&](auto fast_tag) {
         constexpr bool FAST = decltype(fast_tag)::value;
@@ -325,7 +443,7 @@ __global__ __launch_bounds__(FQ_THREADS) void gemm_fp8_fusedq_kernel(
                 const int at = r16 * 128 + (((xc >> 1) ^ ((r16 >> 1) & 7)) << 4) + (xc & 1) * 8;
 #pragma unroll
                 for (int j = 0; j < KPW; ++j)
-                    *reinterpret_cast<uint2*>(my_stage + j * STEP_BYTES + NT * 2048 + mb * XB + at) =
+                    *reinterpret_cast<uint2*>(my_stage + j * STEP_BYTES + WB + mb * XB + at) =
                         encode8<QUANT_ACT_DYNAMIC>(fq_as_uint4(xv[j][mb][i]), dv);
             }
     };
@@ -336,10 +454,10 @@ __global__ __launch_bounds__(FQ_THREADS) void gemm_fp8_fusedq_kernel(
         for (int mb = 0; mb < MB; ++mb)
 #pragma unroll
             for (int i = 0; i < 4; ++i)
-                if (4 * i < rows_in_block(mb)) s_of[mb][i] = fq_bpermute(s_row, mb * 16 + 4 * i + xr);
+                if (4 * i < rows_in_block(mb)) s_of[mb][i] = of_row(s_row, 2 * mb + (i >> 1), 4 * (i & 1) + xr);
         write_codes(std::false_type{});
     }
-    wait_copies<0>();   // the weights (and everything else this wavefront asked for)
+    if constexpr (!DIRECT) wait_copies<0>();   // the weights (and everything else this wavefront asked for)
 
     // ---- 2. MFMA over this wavefront's K steps -------------------------------------------------------
     v4f acc[NT][MB];
@@ -360,12 +478,14 @@ __global__ __launch_bounds__(FQ_THREADS) void gemm_fp8_fusedq_kernel(
             v8i xb[MB];
 #pragma unroll
             for (int mb = 0; mb < MB; ++mb)
-                xb[mb] = fq_join(*reinterpret_cast<const v4i*>(blk + NT * 2048 + mb * XB + xrd_lo),
-                                 *reinterpret_cast<const v4i*>(blk + NT * 2048 + mb * XB + xrd_hi));
+                xb[mb] = fq_join(*reinterpret_cast<const v4i*>(blk + WB + mb * XB + xrd_lo),
+                                 *reinterpret_cast<const v4i*>(blk + WB + mb * XB + xrd_hi));
 #pragma unroll
             for (int nt = 0; nt < NT; ++nt) {
-                const v8i a = fq_join(*reinterpret_cast<const v4i*>(blk + nt * 2048 + rd_lo),
-                                      *reinterpret_cast<const v4i*>(blk + nt * 2048 + rd_hi));
+                v8i a;
+                if constexpr (DIRECT) a = fq_join(wlo[j][nt], whi[j][nt]);
+                else a = fq_join(*reinterpret_cast<const v4i*>(blk + nt * 2048 + rd_lo),
+                                 *reinterpret_cast<const v4i*>(blk + nt * 2048 + rd_hi));
 #pragma unroll
                 for (int mb = 0; mb < MB; ++mb)
                     acc[nt][mb] = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(a, xb[mb], acc[nt][mb], 0, 0, 0, 0, 0, 0);
@@ -374,6 +494,18 @@ __global__ __launch_bounds__(FQ_THREADS) void gemm_fp8_fusedq_kernel(
     }
     // the partial sums below overwrite this wavefront's own staging: its reads must be done
     asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
+
+    // AmaxOut: |bf16| bit patterns order like the values.  The maximum of a lane's outputs (two packed
+    // pairs), then over the four lane groups that share a token row, then over the workgroup's tiles in LDS.
+    auto fold_amax = [&](uint32_t p0, uint32_t p1, int mb) {
+        const u16x2_t m = __builtin_elementwise_max(__builtin_bit_cast(u16x2_t, p0), __builtin_bit_cast(u16x2_t, p1));
+        uint32_t v = absmax_finish(__builtin_bit_cast(uint32_t, m));
+        const auto h16 = __builtin_amdgcn_permlane16_swap(v, v, false, false);
+        v = h16[0] > h16[1] ? h16[0] : h16[1];
+        const auto h32 = __builtin_amdgcn_permlane32_swap(v, v, false, false);
+        v = h32[0] > h32[1] ? h32[0] : h32[1];
+        if (q == 0) atomicMax(&amax_made[mb * 16 + l16], v);
+    };
 
     // ---- 3. add the eight wavefronts' partial sums, in wavefront order ---------------------------
 #pragma unroll
@@ -403,8 +535,10 @@ __global__ __launch_bounds__(FQ_THREADS) void gemm_fp8_fusedq_kernel(
                 round_bf16_pair(v, up);
                 vf[r] = apply_act<EPI>(v) * up;
             }
-            if (e_live[rr])
-                *reinterpret_cast<uint32_t*>(a_out + (int64_t)e_m[rr] * a_ldo + e_n[rr]) = pack_bf16x2(vf[0], vf[1]);
+            const uint32_t packed = pack_bf16x2(vf[0], vf[1]);
+            if (e_live[rr]) *reinterpret_cast<uint32_t*>(a_out + (int64_t)e_m[rr] * a_ldo + e_n[rr]) = packed;
+            if (a_amax_out.table != nullptr)   // wavefront-uniform
+                fold_amax(e_live[rr] ? (packed & 0x7FFF7FFFu) : 0u, 0u, e_mb[rr]);
         } else {
             float vf[4];
 #pragma unroll
@@ -416,9 +550,19 @@ __global__ __launch_bounds__(FQ_THREADS) void gemm_fp8_fusedq_kernel(
             if constexpr (EPI == EPI_NONE) {
                 if (a_res.residual != nullptr) addcmul4(vf, res2[rr], gate2[rr]);
             }
-            if (e_live[rr])
-                *reinterpret_cast<uint2*>(a_out + (int64_t)e_m[rr] * a_ldo + e_n[rr]) =
-                    make_uint2(pack_bf16x2(vf[0], vf[1]), pack_bf16x2(vf[2], vf[3]));
+            const uint2 packed = make_uint2(pack_bf16x2(vf[0], vf[1]), pack_bf16x2(vf[2], vf[3]));
+            if (e_live[rr]) *reinterpret_cast<uint2*>(a_out + (int64_t)e_m[rr] * a_ldo + e_n[rr]) = packed;
+            if constexpr (MAKES_AMAX) {
+                if (a_amax_out.table != nullptr)
+                    fold_amax(e_live[rr] ? (packed.x & 0x7FFF7FFFu) : 0u, e_live[rr] ? (packed.y & 0x7FFF7FFFu) : 0u, e_mb[rr]);
+            }
+        }
+    }
+    if constexpr (MAKES_AMAX) {
+        if (a_amax_out.table != nullptr) {
+            __syncthreads();
+            if (tid < ROWS && m_base + tid < M)
+                a_amax_out.table[(size_t)(m_base + tid) * kAmaxSlots + blockIdx.x] = (uint16_t)amax_made[tid];
         }
     }
 }
@@ -428,31 +572,45 @@ __global__ __launch_bounds__(FQ_THREADS) void gemm_fp8_fusedq_kernel(
 static int fq_ceil_div(int a, int b) { return (a + b - 1) / b; }
 
 // LDS of a workgroup shape, as the kernel lays it out (the table of row maxima has its own 2 KB unless
-// only the staging fits, see the kernel).
-static constexpr bool fq_fits(int rows, int nt, int kpw) {
+// only the staging fits, see the kernel; none with handed-over maxima; weights that go straight to
+// registers are not staged).
+static constexpr bool fq_fits(int rows, int nt, int kpw, bool direct, bool amax_in, bool act_epilogue) {
     const int mb = (rows + 15) / 16;
     const int xb = rows < 16 ? rows * 128 : 2048;
-    const int stage = kpw * (nt * 2048 + mb * xb), redb = nt * mb * 1024;
-    const int waves = FQ_WAVES * (stage > redb ? stage : redb);
+    const int stage = kpw * ((direct ? 0 : nt * 2048) + mb * xb), redb = nt * mb * 1024;
+    const int waves = FQ_WAVES * (stage > redb ? stage : redb) + (act_epilogue ? 256 : 0);   // + the table of AmaxOut
+    if (amax_in) return rows <= 16 && waves <= 160 * 1024;
     if (waves + FQ_WAVES * 64 * 4 <= 160 * 1024) return true;
     return waves <= 160 * 1024 && FQ_WAVES * (rows < 64 ? rows : 64) * 4 <= xb;
+}
+// Registers: weights in registers are kpw * nt * 8 per lane beside kpw * (rows / 4) * 4 for the rows
+// (256 per lane with two wavefronts per SIMD).
+static constexpr bool fq_regs_ok(int rows, int nt, int kpw, bool direct) {
+    return !direct || kpw * nt * 8 + kpw * ((rows + 3) / 4) * 4 <= 160;
 }
 
 // Shapes that exist as kernels: (rows, nt) below, with kpw = 1, 2 or 4 as K asks.
 // Beyond K = 2048 only the 16 x 16 shape fits the LDS and every workgroup would pull eight times the
 // bf16 rows it has weights for: measured 7.7 us against 6.6 us for quantizer + GEMM at 50 x 1024 x 4096.
-// (The kernels with four K steps per wavefront stay compiled: the plan can be forced for tests.)
+// (The kernels with four K steps per wavefront stay compiled: the plan can be forced for tests, and with
+// handed-over row maxima they are what the down projection of an MLP runs.)
 static const int kFusedMaxK = 2048;
 // Up to 128 token rows the kernel is level with or ahead of quantizer + GEMM as long as a workgroup
 // converts 16 rows or fewer (measured at M = 64 ... 256 on the expert shapes: 32-row workgroups lose).
 static const int kFusedMaxM = 128;
 static const int kFusedShapes[][2] = {{8, 2}, {8, 4}, {8, 5}, {8, 8}, {16, 1}, {16, 2}, {16, 4}, {16, 8}, {32, 2}, {32, 4}};
+// with handed-over maxima (plain epilogue)
+static constexpr bool fq_amax_in_shape(int rows, int nt) {
+    return (rows == 8 && (nt == 2 || nt == 4)) || (rows == 16 && (nt == 1 || nt == 2));
+}
 
-FusedPlan fused_plan(int M, int N, int K, int epilogue, int64_t ldo) {
+FusedPlan fused_plan(int M, int N, int K, int epilogue, int64_t ldo, int weight_layout, bool amax_in) {
     FusedPlan pl = {0, 0, 0, 0, 0};
     if (const char* e = tuning_env("PHYAI_FP8_FUSED")) { if (atoi(e) == 0) return pl; }
     if (M < 1 || M > kFusedMaxM || K % 128 != 0 || K > 4096 || ldo % 4 != 0) return pl;
+    if (amax_in && epilogue != EPI_NONE) return pl;
     const bool gated = epi_is_gated(epilogue);
+    const bool direct = weight_layout != W_ROW_MAJOR;
     const int cols = gated ? N / 2 : N;
     if (cols % 8 != 0) return pl;
     const int per_wave = fq_ceil_div(K / 128, FQ_WAVES);
@@ -466,11 +624,14 @@ FusedPlan fused_plan(int M, int N, int K, int epilogue, int64_t ldo) {
     // and 50 x 1024 x 2048.
     double best = 1e30;
     int forced_rows = 0, forced_nt = 0;
-    if (const char* e = tuning_env("PHYAI_FP8_FUSED_PLAN")) sscanf(e, "%d,%d", &forced_rows, &forced_nt);
-    if (K > kFusedMaxK && !forced_rows) return pl;
+    if (const char* e = tuning_env(amax_in ? "PHYAI_FP8_FUSED_PLAN_AMAX" : "PHYAI_FP8_FUSED_PLAN")) sscanf(e, "%d,%d", &forced_rows, &forced_nt);
+    // beyond K = 2048 the kernel pays only when the row maxima are handed over (no pass over the rows
+    // before the conversions) - or when a test forces it
+    if (K > kFusedMaxK && !forced_rows && !amax_in) return pl;
     for (const auto& sh : kFusedShapes) {
         const int rows = sh[0], nt = sh[1];
-        if (!fq_fits(rows, nt, kpw)) continue;
+        if (!fq_fits(rows, nt, kpw, direct, amax_in, epilogue != EPI_NONE) || !fq_regs_ok(rows, nt, kpw, direct)) continue;
+        if (amax_in && !fq_amax_in_shape(rows, nt)) continue;
         if (forced_rows && (rows != forced_rows || nt != forced_nt)) continue;
         const int tiles = fq_ceil_div(cols, per_tile * nt), msplit = fq_ceil_div(M, rows);
         if (!forced_rows) {
@@ -489,29 +650,48 @@ FusedPlan fused_plan(int M, int N, int K, int epilogue, int64_t ldo) {
     return pl;
 }
 
-template <int ROWS, int NT, int KPW, int EPI>
+template <int ROWS, int NT, int KPW, int EPI, bool DIRECT, bool AMAX_IN>
 static int fq_launch_one(const GemmProblem& g, const FusedPlan& pl, hipStream_t st) {
-    if constexpr (!fq_fits(ROWS, NT, KPW)) {
+    if constexpr (!fq_fits(ROWS, NT, KPW, DIRECT, AMAX_IN, EPI != EPI_NONE) || !fq_regs_ok(ROWS, NT, KPW, DIRECT) ||
+                  (AMAX_IN && (EPI != EPI_NONE || !fq_amax_in_shape(ROWS, NT)))) {
         return -2;
     } else {
+        const AmaxOut made = {EPI != EPI_NONE ? g.amax_out : nullptr};
+        const int m_flags = g.M | (g.weight_layout != W_ROW_MAJOR ? 1 << 28 : 0);
+#define PHYAI_FQ_ARGS g.w, reinterpret_cast<const uint8_t*>(g.x_bf16), g.K, g.N, m_flags, (int)(g.ldx * 2),                     \
+                      reinterpret_cast<const uint8_t*>(g.amax_in), g.amax_parts, g.w_scale, g.bias, g.out, g.ldo, residual_of(g), made
         if (g.stream_weights)
-            hipLaunchKernelGGL((gemm_fp8_fusedq_kernel<ROWS, NT, KPW, EPI, true>), dim3(pl.tiles, pl.msplit), dim3(FQ_THREADS), 0, st,
-                               g.w, reinterpret_cast<const uint8_t*>(g.x_bf16), g.w_scale, g.bias, g.K, g.N, g.M | (g.weight_layout != W_ROW_MAJOR ? 1 << 28 : 0),
-                               (int)(g.ldx * 2), g.out, g.ldo, residual_of(g));
+            hipLaunchKernelGGL((gemm_fp8_fusedq_kernel<ROWS, NT, KPW, EPI, true, DIRECT, AMAX_IN>), dim3(pl.tiles, pl.msplit),
+                               dim3(FQ_THREADS), 0, st, PHYAI_FQ_ARGS);
         else
-            hipLaunchKernelGGL((gemm_fp8_fusedq_kernel<ROWS, NT, KPW, EPI, false>), dim3(pl.tiles, pl.msplit), dim3(FQ_THREADS), 0, st,
-                               g.w, reinterpret_cast<const uint8_t*>(g.x_bf16), g.w_scale, g.bias, g.K, g.N, g.M | (g.weight_layout != W_ROW_MAJOR ? 1 << 28 : 0),
-                               (int)(g.ldx * 2), g.out, g.ldo, residual_of(g));
+            hipLaunchKernelGGL((gemm_fp8_fusedq_kernel<ROWS, NT, KPW, EPI, false, DIRECT, AMAX_IN>), dim3(pl.tiles, pl.msplit),
+                               dim3(FQ_THREADS), 0, st, PHYAI_FQ_ARGS);
+#undef PHYAI_FQ_ARGS
         return 0;
     }
+}
+
+template <int ROWS, int NT, int KPW, int EPI>
+static int fq_launch_variant(const GemmProblem& g, const FusedPlan& pl, hipStream_t st) {
+    const bool direct = g.weight_layout != W_ROW_MAJOR;
+    if (g.amax_in != nullptr) {
+        if constexpr (EPI == EPI_NONE) {
+            return direct ? fq_launch_one<ROWS, NT, KPW, EPI, true, true>(g, pl, st)
+                          : fq_launch_one<ROWS, NT, KPW, EPI, false, true>(g, pl, st);
+        } else {
+            return -2;
+        }
+    }
+    return direct ? fq_launch_one<ROWS, NT, KPW, EPI, true, false>(g, pl, st)
+                  : fq_launch_one<ROWS, NT, KPW, EPI, false, false>(g, pl, st);
 }
 
 template <int ROWS, int NT, int EPI>
 static int fq_launch_kpw(const GemmProblem& g, const FusedPlan& pl, hipStream_t st) {
     switch (pl.kpw) {
-    case 1: return fq_launch_one<ROWS, NT, 1, EPI>(g, pl, st);
-    case 2: return fq_launch_one<ROWS, NT, 2, EPI>(g, pl, st);
-    case 4: return fq_launch_one<ROWS, NT, 4, EPI>(g, pl, st);
+    case 1: return fq_launch_variant<ROWS, NT, 1, EPI>(g, pl, st);
+    case 2: return fq_launch_variant<ROWS, NT, 2, EPI>(g, pl, st);
+    case 4: return fq_launch_variant<ROWS, NT, 4, EPI>(g, pl, st);
     default: return -2;
     }
 }
@@ -534,6 +714,8 @@ static int fq_launch_epi(const GemmProblem& g, const FusedPlan& pl, hipStream_t 
 }
 
 int launch_gemm_fused(const GemmProblem& g, const FusedPlan& pl, hipStream_t st) {
+    if (g.amax_out != nullptr && pl.tiles > kAmaxSlots) return -2;   // one slot per workgroup column
+    if (g.amax_in != nullptr && (g.amax_parts < 1 || g.amax_parts > kAmaxSlots)) return -2;
     switch (g.epilogue) {
     case EPI_NONE: return fq_launch_epi<EPI_NONE>(g, pl, st);
     case EPI_GEGLU_TANH: return fq_launch_epi<EPI_GEGLU_TANH>(g, pl, st);

@@ -362,6 +362,7 @@ struct GemmChoice {
     BigPlan big;
     TileConfig tc;
     size_t need;   // workspace bytes (header + split-K partial sums), 0 if the kernel uses none
+    bool takes_amax;   // FUSED: the plan is the one for handed-over row maxima
 };
 
 // Kernel choice (measured on the expert and prefill shapes, M = 50 .. 13056):
@@ -377,10 +378,15 @@ struct GemmChoice {
 // tile kernel's epilogue needs.
 // have_x: the bf16 activations are at hand (whole-linear entry points), so a kernel that quantizes
 // its own rows may serve the call.
-static GemmChoice choose_gemm(int M, int N, int K, int epilogue, int64_t ldo, bool vec_ok, bool out16, bool have_x) {
+static GemmChoice choose_gemm(int M, int N, int K, int epilogue, int64_t ldo, bool vec_ok, bool out16, bool have_x,
+                              int layout = W_ROW_MAJOR, bool amax_in = false) {
     GemmChoice c = {};
     if (have_x && vec_ok) {
-        c.fq = fused_plan(M, N, K, epilogue, ldo);
+        if (amax_in) {
+            c.fq = fused_plan(M, N, K, epilogue, ldo, layout, true);
+            if (c.fq.rows) { c.kind = GemmChoice::FUSED; c.need = 0; c.takes_amax = true; return c; }
+        }
+        c.fq = fused_plan(M, N, K, epilogue, ldo, layout, false);
         if (c.fq.rows) { c.kind = GemmChoice::FUSED; c.need = 0; return c; }
     }
     const bool skinny_ok = vec_ok && skinny_applicable(M, N, K, epilogue, ldo);
@@ -416,7 +422,21 @@ static GemmChoice choose_gemm(const GemmProblem& g) {
     const bool have_x = g.x_bf16 != nullptr && (reinterpret_cast<uintptr_t>(g.x_bf16) & 15) == 0 && g.ldx % 8 == 0 &&
                         (int64_t)g.M * g.ldx * 2 < ((int64_t)1 << 32) && (int64_t)g.N * g.K < ((int64_t)1 << 32) &&
                         g.K < (1 << 24) && g.N < (1 << 24) && !g.x_scale_is_scalar;
-    return choose_gemm(g.M, g.N, g.K, g.epilogue, g.ldo, vec_ok, out16, have_x);
+    return choose_gemm(g.M, g.N, g.K, g.epilogue, g.ldo, vec_ok, out16, have_x, g.weight_layout,
+                       g.amax_in != nullptr && g.amax_parts >= 1 && g.amax_parts <= kRowAmaxSlots &&
+                           (reinterpret_cast<uintptr_t>(g.amax_in) & 15) == 0);
+}
+
+int gemm_row_maxima_slots(const GemmProblem& g) {
+    if (g.M == 0 || g.N == 0 || g.epilogue == EPI_NONE) return 0;
+    const GemmChoice c = choose_gemm(g);
+    return (c.kind == GemmChoice::FUSED && c.fq.tiles <= kRowAmaxSlots) ? c.fq.tiles : 0;
+}
+
+bool gemm_takes_row_maxima(const GemmProblem& g) {
+    if (g.M == 0 || g.N == 0) return false;
+    const GemmChoice c = choose_gemm(g);
+    return c.kind == GemmChoice::FUSED && c.takes_amax;
 }
 
 bool gemm_quantizes_itself(const GemmProblem& g) {
@@ -454,11 +474,40 @@ int describe_linear_plan(int M, int N, int K, int epilogue, char* buf, size_t n)
     return len + describe_gemm_plan(M, N, K, epilogue, buf + len, n - len);
 }
 
+int describe_mlp_plan(int M, int H, int I, int O, int epilogue, char* buf, size_t n) {
+    const int n1 = epi_is_gated(epilogue) ? 2 * I : I;
+    const GemmChoice a = choose_gemm(M, n1, H, epilogue, I, true, I % 8 == 0, true);
+    bool handed = false;
+    if (a.kind == GemmChoice::FUSED && a.fq.tiles <= kRowAmaxSlots) {
+        const GemmChoice b = choose_gemm(M, O, I, EPI_NONE, O, true, O % 8 == 0, true, W_ROW_MAJOR, true);
+        handed = b.kind == GemmChoice::FUSED && b.takes_amax;
+    }
+    int len = handed ? snprintf(buf, n, "row maxima handed over: ") : 0;
+    if (len < 0 || (size_t)len >= n) return len;
+    len += describe_linear_plan(M, n1, H, epilogue, buf + len, n - len);
+    if ((size_t)len >= n) return len;
+    len += snprintf(buf + len, n - len, " | ");
+    if ((size_t)len >= n) return len;
+    if (handed) {
+        const GemmChoice b = choose_gemm(M, O, I, EPI_NONE, O, true, O % 8 == 0, true, W_ROW_MAJOR, true);
+        return len + snprintf(buf + len, n - len, "one launch: small-m rows=%d nt=%d kpw=%d grid=%dx%d", b.fq.rows, b.fq.nt,
+                              b.fq.kpw, b.fq.tiles, b.fq.msplit);
+    }
+    return len + describe_linear_plan(M, O, I, EPI_NONE, buf + len, n - len);
+}
+
 int launch_gemm(const GemmProblem& g, hipStream_t st) {
     if (g.M == 0 || g.N == 0) return 0;
     const GemmChoice ch = choose_gemm(g);
     if (ch.need > 0 && (g.workspace == nullptr || g.workspace_bytes < ch.need)) return -3;
-    if (ch.kind == GemmChoice::FUSED) return launch_gemm_fused(g, ch.fq, st);
+    if (ch.kind == GemmChoice::FUSED) {
+        if (g.amax_in != nullptr && !ch.takes_amax) {   // the plan finds the row maxima itself
+            GemmProblem own = g;
+            own.amax_in = nullptr;
+            return launch_gemm_fused(own, ch.fq, st);
+        }
+        return launch_gemm_fused(g, ch.fq, st);
+    }
     if (ch.kind == GemmChoice::SKINNY) return launch_gemm_skinny(g, ch.sk, st);
     if (ch.kind == GemmChoice::BIG) return launch_gemm_big(g, ch.big, st);
     const TileConfig& c = ch.tc;

@@ -69,6 +69,14 @@ struct GemmProblem {
     // Layout of w (weight_layout.h): 0 row-major [N, K]; 1 MFMA operand order; 2 operand order of a fused
     // gate | up matrix (gated epilogues only).
     int weight_layout;
+    // Row maxima handed from the producer of the activations to their consumer (the gate | up projection
+    // of an MLP to its down projection; the one-launch small-M kernel only): amax_out, when set on a gated
+    // launch, receives per token row and workgroup column the |bf16| maximum of the outputs
+    // (table [M][64] of 16-bit patterns); amax_in / amax_parts give the consumer the table and the
+    // number of slots per row that the producer wrote, and replace its own pass over the rows.
+    uint16_t* amax_out;
+    const uint16_t* amax_in;
+    int amax_parts;
 };
 
 // What the kernels need of the above, by value.
@@ -95,6 +103,12 @@ int launch_gemm(const GemmProblem& p, hipStream_t st);
 // True when launch_gemm would serve this problem (x_bf16 set) with the kernel that quantizes its own
 // rows: the caller then skips the quantizer launch.
 bool gemm_quantizes_itself(const GemmProblem& p);
+// Row maxima handed from one linear to the next (GemmProblem::amax_out / amax_in).  Slots per token row
+// that launch_gemm would write for this producer (x_bf16 set, an activation epilogue), 0 when the kernel
+// that serves it cannot; whether launch_gemm would serve this consumer (amax_in, amax_parts set) with
+// the kernel that takes them.
+int gemm_row_maxima_slots(const GemmProblem& p);
+bool gemm_takes_row_maxima(const GemmProblem& p);
 // Text form of the whole-linear choice for aligned operands and dense activations / output.
 int describe_linear_plan(int M, int N, int K, int epilogue, char* buf, size_t n);
 
@@ -120,7 +134,8 @@ struct FusedPlan {
     int tiles;   // workgroups along N
     int msplit;  // workgroups along M
 };
-FusedPlan fused_plan(int M, int N, int K, int epilogue, int64_t ldo);
+FusedPlan fused_plan(int M, int N, int K, int epilogue, int64_t ldo, int weight_layout = 0, bool amax_in = false);
+constexpr int kRowAmaxSlots = 64;   // slots per token row of a table of handed-over row maxima
 int launch_gemm_fused(const GemmProblem& p, const FusedPlan& pl, hipStream_t st);
 
 // Pipelined tile kernel for large M (gemm_big.hip), 256 x 256 or 128 x 128 tiles; the small
@@ -136,6 +151,8 @@ BigPlan big_plan(int M, int N, int K, int epilogue);
 size_t big_partial_bytes(int M, int N, int epilogue, const BigPlan& pl);
 int launch_gemm_big(const GemmProblem& p, const BigPlan& pl, hipStream_t st);
 
+// Text form of what phyai_fp8_mlp launches for aligned, row-major operands.
+int describe_mlp_plan(int M, int H, int I, int O, int epilogue, char* buf, size_t n);
 // Text form of launch_gemm's choice for aligned operands and a dense output; returns its length.
 int describe_gemm_plan(int M, int N, int K, int epilogue, char* buf, size_t n);
 

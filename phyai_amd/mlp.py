@@ -99,9 +99,33 @@ class DenseMLP(nn.Module):
             self.fc2 = RowParallelLinear(intermediate_size, hidden_size, input_is_parallel=True,
                                          reduce_results=True, spec=spec_out, prefix=child("fc2"), **common)
 
-    def forward(self, x: torch.Tensor) -> torch.Tensor:
+    def _one_call(self, first, second, x) -> bool:
+        """Both projections are per-channel fp8 layers that the HIP kernel serves on bf16 input: the whole
+        MLP is then one library call (``ops.fp8_mlp``), which lets the first kernel hand its output's row
+        maxima to the second."""
+        return (self.fuse_activation and isinstance(x, torch.Tensor) and x.is_cuda and x.dtype == torch.bfloat16
+                and getattr(first.spec, "spec_id", "") == "fp8_per_channel"
+                and getattr(second.spec, "spec_id", "") == "fp8_per_channel"
+                and not first.skip_bias_add and not second.skip_bias_add
+                and first.supports_fused_epilogue(x) and second.supports_fused_epilogue(x))
+
+    def forward(self, x: torch.Tensor, *, residual: torch.Tensor | None = None,
+                gate: torch.Tensor | None = None) -> torch.Tensor:
+        """``residual`` / ``gate``: ``torch.addcmul(residual, mlp(x), gate)`` in the second GEMM's epilogue
+        (the decoder layer's gated residual, reference ``models/pi05/modeling_pi05.py:835``)."""
         first = self.gate_up_proj if self.gated else self.fc1
         second = self.down_proj if self.gated else self.fc2
+        if self._one_call(first, second, x):
+            from phyai_amd import ops
+
+            return ops.fp8_mlp(x, first.weight, first.weight_scale, first.bias, second.weight, second.weight_scale,
+                               second.bias, epilogue=self._epilogue, residual=residual, gate=gate,
+                               stream_weights1=bool(getattr(first, "stream_weights", False)),
+                               stream_weights2=bool(getattr(second, "stream_weights", False)),
+                               weight1_layout=getattr(first, "weight_layout", None),
+                               weight2_layout=getattr(second, "weight_layout", None))
+        if residual is not None or gate is not None:
+            return torch.addcmul(residual, self.forward(x), gate)
         if self.fuse_activation and first.supports_fused_epilogue(x):
             h = first.forward_fused(x, self._epilogue)
         elif getattr(first, "weight_layout", None) == "operand_gated":

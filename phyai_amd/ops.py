@@ -548,6 +548,60 @@ def fp8_linear(x: torch.Tensor, weight: torch.Tensor, weight_scale: torch.Tensor
     return out
 
 
+def describe_mlp_plan(M: int, H: int, I: int, O: int, epilogue) -> str:
+    """What :func:`fp8_mlp` launches for this shape (row-major weights; host only)."""
+    import ctypes
+
+    buf = ctypes.create_string_buffer(256)
+    rc = _lib.load().phyai_fp8_describe_mlp_plan(M, H, I, O, _epi("describe_mlp_plan", epilogue), buf, len(buf))
+    if rc < 0:
+        raise _err("describe_mlp_plan", _lib.load().phyai_fp8_last_error().decode())
+    return buf.value.decode()
+
+
+def fp8_mlp(x: torch.Tensor, weight1: torch.Tensor, weight1_scale: torch.Tensor, bias1: torch.Tensor | None,
+            weight2: torch.Tensor, weight2_scale: torch.Tensor, bias2: torch.Tensor | None, *, epilogue,
+            out: torch.Tensor | None = None, residual: torch.Tensor | None = None, gate: torch.Tensor | None = None,
+            stream_weights1: bool = False, stream_weights2: bool = False, weight1_layout: str | None = None,
+            weight2_layout: str | None = None) -> torch.Tensor:
+    """Both projections of an MLP in one call: ``linear2(act(linear1(x)))`` with ``epilogue`` the
+    activation of the first (gated: ``weight1`` is the fused gate | up matrix ``[2 I, H]``), optionally
+    ``torch.addcmul(residual, ., gate)`` behind the second.  The bits of :func:`fp8_linear` with that
+    epilogue followed by :func:`fp8_linear` on its output; the intermediate tensor lives in the workspace.
+    For small token counts the first kernel hands the row maxima of its output to the second, which then
+    quantizes those rows without first passing over them (see :func:`describe_mlp_plan`).
+
+    Replaces ``DenseMLP.forward`` of the reference (``layers/mlp/dense_mlp.py:256-265``)."""
+    op = "fp8_mlp"
+    epi = _epi(op, epilogue)
+    if epi == EPI_NONE:
+        raise _err(op, "epilogue must be the first projection's activation")
+    x2 = _as_rows(op, x, "x", torch.bfloat16)
+    M, H = x2.shape
+    N1, _ = _check_weight(op, weight1, weight1_scale, H)
+    if epi in _GATED and N1 % 32 != 0:
+        raise _err(op, f"gated epilogue needs N % 32 == 0, got {N1}")
+    I = N1 // 2 if epi in _GATED else N1
+    O, _ = _check_weight(op, weight2, weight2_scale, I)
+    b1, b2 = _check_bias(op, bias1, N1), _check_bias(op, bias2, O)
+    f1 = _layout_flag(op, weight1_layout, epi) | (FLAG_STREAM_WEIGHTS if stream_weights1 else 0)
+    f2 = _layout_flag(op, weight2_layout, EPI_NONE) | (FLAG_STREAM_WEIGHTS if stream_weights2 else 0)
+    r2, g2 = _check_addcmul(op, residual, gate, tuple(x.shape[:-1]), M, O, EPI_NONE, x.device)
+    out = _out_for(op, tuple(x.shape[:-1]), O, out, x.device)
+    if M == 0:
+        return out
+    lib = _lib.load()
+    ws = reserve_workspace(int(lib.phyai_fp8_mlp_workspace_bytes(M, H, I, O, epi)), x.device)
+    rc = lib.phyai_fp8_mlp(
+        x2.data_ptr(), x2.stride(0) if M > 1 else H, weight1.data_ptr(), weight1_scale.data_ptr(), b1, f1,
+        weight2.data_ptr(), weight2_scale.data_ptr(), b2, f2,
+        r2.data_ptr() if r2 is not None else None, (r2.stride(0) if M > 1 else O) if r2 is not None else 0,
+        g2.data_ptr() if g2 is not None else None, (g2.stride(0) if g2.shape[0] > 1 else O) if g2 is not None else 0,
+        g2.shape[0] if g2 is not None else 0, out.data_ptr(), O, M, H, I, O, epi, ws.data_ptr(), ws.numel(), _stream_ptr())
+    _lib.check(rc, op)
+    return out
+
+
 def debug_cast_e4m3(v: torch.Tensor) -> torch.Tensor:
     """Device fp32 -> e4m3fn cast used by the quantizers, exposed for exhaustive tests."""
     if not (v.is_cuda and v.dtype == torch.float32 and v.is_contiguous()):

@@ -68,6 +68,11 @@ def test_every_workgroup_shape_equals_two_launches_bit_for_bit(dev, monkeypatch,
     w = seeded((N, K), seed=N + 7 * K, scale=0.02).to(dev)
     b = seeded((N,), seed=N, scale=0.01).to(dev)
     wq, ws = ops.fp8_weight_quant(w)
+    # the same weights in MFMA operand order: the kernel then loads them straight into registers
+    gated = epi in ("geglu_tanh", "geglu_erf", "swiglu")
+    operand = K % 128 == 0 and N % (32 if gated else 16) == 0
+    wo = ops.fp8_weight_to_operand_order(wq, gated=gated) if operand else None
+    layout = "operand_gated" if gated else "operand"
     res = seeded((M, N), seed=5).to(dev)
     gate = seeded((1, N), seed=6, scale=0.5).to(dev)
 
@@ -93,9 +98,15 @@ def test_every_workgroup_shape_equals_two_launches_bit_for_bit(dev, monkeypatch,
                 assert _same(got, want[bias is None]), \
                     f"{desc}, bias={bias is not None}, streamed={streamed}: " \
                     f"{int((_bits(got) != _bits(want[bias is None])).sum())} outputs differ"
+                if operand:
+                    got = ops.fp8_linear(xd, wo, ws, bias, epilogue=epi, stream_weights=streamed, weight_layout=layout)
+                    assert _same(got, want[bias is None]), f"{desc}, weights in operand order, bias={bias is not None}, streamed={streamed}"
         if want_res is not None:
             got = ops.fp8_linear(xd, wq, ws, b, residual=res, gate=gate)
             assert _same(got, want_res), f"{desc}: gated residual differs"
+            if operand:
+                got = ops.fp8_linear(xd, wo, ws, b, residual=res, gate=gate, weight_layout=layout)
+                assert _same(got, want_res), f"{desc}: gated residual with weights in operand order differs"
             buf = res.clone()                                   # writing over the residual
             ops.fp8_linear(xd, wq, ws, b, residual=buf, gate=gate, out=buf)
             assert _same(buf, want_res), f"{desc}: gated residual written in place differs"
