@@ -10,15 +10,24 @@ layer with its own weight tensors (311 MB of fp8 weights per denoise step), and
 that graph (what the engine launches per action chunk); `value` is the p50 time
 of one denoise step (replay time / 10) in microseconds.
 
+How the linears are called is what a model built on this library does (phyai_amd.linear layers with
+Fp8Spec(operand_order=True), phyai_amd.mlp.DenseMLP): weights re-laid in MFMA operand order once after
+loading, qkv and o as one phyai_fp8_linear each, gate_up + GeGLU and down as one phyai_fp8_mlp call (down
+consumes gate_up's output, as in the model; its own random input tensor is used only by the variants that
+run the four linears separately).  --row-major / --separate-linears switch either back for A/B runs.
+
 Printed JSON (one line):
-  value / ms_per_step  whole-path numbers (quantizer + GEMM + epilogue, graph replay)
-  roofline             the GEMM kernel alone: algorithmic bytes of one layer's four
-                       linears / their measured average launch durations (HIP events
-                       around graph replays that contain only those GEMM launches,
-                       distinct weights per launch so they stream from HBM)
+  value / ms_per_step  whole-path numbers (quantization + GEMM + epilogue, graph replay)
+  roofline             the kernels that read the weights: algorithmic bytes of one layer's four
+                       linears / the measured duration of the launches that read their weights (the
+                       whole linear where it is one kernel that quantizes its own rows, else the GEMM
+                       behind the quantizer), HIP events around replays of a graph that holds only
+                       those launches and walks all 18 layers' distinct weights
+  roofline_prefill     the MFMA-bound regime (M = 816), per shape and for the layer
+  launch_floor         what the kernel nodes of a layer cost before any byte moves
   cpu_baseline         torch CPU dequantize + matmul form of the same layer set on
                        this box's host cores (a reported baseline, not the target)
-  extra                prefix-prefill set (M = 816) in TFLOP/s against dense fp8 peak
+  extra                neighbouring measurements (prefill layer, decoder layer with norms, ...)
 
 Inputs are resident in HBM before the timed region starts.
 """
@@ -74,10 +83,16 @@ def algorithmic_bytes(M: int, N: int, K: int, epilogue, bias: bool = False) -> i
     return 2 * M * K + N * K + 4 * N + (2 * N if bias else 0) + 2 * M * n_out
 
 
+# How the benchmark calls the library (switched by --row-major / --separate-linears for A/B runs)
+OPTS = {"operand": True, "mlp": True}
+
+
 def make_layers(dev, shapes, M, n_layers, seed0=0):
     """Seeded synthetic tensors, generated on the CPU and copied to the device so that
     the CPU baseline sees the same bits.  Weights are quantized on the device by the
-    library's own weight quantizer (bit-exact with the oracle's)."""
+    library's own weight quantizer (bit-exact with the oracle's) and, as Fp8Spec(operand_order=True)
+    does in process_after_loading, re-laid in MFMA operand order (`wo`; `w` stays row-major for the
+    torch and CPU paths)."""
     from phyai_amd import ops
 
     layers = []
@@ -94,18 +109,59 @@ def make_layers(dev, shapes, M, n_layers, seed0=0):
             layer[name] = dict(w=wq, ws=ws, x=x.to(dev), epi=epi, N=N, K=K,
                                out=torch.empty(M, n_out, dtype=torch.bfloat16, device=dev),
                                w_bf16_cpu=w if li == 0 else None, x_cpu=x if li == 0 else None)
+            if K % 128 == 0:
+                layer[name]["wo"] = ops.fp8_weight_to_operand_order(wq, gated=bool(epi))
+                layer[name]["lay"] = ("operand_gated" if epi in ("geglu_tanh", "geglu_erf", "swiglu") else "operand")
         layers.append(layer)
     return layers
 
 
-def run_layers(layers, shapes):
+def weight_of(t):
+    """(weight tensor, weight_layout) the benchmark passes for this linear."""
+    if OPTS["operand"] and "wo" in t:
+        return t["wo"], t["lay"]
+    return t["w"], None
+
+
+def linear(t, x=None, out=None):
     from phyai_amd import ops
 
+    w, lay = weight_of(t)
+    return ops.fp8_linear(t["x"] if x is None else x, w, t["ws"], None, epilogue=t["epi"],
+                          out=t["out"] if out is None else out, stream_weights=t.get("stream", False), weight_layout=lay)
+
+
+def is_mlp_pair(a, b) -> bool:
+    """gate_up (an activation epilogue) followed by the projection that consumes its output."""
+    return bool(a["epi"]) and b["epi"] is None and b["K"] == a["out"].shape[-1] and a["out"].shape[0] == b["out"].shape[0]
+
+
+def mlp(a, b):
+    from phyai_amd import ops
+
+    (w1, l1), (w2, l2) = weight_of(a), weight_of(b)
+    return ops.fp8_mlp(a["x"], w1, a["ws"], None, w2, b["ws"], None, epilogue=a["epi"], out=b["out"],
+                       stream_weights1=a.get("stream", False), stream_weights2=b.get("stream", False),
+                       weight1_layout=l1, weight2_layout=l2)
+
+
+def run_layer(layer, shapes):
+    """One layer's linears as a model calls them: an MLP's two projections as one phyai_fp8_mlp call."""
+    names = [name for name, _, _, _ in shapes]
+    i = 0
+    while i < len(names):
+        t = layer[names[i]]
+        if OPTS["mlp"] and i + 1 < len(names) and is_mlp_pair(t, layer[names[i + 1]]):
+            mlp(t, layer[names[i + 1]])
+            i += 2
+        else:
+            linear(t)
+            i += 1
+
+
+def run_layers(layers, shapes):
     for layer in layers:
-        for name, _, _, _ in shapes:
-            t = layer[name]
-            ops.fp8_linear(t["x"], t["w"], t["ws"], None, epilogue=t["epi"], out=t["out"],
-                           stream_weights=t.get("stream", False))
+        run_layer(layer, shapes)
 
 
 def torch_reference_times(dev, layers, shapes, denoise_steps, steps, warmup):
@@ -392,6 +448,22 @@ def ops_plan(M, N, K, epi):
     return ops.describe_linear_plan(M, N, K, epi)
 
 
+def layer_plans(layer, shapes, M):
+    """What each linear of a layer is launched as, by name (the second projection of an MLP that takes the
+    first's row maxima: the part of phyai_fp8_describe_mlp_plan behind the bar)."""
+    from phyai_amd import ops
+
+    names = [name for name, _, _, _ in shapes]
+    plans = {name: ops_plan(M, N, K, epi) for name, N, K, epi in shapes}
+    for i in range(len(names) - 1):
+        a, b = layer[names[i]], layer[names[i + 1]]
+        if mlp_hands_over(a, b):
+            first, second = ops.describe_mlp_plan(M, a["K"], b["K"], b["N"], a["epi"]).split(": ", 1)[1].split(" | ")
+            plans[names[i]] = first + " (leaves its output's row maxima)"
+            plans[names[i + 1]] = second + " (takes them)"
+    return plans
+
+
 def time_replays(graph, n, warmup):
     """HIP events around each replay, on the stream the replays are launched on."""
     for _ in range(warmup):
@@ -421,9 +493,36 @@ def weight_kernel_launch(xq, xs, t):
     from phyai_amd import ops
 
     if one_launch(t["x"].shape[0], t["N"], t["K"], t["epi"]):
-        ops.fp8_linear(t["x"], t["w"], t["ws"], None, epilogue=t["epi"], out=t["out"], stream_weights=t.get("stream", False))
+        linear(t)
     else:
-        ops.fp8_gemm(xq, xs, t["w"], t["ws"], None, epilogue=t["epi"], out=t["out"], stream_weights=t.get("stream", False))
+        w, lay = weight_of(t)
+        ops.fp8_gemm(xq, xs, w, t["ws"], None, epilogue=t["epi"], out=t["out"], stream_weights=t.get("stream", False),
+                     weight_layout=lay)
+
+
+def mlp_hands_over(a, b) -> bool:
+    """Do both projections of this MLP run as one kernel each, the second on the first's row maxima?"""
+    from phyai_amd import ops
+
+    M = a["x"].shape[0]
+    return OPTS["mlp"] and is_mlp_pair(a, b) and \
+        ops.describe_mlp_plan(M, a["K"], b["K"], b["N"], a["epi"]).startswith("row maxima handed over")
+
+
+def layer_weight_kernels(layer, shapes, codes):
+    """The launches of one layer that read its weights, as the benchmark runs them: an MLP whose second
+    projection takes the first's row maxima is one call of two kernels; a linear that is one kernel is that
+    kernel; any other is the GEMM on the codes the quantizer left (`codes[name]`)."""
+    names = [name for name, _, _, _ in shapes]
+    i = 0
+    while i < len(names):
+        t = layer[names[i]]
+        if i + 1 < len(names) and mlp_hands_over(t, layer[names[i + 1]]):
+            mlp(t, layer[names[i + 1]])
+            i += 2
+        else:
+            weight_kernel_launch(*codes[names[i]], t)
+            i += 1
 
 
 def gemm_only_times(dev, layers, shapes, M, reps=8, iters=30):
@@ -450,6 +549,22 @@ def gemm_only_times(dev, layers, shapes, M, reps=8, iters=30):
         ts, _ = time_replays(g, iters, 3)
         launches = reps * len(pre)
         out[name] = statistics.median(ts) * 1e3 / launches  # us per launch
+    # an MLP whose second projection takes the first's row maxima: the pair is timed as the one call it is,
+    # and the second projection's kernel is that minus the first projection alone
+    names = [name for name, _, _, _ in shapes]
+    for i in range(len(names) - 1):
+        if mlp_hands_over(layers[0][names[i]], layers[0][names[i + 1]]):
+            def fn(a=names[i], b=names[i + 1]):
+                for _ in range(reps):
+                    for layer in layers:
+                        mlp(layer[a], layer[b])
+
+            g = HipGraph()
+            g.capture(fn, {})
+            ts, _ = time_replays(g, iters, 3)
+            pair = statistics.median(ts) * 1e3 / (reps * len(layers))
+            out[names[i] + "+" + names[i + 1]] = pair
+            out[names[i + 1]] = pair - out[names[i]]
     return out
 
 
@@ -463,21 +578,19 @@ def gemm_only_layer_time(dev, layers, shapes, reps=8, iters=30, ready_codes=Fals
     from phyai_amd import ops
     from phyai_amd.runtime import HipGraph
 
-    pre = []
-    for layer in layers:
-        for name, _, _, _ in shapes:
-            t = layer[name]
-            xq, xs = ops.fp8_quant_rowwise(t["x"])
-            pre.append((xq, xs, t))
+    pre = [{name: ops.fp8_quant_rowwise(layer[name]["x"]) for name, _, _, _ in shapes} for layer in layers]
 
     def fn():
         for _ in range(reps):
-            for xq, xs, t in pre:
+            for layer, codes in zip(layers, pre):
                 if ready_codes:
-                    ops.fp8_gemm(xq, xs, t["w"], t["ws"], None, epilogue=t["epi"], out=t["out"],
-                                 stream_weights=t.get("stream", False))
+                    for name, _, _, _ in shapes:
+                        t = layer[name]
+                        w, lay = weight_of(t)
+                        ops.fp8_gemm(*codes[name], w, t["ws"], None, epilogue=t["epi"], out=t["out"],
+                                     stream_weights=t.get("stream", False), weight_layout=lay)
                 else:
-                    weight_kernel_launch(xq, xs, t)
+                    layer_weight_kernels(layer, shapes, codes)
 
     g = HipGraph()
     g.capture(fn, {})
@@ -564,11 +677,18 @@ def probe(dev, layers, M, shapes=EXPERT_SET):
     read, 64 MiB written) to calibrate the counters."""
     from phyai_amd import ops
 
-    for name, N, K, epi in shapes:
+    names = [name for name, _, _, _ in shapes]
+    for i, name in enumerate(names):
         pre = [(ops.fp8_quant_rowwise(layer[name]["x"]), layer[name]) for layer in layers]
         torch.cuda.synchronize()
-        for (xq, xs), t in pre:
-            weight_kernel_launch(xq, xs, t)
+        if i > 0 and mlp_hands_over(layers[0][names[i - 1]], layers[0][name]):
+            # the second projection of an MLP exists only behind the first: the pair, one call per layer
+            # (the first projection's kernel appears a second time in the trace)
+            for layer in layers:
+                mlp(layer[names[i - 1]], layer[name])
+        else:
+            for (xq, xs), t in pre:
+                weight_kernel_launch(xq, xs, t)
         torch.cuda.synchronize()
     src = torch.empty(64 << 20, dtype=torch.uint8, device=dev).fill_(1)
     dst = torch.empty_like(src)
@@ -654,6 +774,21 @@ def cpu_baseline(layers, shapes, M, n_layers):
                           "layer_quantizer_gemm": _cpu_time(layer_full, budget),
                           "layer_gemm_only": _cpu_time(layer_gemm_only, budget),
                           "config1_linear": _cpu_time(config1, budget / 4)}
+        # benchmark configuration 3: one layer of the prefix-prefill set (M = 816, 180 GFLOP), all threads,
+        # a handful of passes (own seeded tensors: the GPU run's prefill layers are not kept on the host)
+        torch.set_num_threads(all_threads)
+        pitems = []
+        for i, (name, N, K, epi) in enumerate(PREFILL_SET):
+            gp = torch.Generator().manual_seed(20_000 + i)
+            wq, ws = ref.weight_quant((torch.randn(N, K, generator=gp) * 0.02).to(torch.bfloat16))
+            pitems.append((torch.randn(816, K, generator=gp).to(torch.bfloat16), wq, ws, {None: 0, "geglu_tanh": 1}[epi]))
+
+        def prefill_layer():
+            for x, wq, ws, epi in pitems:
+                ref.linear(x, wq, ws, None, epi)
+
+        out["all_threads"]["prefill_layer_quantizer_gemm_M816"] = _cpu_time(prefill_layer, 6.0, min_iters=5, warmup=1)
+        del pitems
     finally:
         torch.set_num_threads(all_threads)
     model, phys = cpu_info()
@@ -663,7 +798,8 @@ def cpu_baseline(layers, shapes, M, n_layers):
             "sample": f"torch CPU dequantize+matmul incl. quantizer and GeGLU on 1 of {n_layers} layers (4 linears, "
                       f"M={M}), p50 of {full['iters']} passes at {all_threads} threads, scaled x{n_layers}; `variants` "
                       "holds the per-layer times (us) of GEMM only and quantizer+GEMM at all threads and at one "
-                      "thread, and benchmark configuration 1",
+                      "thread, benchmark configuration 1, and one layer of the prefix-prefill set (configuration 3, "
+                      "M = 816, at least 5 passes at all threads)",
             "variants": out}
 
 
@@ -688,7 +824,13 @@ def main() -> int:
                     help="the same for the prefill GEMM shapes (M = 816, 4 weight sets), for the MFMA / LDS counters")
     ap.add_argument("--probe-m", type=int, default=816,
                     help="token rows of --probe-prefill (816 x batch for the batched-serving shapes)")
+    ap.add_argument("--row-major", action="store_true",
+                    help="A/B: pass the weights row-major [N, K] instead of in MFMA operand order")
+    ap.add_argument("--separate-linears", action="store_true",
+                    help="A/B: gate_up and down as two phyai_fp8_linear calls instead of one phyai_fp8_mlp call")
     args = ap.parse_args()
+    OPTS["operand"] = not args.row_major
+    OPTS["mlp"] = not args.separate_linears
     if args.gpus != 1 or int(os.environ.get("WORLD_SIZE", "1")) != 1:
         print("bench.py: this path is built and measured on ONE GPU (TP=1, no collectives); "
               "run with --gpus 1", file=sys.stderr)
@@ -743,20 +885,23 @@ def main() -> int:
     roofline = {
         "bound": "hbm", "achieved": round(achieved, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
         "frac": round(achieved / HBM_PEAK_GBS, 4), "traffic": profiled_layer_traffic(),
-        "kernel": " + ".join(sorted({"gemm_fp8_fusedq_kernel" if one_launch(M, N, K, epi) else "gemm_fp8_skinny_kernel"
-                                     for _, N, K, epi in EXPERT_SET})) + " (M=50, four expert shapes)",
+        "kernel": "gemm_fp8_fusedq_kernel (M=50, four expert shapes)",   # completed below from the plans
         "bytes_per_layer": layer_bytes, "us_per_layer": round(layer_us, 3),
         "note": "achieved = bytes_per_layer / us_per_layer, the four weight-reading launches of a layer (the whole "
                 "linear where it is one kernel that quantizes its own rows, else the GEMM behind the quantizer) timed "
                 "in a graph of those launches only that walks all 18 layers (311 MB of weights per pass); per_shape "
                 "times come from graphs of one shape alone, whose 47-151 MB of weights fit the Infinity Cache",
-        "plans": {name: ops_plan(M, N, K, epi) for name, N, K, epi in EXPERT_SET},
+        "plans": layer_plans(layers[0], EXPERT_SET, M),
+        "weight_layout": "MFMA operand order (re-laid once after loading)" if OPTS["operand"] else "row-major [N, K]",
         "gemm_on_ready_codes": None,
         "per_shape": {name: {"us": round(per_launch_us[name], 3),
                              "GB/s": round(algorithmic_bytes(M, N, K, epi) / per_launch_us[name] / 1e3, 1)}
                       for name, N, K, epi in EXPERT_SET},
+        "per_pair_us": {k: round(v, 3) for k, v in per_launch_us.items() if "+" in k},
         "whole_path_frac": round(layer_bytes * n_layers / (value_us * 1e-6) / 1e9 / HBM_PEAK_GBS, 4),
     }
+    if not all(p.startswith("one launch") for p in roofline["plans"].values()):
+        roofline["kernel"] = "gemm_fp8_fusedq_kernel + gemm_fp8_skinny_kernel (M=50, four expert shapes)"
     if not args.no_extras:
         codes_us = gemm_only_layer_time(dev, layers, EXPERT_SET, ready_codes=True)
         roofline["gemm_on_ready_codes"] = {
@@ -770,7 +915,7 @@ def main() -> int:
         roofline["frac_of_measured_peak"] = round(achieved / measured["copy_GBps"], 4)
     node_us = launch_floor_us(dev)
     # one kernel per linear where it quantizes its own rows, else a quantizer and a GEMM
-    nodes_per_layer = sum(1 if one_launch(M, N, K, epi) else 2 for _, N, K, epi in EXPERT_SET)
+    nodes_per_layer = sum(1 if p.startswith("one launch") else 2 for p in roofline["plans"].values())
     floor_us = node_us * nodes_per_layer
     launch_floor = {
         "node_us": round(node_us, 3), "nodes_per_layer": nodes_per_layer, "floor_us_per_layer": round(floor_us, 2),

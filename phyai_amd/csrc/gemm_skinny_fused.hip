@@ -92,7 +92,7 @@ struct AmaxOut {
 // DIRECT: the weights are in MFMA operand order (weight_layout.h): lane i of a wavefront wants bytes
 // [16 i, 16 i + 16) and [1024 + 16 i, ...) of a 2 KB unit, so every request is 1 KB in a row and goes
 // straight into registers; LDS then holds only the activation codes.  Otherwise the weights are
-// row-major or in operand order and are staged through the wavefront's LDS slice.
+// row-major and are staged through the wavefront's LDS slice.
 //
 // AMAX_IN: the row maxima come from the producer of the activations (AmaxOut of an earlier launch)
 // instead of being found here: no table of per-wavefront maxima, no barrier before the conversions.
@@ -139,12 +139,7 @@ __global__ __launch_bounds__(FQ_THREADS) void gemm_fp8_fusedq_kernel(
 
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     const int l16 = lane & 15, q = lane >> 4;
-    // a_M = M | weights in MFMA operand order << 28 (weight_layout.h; gemm_skinny.hip reads them the same way)
-    const int M = a_M & 0x0FFFFFFF, N = a_N, K = a_K;
-    // (selected with masks and shifts, not with conditions: the code between the row loads and their
-    // wait must stay free of branches, see above)
-    const uint32_t om = DIRECT ? ~0u : 0u - (uint32_t)__builtin_amdgcn_readfirstlane((a_M >> 28) & 1);   // all ones: operand order
-    const int w_step_shift = 7 + (int)(om & 4);
+    const int M = a_M, N = a_N, K = a_K;
     const int half_n = N / 2;
     const int n_out_total = GATED ? half_n : N;
     const int col0 = blockIdx.x * (COLS_PER_TILE * NT);
@@ -239,11 +234,7 @@ __global__ __launch_bounds__(FQ_THREADS) void gemm_fp8_fusedq_kernel(
                     const int r = col0 + nt * 16 + r16;
                     wr = r < N ? r : N - 1;
                 }
-                // row-major: wr * K + 16 * chunk index; operand order: unit * 16 K + 16 * r16 + 256 * chunk index
-                const uint32_t w_units = (uint32_t)N >> 4, wu = blockIdx.x * NT + nt;
-                const uint32_t unit = wu < w_units ? wu : w_units - 1;
-                const uint32_t row = (uint32_t)wr + ((unit - (uint32_t)wr) & om);
-                woff[nt][hf] = __umul24(row, (uint32_t)K << (om & 4)) + (((uint32_t)r16 << 4) & om) + (chunk << (om & 4));
+                woff[nt][hf] = __umul24((uint32_t)wr, (uint32_t)K) + chunk;
             }
         }
 #pragma unroll
@@ -255,8 +246,8 @@ __global__ __launch_bounds__(FQ_THREADS) void gemm_fp8_fusedq_kernel(
             for (int nt = 0; nt < NT; ++nt)
 #pragma unroll
                 for (int hf = 0; hf < 2; ++hf) {
-                    if constexpr (STREAM) copy16_to_lds_nt(a_w + ((size_t)s_safe << w_step_shift), woff[nt][hf], dst + (nt * 2 + hf) * 1024);
-                    else copy16_to_lds(a_w + ((size_t)s_safe << w_step_shift), woff[nt][hf], dst + (nt * 2 + hf) * 1024);
+                    if constexpr (STREAM) copy16_to_lds_nt(a_w + ((size_t)s_safe << 7), woff[nt][hf], dst + (nt * 2 + hf) * 1024);
+                    else copy16_to_lds(a_w + ((size_t)s_safe << 7), woff[nt][hf], dst + (nt * 2 + hf) * 1024);
                 }
         }
     }
@@ -657,7 +648,7 @@ static int fq_launch_one(const GemmProblem& g, const FusedPlan& pl, hipStream_t 
         return -2;
     } else {
         const AmaxOut made = {EPI != EPI_NONE ? g.amax_out : nullptr};
-        const int m_flags = g.M | (g.weight_layout != W_ROW_MAJOR ? 1 << 28 : 0);
+        const int m_flags = g.M;   // (weights in operand order take the DIRECT kernels)
 #define PHYAI_FQ_ARGS g.w, reinterpret_cast<const uint8_t*>(g.x_bf16), g.K, g.N, m_flags, (int)(g.ldx * 2),                     \
                       reinterpret_cast<const uint8_t*>(g.amax_in), g.amax_parts, g.w_scale, g.bias, g.out, g.ldo, residual_of(g), made
         if (g.stream_weights)
