@@ -48,6 +48,7 @@
 #include "splitk.h"
 #include "weight_layout.h"
 #include <stdlib.h>
+#include <type_traits>
 
 namespace phyai {
 
@@ -144,6 +145,20 @@ __device__ __forceinline__ v8i big_frag(const uint8_t* buf, int row, int h, int 
     return f;
 }
 
+__device__ __forceinline__ v8i big_join(v4i lo, v4i hi) {
+    v8i f;
+    f[0] = lo[0]; f[1] = lo[1]; f[2] = lo[2]; f[3] = lo[3];
+    f[4] = hi[0]; f[5] = hi[1]; f[6] = hi[2]; f[7] = hi[3];
+    return f;
+}
+// The same block out of weights staged in operand order (WMODE 1): `row` is the block's first row plus l32;
+// chunk c of it lies at unit * 2 KB + c * 256 + (row % 16) * 16.  Sixteen consecutive lanes read 256 bytes in a
+// row: no bank conflicts.
+__device__ __forceinline__ v8i big_frag_operand(const uint8_t* buf, int row, int h, int kh) {
+    const uint8_t* r = buf + (row >> 4) * 2048 + (row & 15) * 16;
+    return big_join(*reinterpret_cast<const v4i*>(r + (4 * kh + h) * 256), *reinterpret_cast<const v4i*>(r + (4 * kh + 2 + h) * 256));
+}
+
 // DEPTH: stages of the LDS ring, each holding BIG_BK bytes of K for the whole tile.
 // Variants whose ring leaves room for two workgroups per CU are held to the register budget of
 // two wavefronts per SIMD: while one workgroup is in its prologue or epilogue the other one
@@ -151,7 +166,15 @@ __device__ __forceinline__ v8i big_frag(const uint8_t* buf, int row, int h, int 
 //
 // WGM x WGN: how the four wavefronts tile the workgroup's output (2 x 2, or 1 x 4 for the
 // 224 x 256 tile: every wavefront then walks all the tile's token rows and a quarter of its columns).
-template <int TM, int TN, int DEPTH, int EPI, bool SPLIT, int WGM = 2, int WGN = 2>
+//
+// WMODE: how the weights are laid out and reach the MFMA.  0: row-major [N, K] (or operand order, gathered
+// row by row into the same LDS layout: the slow way, kept for shapes without a dedicated variant), staged
+// through LDS in 128-byte rows.  1: MFMA operand order (weight_layout.h), staged through LDS as they lie:
+// a copy instruction moves 1 KB in a row, and lane (l32, h) finds chunk c of its row at
+// unit * 2 KB + c * 256 + (l32 % 16) * 16.  2: operand order and WGM == 1, so that a wavefront's weight
+// blocks are its own: they go global -> registers, DEPTH stage-loads ahead through a ring of register
+// sets, and LDS carries the activations only.
+template <int TM, int TN, int DEPTH, int EPI, bool SPLIT, int WGM = 2, int WGN = 2, int WMODE = 0>
 __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu((DEPTH == 2 && TM < 4) ? 2 : 1)))
 void gemm_fp8_big_kernel(
     const uint8_t* __restrict__ a_a, const uint8_t* __restrict__ a_b, int a_K, int a_M, int a_N, int a_m_tiles,
@@ -168,14 +191,26 @@ void gemm_fp8_big_kernel(
     p.m_tiles = a_m_tiles; p.n_tiles = a_n_tiles; p.band = a_band; p.by_rows = a_by_rows & 15; p.res = a_res;
     p.operand_w = __builtin_amdgcn_readfirstlane(a_by_rows >> 4);
     constexpr bool GATED = epi_is_gated(EPI);
+    constexpr bool OPW = WMODE != 0, BDIRECT = WMODE == 2;
     static_assert(WGM * WGN == 4, "four wavefronts per workgroup");
+    static_assert(!BDIRECT || (WGM == 1 && DEPTH == 4), "weights go straight to registers only where a wavefront owns them");
     constexpr int BM = WGM * 32 * TM, BN = WGN * 32 * TN;   // workgroup tile
     constexpr int WM = 32 * TM, WN = 32 * TN;        // wavefront tile
-    constexpr int STAGE_BYTES = (BM + BN) * BIG_BK;  // one stage: A rows, then B rows
-    constexpr int CA = BM / 32, CB = BN / 32;        // copy instructions (8 rows each) per wavefront per stage
-    constexpr int COPIES = CA + CB;
+    constexpr int STAGE_BYTES = (BM + (BDIRECT ? 0 : BN)) * BIG_BK;  // one stage: A rows, then B rows (if staged)
+    constexpr int CA = BM / 32, CB = BDIRECT ? 0 : BN / 32;   // copy instructions (8 rows each) per wavefront per stage
+    constexpr int BL = BDIRECT ? TN * 4 : 0;         // 16-byte weight loads per lane per stage: TN blocks x 2 K halves x 2
+    constexpr int COPIES = CA + CB + BL;             // vector-memory instructions per wavefront per stage-load
     constexpr int SLOTS_PER_STAGE = 2 * TM * TN;     // MFMAs of a wavefront per stage
-    constexpr int CPS = (COPIES * 2 + SLOTS_PER_STAGE - 1) / SLOTS_PER_STAGE;   // copies per MFMA: done by mid-stage
+    // Requests of a stage-load are numbered; request n goes out behind MFMA n / CPS counted from the barrier of
+    // the stage that frees its target.  Copies into LDS: CPS per MFMA, so that they are out by mid-stage.  With
+    // the weights going to registers: one per MFMA - the activation copies, then the weight loads of K half 0
+    // (whose registers are free once half 0 is done, i.e. at the barrier), and, numbered from LATE on so that
+    // they go out at the head of the NEXT stage, the weight loads of K half 1: its registers serve the MFMAs of
+    // the stage to its end.
+    constexpr int CPS = BDIRECT ? 1 : (COPIES * 2 + SLOTS_PER_STAGE - 1) / SLOTS_PER_STAGE;
+    constexpr int LATE = (TM - 1) * TN * CPS;        // first request number that falls into the next stage
+    constexpr int IDX_END = BDIRECT ? LATE + BL / 2 : COPIES;
+    static_assert(!BDIRECT || CA + BL / 2 <= LATE, "the requests behind the barrier fit the MFMAs of the half");
     static_assert((TM == TN && TM % 2 == 0) || (TM == 3 && TN == 2) || (TM == 7 && TN == 2) || (TM == 2 && TN == 1 && !GATED),
                   "supported wavefront tiles");
     static_assert(BM % 32 == 0 && BN % 32 == 0, "every wavefront copies whole groups of 8 rows");
@@ -185,6 +220,7 @@ void gemm_fp8_big_kernel(
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     const int wm = wave / WGN, wn = wave % WGN;
     const int l32 = lane & 31, h = lane >> 5;
+    (void)wm;
     const int half_n = p.N / 2;
     BigTile tile_id;
     int split_z = SPLIT ? (int)blockIdx.z : 0, n_splits = SPLIT ? (int)gridDim.z : 1;
@@ -210,7 +246,7 @@ void gemm_fp8_big_kernel(
 
     // ---- copy geometry: wavefront w moves 8-row groups w*CA .. of A and w*CB .. of B; lane i
     // fills slot i%8 of row i/8 of its group with the chunk that the swizzle assigns to it ------
-    uint32_t aoff[CA], boff[CB];
+    uint32_t aoff[CA], boff[CB > 0 ? CB : 1];
 #pragma unroll
     for (int i = 0; i < CA; ++i) {
         const int rt = (wave * CA + i) * 8 + (lane >> 3);         // row of the tile
@@ -218,8 +254,17 @@ void gemm_fp8_big_kernel(
         r = r < p.M ? r : p.M - 1;
         aoff[i] = (uint32_t)r * (uint32_t)p.K + (((lane & 7) ^ big_swizzle(rt)) << 4);
     }
+    // first 16-row unit of the tile in an operand-order matrix (plain: 16 weight rows; gated: 8 gate
+    // columns and the 8 up columns that pair with them), and the units the matrix has
+    const uint32_t unit0 = GATED ? (uint32_t)n0 >> 3 : (uint32_t)n0 >> 4, units = (uint32_t)p.N >> 4;
 #pragma unroll
     for (int i = 0; i < CB; ++i) {
+        if constexpr (WMODE == 1) {
+            // instruction i moves half a unit (1 KB) as it lies; units past the matrix repeat the last one
+            const uint32_t hu = wave * CB + i, u = unit0 + (hu >> 1);
+            boff[i] = (u < units ? u : units - 1) * ((uint32_t)p.K << 4) + (hu & 1) * 1024 + lane * 16;
+            continue;
+        }
         const int jj = (wave * CB + i) * 8 + (lane >> 3);         // column of the output tile
         int rb;
         uint32_t ob;   // the row's place in operand order
@@ -238,17 +283,40 @@ void gemm_fp8_big_kernel(
         boff[i] = p.operand_w ? ob + chunk * kOperandChunkBytes : (uint32_t)rb * (uint32_t)p.K + (chunk << 4);
     }
     const int k_begin = SPLIT ? split_z * p.k_per_split : 0;
-    const int b_step_shift = p.operand_w ? 4 : 0;   // a K step of operand-order weights is 2 KB away, not 128 bytes
+    const int b_step_shift = (OPW || p.operand_w) ? 4 : 0;   // a K step of operand-order weights is 2 KB away, not 128 bytes
+    // BDIRECT: this lane's 16 bytes of chunk h of row l32 of weight block j, K step 0; chunk c of the same row
+    // is c * 256 further, the next K step 2 KB
+    const uint8_t* bsrc[BDIRECT ? TN : 1];
+    v4i bring[BDIRECT ? DEPTH : 1][BDIRECT ? TN : 1][2][2];   // [stage-load % DEPTH][block][K half][chunk pair]
+    if constexpr (BDIRECT) {
+#pragma unroll
+        for (int j = 0; j < TN; ++j) {
+            const uint32_t u = unit0 + (uint32_t)(wn * (WN / 16) + 2 * j) + ((uint32_t)l32 >> 4);
+            bsrc[j] = p.b + (size_t)(u < units ? u : units - 1) * ((size_t)p.K << 4) + ((size_t)k_begin << 4) + h * 256 + (l32 & 15) * 16;
+        }
+    }
     const uint32_t lds_base = (uint32_t)(uintptr_t)lds;
     const uint32_t wave_a = __builtin_amdgcn_readfirstlane(lds_base + wave * (CA * 1024));
     const uint32_t wave_b = __builtin_amdgcn_readfirstlane(lds_base + BM * BIG_BK + wave * (CB * 1024));
     // copy c (0 .. COPIES-1) of this wavefront's share of stage-load `d` (K bytes [128 d, 128 d + 128))
-    auto issue = [&](int d, int c) {
+    // (slot: d % DEPTH as a compile-time value, needed where the target is a register set)
+    auto issue = [&](int d, int c, auto slot) {
         const int k = k_begin + d * BIG_BK;
         const uint32_t stage_off = (d % DEPTH) * STAGE_BYTES;
-        if (c < CA) copy16_to_lds(p.a + k, aoff[c], wave_a + stage_off + c * 1024);
-        else copy16_to_lds(p.b + ((size_t)k << b_step_shift), boff[c - CA], wave_b + stage_off + (c - CA) * 1024);
+        if (c < CA) {
+            copy16_to_lds(p.a + k, aoff[c], wave_a + stage_off + c * 1024);
+        } else if constexpr (BDIRECT) {
+            constexpr int S = decltype(slot)::value;
+            const int kh = c >= LATE ? 1 : 0, e = kh ? c - LATE : c - CA;       // request numbers CA .. and LATE ..
+            if (e < BL / 2) {
+                const int j = e >> 1, pr = e & 1;                              // chunk 4 kh + 2 pr + h of block j
+                bring[S][j][kh][pr] = *reinterpret_cast<const v4i*>(bsrc[j] + ((size_t)d << 11) + (4 * kh + 2 * pr) * 256);
+            }
+        } else {
+            copy16_to_lds(p.b + ((size_t)k << b_step_shift), boff[c - CA], wave_b + stage_off + (c - CA) * 1024);
+        }
     };
+    using Slot0 = std::integral_constant<int, 0>;
 
     v16f acc[TM][TN];
 #pragma unroll
@@ -261,6 +329,11 @@ void gemm_fp8_big_kernel(
     const int n_loads = (SPLIT ? p.k_per_split : p.K) / BIG_BK;   // stage-loads in all, >= DEPTH
     const int arow = wm * WM + l32, brow = wn * WN + l32;
     auto stage_ptr = [&](int d) -> const uint8_t* { return lds + (d % DEPTH) * STAGE_BYTES; };
+    // weight block with first row `row` - l32 out of the staged B rows, K half kh
+    auto read_b = [&](const uint8_t* bbuf, int row, int kh) -> v8i {
+        if constexpr (WMODE == 1) return big_frag_operand(bbuf, row, h, kh);
+        else return big_frag(bbuf, row, h, kh);
+    };
 
     // Operand blocks read one K half ahead: those of the current half (cur) and of the next one
     // (nxt); the two sets swap roles every half.  All B blocks and the first A block - or all A
@@ -285,7 +358,7 @@ void gemm_fp8_big_kernel(
 // MFMA pipe runs dry.  ISSUE: load D+DEPTH exists (requests after the barrier); ISSUE_P: load
 // D-1+DEPTH exists (requests still being spread before the barrier).  All flags are literals, so
 // the steady-state loop body is straight-line code.
-#define PHYAI_RUN_HALF(D, KH, NEXT, AHEAD, ISSUE_P, ISSUE, FA0, FB, NFA0, NFB)                                 \
+#define PHYAI_RUN_HALF(D, SLOT, KH, NEXT, AHEAD, ISSUE_P, ISSUE, FA0, FB, NFA0, NFB)                           \
     {                                                                                                          \
         const int d_ = (D);                                                                                    \
         const uint8_t* abuf_ = stage_ptr(d_);                                                                  \
@@ -302,9 +375,9 @@ void gemm_fp8_big_kernel(
                 _Pragma("unroll") for (int q_ = 0; q_ < TN + NA; ++q_) {                                       \
                     if (q_ * (TM - 1) / (TN + NA) != i_ - 1) continue;                                         \
                     if (q_ >= 1 && q_ <= NA) NFA0[q_ - 1] = big_frag(nbuf_, arow + (q_ - 1) * 32, h, 1 - (KH)); \
-                    else {                                                                                     \
+                    else if constexpr (!BDIRECT) {                                                             \
                         const int j_ = q_ == 0 ? 0 : q_ - NA;                                                  \
-                        NFB[j_] = big_frag(nbuf_ + BM * BIG_BK, brow + j_ * 32, h, 1 - (KH));                  \
+                        NFB[j_] = read_b(nbuf_ + BM * BIG_BK, brow + j_ * 32, 1 - (KH));                       \
                     }                                                                                          \
                 }                                                                                              \
             }                                                                                                  \
@@ -314,10 +387,17 @@ void gemm_fp8_big_kernel(
             /* MFMAs since the last barrier */                                                                 \
             const int slot0_ = after_ ? (i_ - 1) * TN : (TM - 1) * TN + ((KH) * TM + i_) * TN;                 \
             _Pragma("unroll") for (int j_ = 0; j_ < TN; ++j_) {                                                \
-                acc[i_][j_] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(FB[j_], fa_[i_], acc[i_][j_],    \
+                v8i fb_;                                                                                       \
+                if constexpr (BDIRECT) fb_ = big_join(bring[SLOT][j_][KH][0], bring[SLOT][j_][KH][1]);         \
+                else fb_ = FB[j_];                                                                             \
+                acc[i_][j_] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(fb_, fa_[i_], acc[i_][j_],       \
                                                                                0, 0, 0, 0, 0, 0);              \
                 _Pragma("unroll") for (int c_ = 0; c_ < CPS; ++c_)                                             \
-                    if (req_ && (slot0_ + j_) * CPS + c_ < COPIES) issue(load_, (slot0_ + j_) * CPS + c_);     \
+                    if (req_ && (slot0_ + j_) * CPS + c_ < IDX_END) {                                          \
+                        /* load d + DEPTH lands where load d was, load d - 1 + DEPTH where load d - 1 was */   \
+                        if (after_) issue(load_, (slot0_ + j_) * CPS + c_, std::integral_constant<int, (SLOT)>{});            \
+                        else issue(load_, (slot0_ + j_) * CPS + c_, std::integral_constant<int, ((SLOT) + DEPTH - 1) % DEPTH>{}); \
+                    }                                                                                          \
                 __builtin_amdgcn_sched_barrier(0);                                                             \
             }                                                                                                  \
             if ((KH) == 1 && i_ == 0 && (NEXT)) {                                                              \
@@ -328,37 +408,62 @@ void gemm_fp8_big_kernel(
         }                                                                                                      \
     }
 // a whole stage-load: half 0 with the cur register set, half 1 with the nxt set
-#define PHYAI_RUN_STAGE(D, NEXT, AHEAD, ISSUE_P, ISSUE)                                                        \
-    PHYAI_RUN_HALF(D, 0, 1, 0, ISSUE_P, 0, fa_cur, fb_cur, fa_nxt, fb_nxt)                                     \
-    PHYAI_RUN_HALF(D, 1, NEXT, AHEAD, ISSUE_P, ISSUE, fa_nxt, fb_nxt, fa_cur, fb_cur)
+#define PHYAI_RUN_STAGE(D, SLOT, NEXT, AHEAD, ISSUE_P, ISSUE)                                                  \
+    PHYAI_RUN_HALF(D, SLOT, 0, 1, 0, ISSUE_P, 0, fa_cur, fb_cur, fa_nxt, fb_nxt)                               \
+    PHYAI_RUN_HALF(D, SLOT, 1, NEXT, AHEAD, ISSUE_P, ISSUE, fa_nxt, fb_nxt, fa_cur, fb_cur)
 
     // prologue: stage-loads 0 .. DEPTH-2 and the copies of load DEPTH-1 that the row groups after
     // a barrier would have requested in flight (the rest of it is spread over stage-load 0 like
     // every later one), load 0 published, its opening blocks in registers.
-    constexpr int HEAD = (TM - 1) * TN * CPS < COPIES ? (TM - 1) * TN * CPS : COPIES;
+    // (as request numbers up to LATE, and as the instructions they are)
+    constexpr int HEAD_IDX = LATE < IDX_END ? LATE : IDX_END;
+    constexpr int HEAD = BDIRECT ? CA + BL / 2 : HEAD_IDX;
+    if constexpr (BDIRECT) {   // DEPTH == 4: stage-load d fills register set d
 #pragma unroll
-    for (int d = 0; d < DEPTH - 1; ++d)
+        for (int c = 0; c < IDX_END; ++c) issue(0, c, std::integral_constant<int, 0>{});
 #pragma unroll
-        for (int c = 0; c < COPIES; ++c) issue(d, c);
+        for (int c = 0; c < IDX_END; ++c) issue(1, c, std::integral_constant<int, 1>{});
 #pragma unroll
-    for (int c = 0; c < HEAD; ++c) issue(DEPTH - 1, c);
+        for (int c = 0; c < IDX_END; ++c) issue(2, c, std::integral_constant<int, 2>{});
+#pragma unroll
+        for (int c = 0; c < HEAD_IDX; ++c) issue(3, c, std::integral_constant<int, 3>{});
+    } else {
+#pragma unroll
+        for (int d = 0; d < DEPTH - 1; ++d)
+#pragma unroll
+            for (int c = 0; c < COPIES; ++c) issue(d, c, Slot0{});
+#pragma unroll
+        for (int c = 0; c < HEAD_IDX; ++c) issue(DEPTH - 1, c, Slot0{});
+    }
     wait_copies<COPIES * (DEPTH - 2) + HEAD>();
     __syncthreads();
 #pragma unroll
-    for (int j = 0; j < TN; ++j) fb_cur[j] = big_frag(lds + BM * BIG_BK, brow + j * 32, h, 0);
+    for (int j = 0; j < TN; ++j)
+        if constexpr (!BDIRECT) fb_cur[j] = read_b(lds + BM * BIG_BK, brow + j * 32, 0);
 #pragma unroll
     for (int i = 0; i < (A_AHEAD ? TM : 1); ++i) fa_cur[i] = big_frag(lds, arow + i * 32, h, 0);
     int d = 0;
-    for (; d < n_loads - DEPTH; ++d) { PHYAI_RUN_STAGE(d, 1, DEPTH - 2, 1, 1) }
+    if constexpr (BDIRECT) {
+        // the register sets are named at compile time: four stage-loads per trip (the launcher sees to it
+        // that their number is a multiple of four)
+        for (; d < n_loads - DEPTH; d += DEPTH) {
+            PHYAI_RUN_STAGE(d, 0, 1, DEPTH - 2, 1, 1)
+            PHYAI_RUN_STAGE(d + 1, 1, 1, DEPTH - 2, 1, 1)
+            PHYAI_RUN_STAGE(d + 2, 2, 1, DEPTH - 2, 1, 1)
+            PHYAI_RUN_STAGE(d + 3, 3, 1, DEPTH - 2, 1, 1)
+        }
+    } else {
+        for (; d < n_loads - DEPTH; ++d) { PHYAI_RUN_STAGE(d, 0, 1, DEPTH - 2, 1, 1) }
+    }
     // d == n_loads - DEPTH: the last requests are still being spread, then the ring drains
     if constexpr (DEPTH == 2) {
-        PHYAI_RUN_STAGE(d, 1, 0, 1, 0)
-        PHYAI_RUN_STAGE(d + 1, 0, 0, 0, 0)
+        PHYAI_RUN_STAGE(d, 0, 1, 0, 1, 0)
+        PHYAI_RUN_STAGE(d + 1, 0, 0, 0, 0, 0)
     } else {
-        PHYAI_RUN_STAGE(d, 1, 2, 1, 0)
-        PHYAI_RUN_STAGE(d + 1, 1, 1, 0, 0)
-        PHYAI_RUN_STAGE(d + 2, 1, 0, 0, 0)
-        PHYAI_RUN_STAGE(d + 3, 0, 0, 0, 0)
+        PHYAI_RUN_STAGE(d, 0, 1, 2, 1, 0)
+        PHYAI_RUN_STAGE(d + 1, 1, 1, 1, 0, 0)
+        PHYAI_RUN_STAGE(d + 2, 2, 1, 0, 0, 0)
+        PHYAI_RUN_STAGE(d + 3, 3, 0, 0, 0, 0)
     }
 #undef PHYAI_RUN_STAGE
 #undef PHYAI_RUN_HALF
@@ -442,6 +547,47 @@ void gemm_fp8_big_kernel(
     }
     __syncthreads();  // every wavefront is done reading operands from LDS
     uint8_t* stg = lds + wave * STG_BYTES;
+    if constexpr (OPW && GATED) {
+        // Weights in the gated operand order: rows 4p .. 4p+3 of a 16-row unit are gate columns 2p, 2p+1 and up
+        // columns 2p, 2p+1.  Accumulator 4k + e of lane (l32, h) of block j is block row 8k + 4h + e, i.e. with
+        // e = 2t + b: gate (t = 0) / up (t = 1) of output column 16 j + 4 k + 2 h + b of the wavefront - a lane
+        // holds both halves of two neighbouring output columns per k.  Same arithmetic as below, operation for
+        // operation.
+#pragma unroll
+        for (int j = 0; j < TN; ++j) {
+            float sgk[4][2], suk[4][2], bgk[4][2], buk[4][2];
+#pragma unroll
+            for (int k = 0; k < 4; ++k) {
+                const int n = nbase + 16 * j + 4 * k + 2 * h;
+                const int n_safe = n < n_lim ? n : 0;
+#pragma unroll
+                for (int b = 0; b < 2; ++b) {
+                    sgk[k][b] = p.b_scale[n_safe + b];
+                    suk[k][b] = p.b_scale[half_n + n_safe + b];
+                    bgk[k][b] = p.bias ? bf16_bits_to_f32(p.bias[n_safe + b]) : 0.f;
+                    buk[k][b] = p.bias ? bf16_bits_to_f32(p.bias[half_n + n_safe + b]) : 0.f;
+                }
+            }
+#pragma unroll
+            for (int i = 0; i < TM; ++i) {
+                const int row = i * 32 + l32;
+                const int sw = (row / ROWS_PER_PASS) & (SLOTS - 1);
+#pragma unroll
+                for (int k = 0; k < 4; ++k) {
+                    const float g0 = __builtin_fmaf(acc[i][j][4 * k + 0], sa[i] * sgk[k][0], bgk[k][0]);
+                    const float g1 = __builtin_fmaf(acc[i][j][4 * k + 1], sa[i] * sgk[k][1], bgk[k][1]);
+                    const float u0 = __builtin_fmaf(acc[i][j][4 * k + 2], sa[i] * suk[k][0], buk[k][0]);
+                    const float u1 = __builtin_fmaf(acc[i][j][4 * k + 3], sa[i] * suk[k][1], buk[k][1]);
+                    // gate and up pass through bf16 first, as the two-launch form materialises them
+                    const uint32_t g01 = pack_bf16x2(g0, g1), u01 = pack_bf16x2(u0, u1);
+                    const float o0 = apply_act<EPI>(__uint_as_float(g01 << 16)) * __uint_as_float(u01 << 16);
+                    const float o1 = apply_act<EPI>(__uint_as_float(g01 & 0xFFFF0000u)) * __uint_as_float(u01 & 0xFFFF0000u);
+                    const int slot = (2 * j + (k >> 1)) ^ sw;
+                    *reinterpret_cast<uint32_t*>(stg + row * ROWB + slot * 16 + 8 * (k & 1) + 4 * h) = pack_bf16x2(o0, o1);
+                }
+            }
+        }
+    } else {
 #pragma unroll
     for (int j = 0; j < TNO; ++j) {
         v4f sg[4], bg[4], su[4], bu[4];
@@ -497,6 +643,7 @@ void gemm_fp8_big_kernel(
                 *reinterpret_cast<uint2*>(stg + row * ROWB + slot * 16 + h * 8) = w;
             }
         }
+    }
     }
     // write the staged tile out: 1 KB (whole rows) per instruction.  The output is written once
     // and never read here: non-temporal stores keep it from evicting the operands that the
@@ -599,7 +746,8 @@ BigPlan big_plan(int M, int N, int K, int epilogue) {
     }
     if (const char* e = tuning_env("PHYAI_FP8_BIG_SPLITS")) {
         const int s = atoi(e);
-        if (pl.tile != 192 && pl.tile != 224 && pl.cols != 64 && s >= 1 && K % (s * 128) == 0 && K / s >= 512 && tiles * s <= 4096) pl.splits = s;
+        // (224-row tiles exist with a split K only for weights in operand order, see launch_gemm_big)
+        if (pl.tile != 192 && pl.cols != 64 && s >= 1 && K % (s * 128) == 0 && K / s >= 512 && tiles * s <= 4096) pl.splits = s;
     }
     if (const char* e = tuning_env("PHYAI_FP8_BIG_DEPTH")) {
         const int d = atoi(e);
@@ -614,7 +762,7 @@ size_t big_partial_bytes(int M, int N, int epilogue, const BigPlan& pl) {
     return (size_t)big_tiles(M, N, epilogue, pl.tile, bn) * pl.splits * pl.tile * bn * sizeof(float);
 }
 
-template <int TM, int TN, int DEPTH, int EPI, int WGM = 2, int WGN = 2>
+template <int TM, int TN, int DEPTH, int EPI, int WGM = 2, int WGN = 2, int WMODE = 0>
 static void big_launch(BigArgs a, const GemmProblem& g, int splits, hipStream_t st) {
     const bool gated = epi_is_gated(EPI);
     constexpr int BM = WGM * 32 * TM, BN = WGN * 32 * TN;
@@ -670,25 +818,33 @@ static void big_launch(BigArgs a, const GemmProblem& g, int splits, hipStream_t 
 #define PHYAI_BIG_ARGS a.a, a.b, a.K, a.M, a.N, a.m_tiles, a.n_tiles, a.band, a.by_rows | (a.operand_w << 4), a.k_per_split, a.a_scale, \
                        a.b_scale, a.bias, a.out, a.ldo, a.a_scale_scalar, a.partials, a.counters, a.res
     if (splits > 1) {
-        if constexpr (TM == TN && (TM == 4 || DEPTH == 4))
-            hipLaunchKernelGGL((gemm_fp8_big_kernel<TM, TN, DEPTH, EPI, true, WGM, WGN>), grid, dim3(256), 0, st, PHYAI_BIG_ARGS);
+        if constexpr ((TM == TN && (TM == 4 || DEPTH == 4)) || WMODE == 2)
+            hipLaunchKernelGGL((gemm_fp8_big_kernel<TM, TN, DEPTH, EPI, true, WGM, WGN, WMODE>), grid, dim3(256), 0, st, PHYAI_BIG_ARGS);
     } else {
-        hipLaunchKernelGGL((gemm_fp8_big_kernel<TM, TN, DEPTH, EPI, false, WGM, WGN>), grid, dim3(256), 0, st, PHYAI_BIG_ARGS);
+        hipLaunchKernelGGL((gemm_fp8_big_kernel<TM, TN, DEPTH, EPI, false, WGM, WGN, WMODE>), grid, dim3(256), 0, st, PHYAI_BIG_ARGS);
     }
 #undef PHYAI_BIG_ARGS
 }
 
-template <int TM, int TN, int DEPTH, int WGM = 2, int WGN = 2>
+template <int TM, int TN, int DEPTH, int WGM = 2, int WGN = 2, int WMODE = 0>
 static int big_launch_epi(const BigArgs& a, const GemmProblem& g, int splits, hipStream_t st) {
     switch (g.epilogue) {
-    case EPI_NONE: big_launch<TM, TN, DEPTH, EPI_NONE, WGM, WGN>(a, g, splits, st); return 0;
-    case EPI_GEGLU_TANH: big_launch<TM, TN, DEPTH, EPI_GEGLU_TANH, WGM, WGN>(a, g, splits, st); return 0;
-    case EPI_GEGLU_ERF: big_launch<TM, TN, DEPTH, EPI_GEGLU_ERF, WGM, WGN>(a, g, splits, st); return 0;
-    case EPI_SWIGLU: big_launch<TM, TN, DEPTH, EPI_SWIGLU, WGM, WGN>(a, g, splits, st); return 0;
-    case EPI_GELU_TANH: big_launch<TM, TN, DEPTH, EPI_GELU_TANH, WGM, WGN>(a, g, splits, st); return 0;
-    case EPI_GELU_ERF: big_launch<TM, TN, DEPTH, EPI_GELU_ERF, WGM, WGN>(a, g, splits, st); return 0;
+    case EPI_NONE: big_launch<TM, TN, DEPTH, EPI_NONE, WGM, WGN, WMODE>(a, g, splits, st); return 0;
+    case EPI_GEGLU_TANH: big_launch<TM, TN, DEPTH, EPI_GEGLU_TANH, WGM, WGN, WMODE>(a, g, splits, st); return 0;
+    case EPI_GEGLU_ERF: big_launch<TM, TN, DEPTH, EPI_GEGLU_ERF, WGM, WGN, WMODE>(a, g, splits, st); return 0;
+    case EPI_SWIGLU: big_launch<TM, TN, DEPTH, EPI_SWIGLU, WGM, WGN, WMODE>(a, g, splits, st); return 0;
+    case EPI_GELU_TANH: big_launch<TM, TN, DEPTH, EPI_GELU_TANH, WGM, WGN, WMODE>(a, g, splits, st); return 0;
+    case EPI_GELU_ERF: big_launch<TM, TN, DEPTH, EPI_GELU_ERF, WGM, WGN, WMODE>(a, g, splits, st); return 0;
     default: return -2;
     }
+}
+
+// The same tile shape for row-major weights (or operand order gathered row by row) and for weights staged in
+// operand order as they lie.
+template <int TM, int TN, int DEPTH, int WGM = 2, int WGN = 2>
+static int big_launch_layout(const BigArgs& a, const GemmProblem& g, int splits, hipStream_t st) {
+    if (a.operand_w && !tuning_env("PHYAI_FP8_BIG_GATHER")) return big_launch_epi<TM, TN, DEPTH, WGM, WGN, 1>(a, g, splits, st);
+    return big_launch_epi<TM, TN, DEPTH, WGM, WGN, 0>(a, g, splits, st);
 }
 
 int launch_gemm_big(const GemmProblem& g, const BigPlan& pl, hipStream_t st) {
@@ -706,20 +862,28 @@ int launch_gemm_big(const GemmProblem& g, const BigPlan& pl, hipStream_t st) {
     if (pl.splits > 1 && (g.workspace == nullptr ||
                           g.workspace_bytes < kGemmHeaderBytes + big_partial_bytes(g.M, g.N, g.epilogue, pl)))
         return -3;
-    if (pl.tile == 256) return big_launch_epi<4, 4, 2>(a, g, pl.splits, st);
-    if (pl.tile == 224 && pl.splits == 1) return big_launch_epi<7, 2, 2, 1, 4>(a, g, 1, st);
-    if (pl.tile == 192 && pl.splits == 1) return big_launch_epi<3, 2, 2>(a, g, 1, st);
+    if (pl.tile == 256) return big_launch_layout<4, 4, 2>(a, g, pl.splits, st);
+    if (pl.tile == 224) {
+        // weights in operand order and a whole number of four-stage trips per K range: the wavefronts load
+        // their own weight blocks straight into registers (PHYAI_FP8_BIG_DIRECT=0: stage them like the rest)
+        const bool direct = a.operand_w && (g.K / pl.splits) % 512 == 0 && g.K / pl.splits >= 512 &&
+                            !(tuning_env("PHYAI_FP8_BIG_DIRECT") && atoi(tuning_env("PHYAI_FP8_BIG_DIRECT")) == 0);
+        if (direct) return big_launch_epi<7, 2, 4, 1, 4, 2>(a, g, pl.splits, st);
+        if (pl.splits == 1) return big_launch_layout<7, 2, 2, 1, 4>(a, g, 1, st);
+        return -2;
+    }
+    if (pl.tile == 192 && pl.splits == 1) return big_launch_layout<3, 2, 2>(a, g, 1, st);
     if (pl.tile == 128 && pl.cols == 64) {
         if (pl.splits != 1) return -2;
         switch (g.epilogue) {   // plain epilogues only: one column block per wavefront cannot hold a gate / up pair
-        case EPI_NONE: big_launch<2, 1, 4, EPI_NONE>(a, g, 1, st); return 0;
-        case EPI_GELU_TANH: big_launch<2, 1, 4, EPI_GELU_TANH>(a, g, 1, st); return 0;
-        case EPI_GELU_ERF: big_launch<2, 1, 4, EPI_GELU_ERF>(a, g, 1, st); return 0;
+        case EPI_NONE: a.operand_w ? big_launch<2, 1, 4, EPI_NONE, 2, 2, 1>(a, g, 1, st) : big_launch<2, 1, 4, EPI_NONE>(a, g, 1, st); return 0;
+        case EPI_GELU_TANH: a.operand_w ? big_launch<2, 1, 4, EPI_GELU_TANH, 2, 2, 1>(a, g, 1, st) : big_launch<2, 1, 4, EPI_GELU_TANH>(a, g, 1, st); return 0;
+        case EPI_GELU_ERF: a.operand_w ? big_launch<2, 1, 4, EPI_GELU_ERF, 2, 2, 1>(a, g, 1, st) : big_launch<2, 1, 4, EPI_GELU_ERF>(a, g, 1, st); return 0;
         default: return -2;
         }
     }
-    if (pl.tile == 128 && pl.depth == 4) return big_launch_epi<2, 2, 4>(a, g, pl.splits, st);
-    if (pl.tile == 128 && pl.splits == 1) return big_launch_epi<2, 2, 2>(a, g, 1, st);
+    if (pl.tile == 128 && pl.depth == 4) return big_launch_layout<2, 2, 4>(a, g, pl.splits, st);
+    if (pl.tile == 128 && pl.splits == 1) return big_launch_layout<2, 2, 2>(a, g, 1, st);
     return -2;
 }
 

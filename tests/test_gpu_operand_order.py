@@ -125,16 +125,43 @@ def test_operand_order_with_the_gated_residual(dev, M, N, K):
     assert torch.equal(_bits(lin_op), _bits(lin_rm)) and torch.equal(_bits(gemm_op), _bits(gemm_rm))
 
 
+# how the pipelined tile kernel takes weights in operand order: staged through LDS as they lie (and, for the
+# 224-row tile with K a multiple of 512, straight into registers); the same without the register path; gathered
+# row by row into the row-major staging layout
+@pytest.mark.parametrize("mode", ["", "PHYAI_FP8_BIG_DIRECT=0", "PHYAI_FP8_BIG_GATHER=1"])
 @pytest.mark.parametrize("tile", ["256", "224", "192", "128", "128/2", "12864"])
 @pytest.mark.parametrize("M,N,K,epi", [(816, 768, 1024, None), (513, 400, 1536, "gelu"), (816, 1024, 1152, "geglu_tanh"),
-                                       (260, 288, 1024, "swiglu")])
-def test_operand_order_in_every_pipelined_tile_shape(dev, monkeypatch, tile, M, N, K, epi):
+                                       (260, 288, 1024, "swiglu"), (300, 544, 2048, "geglu_erf")])
+def test_operand_order_in_every_pipelined_tile_shape(dev, monkeypatch, mode, tile, M, N, K, epi):
     t, _, depth = tile.partition("/")
     monkeypatch.setenv("PHYAI_FP8_BIG", t)
     if depth:
         monkeypatch.setenv("PHYAI_FP8_BIG_DEPTH", depth)
+    if mode:
+        monkeypatch.setenv(*mode.split("="))
     (lin_rm, _), (lin_op, _) = _both_layouts(dev, M, N, K, epi, seed=M + N + K + 1)
     assert torch.equal(_bits(lin_op), _bits(lin_rm))
+
+
+@pytest.mark.parametrize("splits", ["2", "4"])
+@pytest.mark.parametrize("M,N,K,epi", [(816, 512, 4096, None), (300, 544, 2048, "swiglu"), (816, 2048, 16384, None)])
+def test_split_k_of_the_224_row_tile_with_weights_in_registers(dev, monkeypatch, splits, M, N, K, epi):
+    """Only weights in operand order give the 224-row tile a split K; the result is held to the unsplit row-major
+    one (split-K changes the order of additions: close, not equal) and is the same from run to run."""
+    ops = _ops()
+    x, wq, ws, b = _problem(dev, M, N, K, seed=M + N + K + 5)
+    gated = epi in GATED
+    wo = ops.fp8_weight_to_operand_order(wq, gated=gated)
+    want = ops.fp8_linear(x, wq, ws, b, epilogue=epi).float()
+    monkeypatch.setenv("PHYAI_FP8_BIG", "224")
+    monkeypatch.setenv("PHYAI_FP8_BIG_SPLITS", splits)
+    outs = [ops.fp8_linear(x, wo, ws, b, epilogue=epi, weight_layout="operand_gated" if gated else "operand") for _ in range(3)]
+    torch.cuda.synchronize()
+    assert torch.equal(_bits(outs[0]), _bits(outs[1])) and torch.equal(_bits(outs[0]), _bits(outs[2]))
+    err = (outs[0].float() - want).abs().max().item()
+    assert err <= 1e-2 * want.abs().max().item(), err
+    for w in ops._workspaces.values():
+        assert int(w[: ops.WORKSPACE_HEADER_BYTES].max().item()) == 0
 
 
 @pytest.mark.parametrize("force", [("PHYAI_FP8_BIG_SPLITS", "2"), ("PHYAI_FP8_BIG_SPLITS", "4"), ("PHYAI_FP8_TILE", "128,128,1"),
