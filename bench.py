@@ -238,16 +238,29 @@ def decoder_layer_times(dev, layers, M, denoise_steps, steps, warmup):
         for _ in range(denoise_steps):
             for layer in layers:
                 q, o, gu, dn = layer["qkv"], layer["o"], layer["gate_up"], layer["down"]
+                (wq_, lq), (wo_, lo), (wg_, lg), (wd_, ld) = weight_of(q), weight_of(o), weight_of(gu), weight_of(dn)
                 nq, ns, gate = ops.adarmsnorm_fp8(h, mods[0], 1e-6)
-                ops.fp8_gemm(nq, ns, q["w"], q["ws"], None, out=q["out"])
-                ops.fp8_linear(attn, o["w"], o["ws"], None, residual=h, gate=gate, out=h1)
+                ops.fp8_gemm(nq, ns, wq_, q["ws"], None, out=q["out"], weight_layout=lq)
+                ops.fp8_linear(attn, wo_, o["ws"], None, residual=h, gate=gate, out=h1, weight_layout=lo)
                 mq, ms, gate2 = ops.adarmsnorm_fp8(h1, mods[1], 1e-6)
-                a = ops.fp8_gemm(mq, ms, gu["w"], gu["ws"], None, epilogue="geglu_tanh", out=gu["out"],
-                                 stream_weights=gu.get("stream", False))
-                ops.fp8_linear(a, dn["w"], dn["ws"], None, residual=h1, gate=gate2, out=h2)
+                a = ops.fp8_gemm(mq, ms, wg_, gu["ws"], None, epilogue="geglu_tanh", out=gu["out"],
+                                 stream_weights=gu.get("stream", False), weight_layout=lg)
+                ops.fp8_linear(a, wd_, dn["ws"], None, residual=h1, gate=gate2, out=h2, weight_layout=ld)
+
+    def one_launch_linears():
+        for _ in range(denoise_steps):
+            for layer in layers:
+                q, o, gu, dn = layer["qkv"], layer["o"], layer["gate_up"], layer["down"]
+                (wq_, lq), (wo_, lo), (wg_, lg), (wd_, ld) = weight_of(q), weight_of(o), weight_of(gu), weight_of(dn)
+                n, gate = ops.adarmsnorm(h, mods[0], 1e-6)
+                ops.fp8_linear(n, wq_, q["ws"], None, out=q["out"], weight_layout=lq)
+                ops.fp8_linear(attn, wo_, o["ws"], None, residual=h, gate=gate, out=h1, weight_layout=lo)
+                m, gate2 = ops.adarmsnorm(h1, mods[1], 1e-6)
+                ops.fp8_mlp(m, wg_, gu["ws"], None, wd_, dn["ws"], None, epilogue="geglu_tanh", residual=h1, gate=gate2,
+                            out=h2, stream_weights1=gu.get("stream", False), weight1_layout=lg, weight2_layout=ld)
 
     res = {}
-    for name, fn in (("separate", separate), ("fused", fused)):
+    for name, fn in (("separate", separate), ("fused", fused), ("one_launch_linears", one_launch_linears)):
         gr = HipGraph()
         gr.capture(fn, {})
         ts, _ = time_replays(gr, steps, warmup)
@@ -981,7 +994,8 @@ def main() -> int:
                           "gate_up+GeGLU, down -> gated residual; kernels per layer: separate = "
                           f"{4 + sum(lin.values())} (2 norms, 2 addcmul, the four linears), fused = "
                           f"{4 + lin['o'] + lin['down']} (2 norm+quantizer, qkv and gate_up GEMMs on their codes, o and down "
-                          "with the gated residual in the epilogue)"}
+                          "with the gated residual in the epilogue), one_launch_linears = 6 (2 norms writing bf16, qkv and "
+                          "o + residual as one-launch linears, the MLP as one call of two kernels with the residual behind it)"}
         extra["torch_reference_path_us"] = {
             "expert_step": torch_reference_times(dev, layers, EXPERT_SET, denoise_steps, max(10, args.steps // 10), 3),
             "note": "same linears through the reference's own arithmetic on this GPU: torch-op quantizer + "

@@ -159,6 +159,11 @@ __device__ __forceinline__ v8i big_frag_operand(const uint8_t* buf, int row, int
     return big_join(*reinterpret_cast<const v4i*>(r + (4 * kh + h) * 256), *reinterpret_cast<const v4i*>(r + (4 * kh + 2 + h) * 256));
 }
 
+// Variants held to the register and LDS budget of two workgroups per CU (two wavefronts per SIMD).
+__host__ __device__ constexpr bool big_two_per_cu(int tm, int tn, int depth, int wmode) {
+    return depth == 2 && tm < 4;
+}
+
 // DEPTH: stages of the LDS ring, each holding BIG_BK bytes of K for the whole tile.
 // Variants whose ring leaves room for two workgroups per CU are held to the register budget of
 // two wavefronts per SIMD: while one workgroup is in its prologue or epilogue the other one
@@ -175,7 +180,7 @@ __device__ __forceinline__ v8i big_frag_operand(const uint8_t* buf, int row, int
 // blocks are its own: they go global -> registers, DEPTH stage-loads ahead through a ring of register
 // sets, and LDS carries the activations only.
 template <int TM, int TN, int DEPTH, int EPI, bool SPLIT, int WGM = 2, int WGN = 2, int WMODE = 0>
-__global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu((DEPTH == 2 && TM < 4) ? 2 : 1)))
+__global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(big_two_per_cu(TM, TN, DEPTH, WMODE) ? 2 : 1)))
 void gemm_fp8_big_kernel(
     const uint8_t* __restrict__ a_a, const uint8_t* __restrict__ a_b, int a_K, int a_M, int a_N, int a_m_tiles,
     int a_n_tiles, int a_band, int a_by_rows, int a_k_per_split, const float* __restrict__ a_a_scale,
@@ -202,20 +207,26 @@ void gemm_fp8_big_kernel(
     constexpr int COPIES = CA + CB + BL;             // vector-memory instructions per wavefront per stage-load
     constexpr int SLOTS_PER_STAGE = 2 * TM * TN;     // MFMAs of a wavefront per stage
     // Requests of a stage-load are numbered; request n goes out behind MFMA n / CPS counted from the barrier of
-    // the stage that frees its target.  Copies into LDS: CPS per MFMA, so that they are out by mid-stage.  With
-    // the weights going to registers: one per MFMA - the activation copies, then the weight loads of K half 0
-    // (whose registers are free once half 0 is done, i.e. at the barrier), and, numbered from LATE on so that
-    // they go out at the head of the NEXT stage, the weight loads of K half 1: its registers serve the MFMAs of
-    // the stage to its end.
-    constexpr int CPS = BDIRECT ? 1 : (COPIES * 2 + SLOTS_PER_STAGE - 1) / SLOTS_PER_STAGE;
+    // the stage that frees its target: CPS per MFMA, so that they are out by mid-stage.
+    // LEAD: the barrier of stage d frees the target of stage-load d + LEAD.  Staged operands: LEAD = DEPTH - the
+    // barrier waits for this wavefront's LDS reads of stage d, whose stage is then refilled.  Weights in registers:
+    // LEAD = DEPTH - 1 - the targets (LDS stage and register set of stage d - 1) were last read by MFMAs that
+    // every wavefront has issued before it reaches the barrier of stage d, so the barrier need not wait for the
+    // LDS reads in flight (the activation blocks of the second K half, requested just before it), and no register
+    // set is written while MFMAs of its stage are still to come.
+    constexpr int CPS = (COPIES * 2 + SLOTS_PER_STAGE - 1) / SLOTS_PER_STAGE;
+    constexpr int LEAD = BDIRECT ? DEPTH - 1 : DEPTH;
     constexpr int LATE = (TM - 1) * TN * CPS;        // first request number that falls into the next stage
-    constexpr int IDX_END = BDIRECT ? LATE + BL / 2 : COPIES;
-    static_assert(!BDIRECT || CA + BL / 2 <= LATE, "the requests behind the barrier fit the MFMAs of the half");
+    constexpr int IDX_END = COPIES;
+    static_assert(!BDIRECT || COPIES <= LATE, "with weights in registers every request goes out behind the barrier");
     static_assert((TM == TN && TM % 2 == 0) || (TM == 3 && TN == 2) || (TM == 7 && TN == 2) || (TM == 2 && TN == 1 && !GATED),
                   "supported wavefront tiles");
     static_assert(BM % 32 == 0 && BN % 32 == 0, "every wavefront copies whole groups of 8 rows");
     static_assert(DEPTH == 2 || DEPTH == 4, "ring depth");
-    __shared__ __attribute__((aligned(1024))) uint8_t lds[DEPTH * STAGE_BYTES];
+    // (the epilogue stages the bf16 tile in the same LDS; where the ring is smaller than that, the ring grows)
+    constexpr int EPI_STAGING = 4 * WM * ((GATED ? TN / 2 : TN) * 64);
+    constexpr int LDS_BYTES = DEPTH * STAGE_BYTES > EPI_STAGING ? DEPTH * STAGE_BYTES : EPI_STAGING;
+    __shared__ __attribute__((aligned(1024))) uint8_t lds[LDS_BYTES];
 
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     const int wm = wave / WGN, wn = wave % WGN;
@@ -243,6 +254,14 @@ void gemm_fp8_big_kernel(
     if (tile_id.n >= p.n_tiles || tile_id.m >= p.m_tiles) return;   // padding of the tile order
     const int m0 = tile_id.m * BM;
     const int n0 = GATED ? tile_id.n * (BN / 2) : tile_id.n * BN;
+
+    v16f acc[TM][TN];
+#pragma unroll
+    for (int i = 0; i < TM; ++i)
+#pragma unroll
+        for (int j = 0; j < TN; ++j)
+#pragma unroll
+            for (int r = 0; r < 16; ++r) acc[i][j][r] = 0.f;
 
     // ---- copy geometry: wavefront w moves 8-row groups w*CA .. of A and w*CB .. of B; lane i
     // fills slot i%8 of row i/8 of its group with the chunk that the swizzle assigns to it ------
@@ -307,24 +326,13 @@ void gemm_fp8_big_kernel(
             copy16_to_lds(p.a + k, aoff[c], wave_a + stage_off + c * 1024);
         } else if constexpr (BDIRECT) {
             constexpr int S = decltype(slot)::value;
-            const int kh = c >= LATE ? 1 : 0, e = kh ? c - LATE : c - CA;       // request numbers CA .. and LATE ..
-            if (e < BL / 2) {
-                const int j = e >> 1, pr = e & 1;                              // chunk 4 kh + 2 pr + h of block j
-                bring[S][j][kh][pr] = *reinterpret_cast<const v4i*>(bsrc[j] + ((size_t)d << 11) + (4 * kh + 2 * pr) * 256);
-            }
+            const int e = c - CA, j = e >> 2, kh = (e >> 1) & 1, pr = e & 1;   // chunk 4 kh + 2 pr + h of block j
+            bring[S][j][kh][pr] = *reinterpret_cast<const v4i*>(bsrc[j] + ((size_t)d << 11) + (4 * kh + 2 * pr) * 256);
         } else {
             copy16_to_lds(p.b + ((size_t)k << b_step_shift), boff[c - CA], wave_b + stage_off + (c - CA) * 1024);
         }
     };
     using Slot0 = std::integral_constant<int, 0>;
-
-    v16f acc[TM][TN];
-#pragma unroll
-    for (int i = 0; i < TM; ++i)
-#pragma unroll
-        for (int j = 0; j < TN; ++j)
-#pragma unroll
-            for (int r = 0; r < 16; ++r) acc[i][j][r] = 0.f;
 
     const int n_loads = (SPLIT ? p.k_per_split : p.K) / BIG_BK;   // stage-loads in all, >= DEPTH
     const int arow = wm * WM + l32, brow = wn * WN + l32;
@@ -383,7 +391,7 @@ void gemm_fp8_big_kernel(
             }                                                                                                  \
             const bool after_ = (KH) == 1 && i_ >= 1;   /* past this stage-load's barrier */                   \
             const bool req_ = after_ ? (ISSUE) : (ISSUE_P);                                                    \
-            const int load_ = after_ ? d_ + DEPTH : d_ - 1 + DEPTH;                                            \
+            const int load_ = after_ ? d_ + LEAD : d_ - 1 + LEAD;                                              \
             /* MFMAs since the last barrier */                                                                 \
             const int slot0_ = after_ ? (i_ - 1) * TN : (TM - 1) * TN + ((KH) * TM + i_) * TN;                 \
             _Pragma("unroll") for (int j_ = 0; j_ < TN; ++j_) {                                                \
@@ -394,16 +402,22 @@ void gemm_fp8_big_kernel(
                                                                                0, 0, 0, 0, 0, 0);              \
                 _Pragma("unroll") for (int c_ = 0; c_ < CPS; ++c_)                                             \
                     if (req_ && (slot0_ + j_) * CPS + c_ < IDX_END) {                                          \
-                        /* load d + DEPTH lands where load d was, load d - 1 + DEPTH where load d - 1 was */   \
-                        if (after_) issue(load_, (slot0_ + j_) * CPS + c_, std::integral_constant<int, (SLOT)>{});            \
-                        else issue(load_, (slot0_ + j_) * CPS + c_, std::integral_constant<int, ((SLOT) + DEPTH - 1) % DEPTH>{}); \
+                        /* (register set of the load: its number modulo DEPTH) */                              \
+                        if (after_) issue(load_, (slot0_ + j_) * CPS + c_, std::integral_constant<int, ((SLOT) + LEAD) % DEPTH>{});     \
+                        else issue(load_, (slot0_ + j_) * CPS + c_, std::integral_constant<int, ((SLOT) + LEAD - 1) % DEPTH>{}); \
                     }                                                                                          \
                 __builtin_amdgcn_sched_barrier(0);                                                             \
             }                                                                                                  \
             if ((KH) == 1 && i_ == 0 && (NEXT)) {                                                              \
-                asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory"); /* my reads of stage-load D have landed */  \
-                wait_copies<COPIES * (AHEAD)>();                   /* ... my copies of D+1 too ... */          \
-                __syncthreads();                                   /* ... and so have everybody's */           \
+                if constexpr (BDIRECT) {                                                                       \
+                    wait_copies<COPIES * (AHEAD)>();               /* my requests of D+1 have landed ... */    \
+                    __builtin_amdgcn_s_barrier();                  /* ... and so have everybody's */           \
+                    asm volatile("" ::: "memory");                                                             \
+                } else {                                                                                       \
+                    asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory"); /* my reads of stage-load D have landed */ \
+                    wait_copies<COPIES * (AHEAD)>();               /* ... my copies of D+1 too ... */          \
+                    __syncthreads();                               /* ... and so have everybody's */           \
+                }                                                                                              \
             }                                                                                                  \
         }                                                                                                      \
     }
@@ -417,16 +431,14 @@ void gemm_fp8_big_kernel(
     // every later one), load 0 published, its opening blocks in registers.
     // (as request numbers up to LATE, and as the instructions they are)
     constexpr int HEAD_IDX = LATE < IDX_END ? LATE : IDX_END;
-    constexpr int HEAD = BDIRECT ? CA + BL / 2 : HEAD_IDX;
-    if constexpr (BDIRECT) {   // DEPTH == 4: stage-load d fills register set d
+    constexpr int HEAD = BDIRECT ? 0 : HEAD_IDX;
+    if constexpr (BDIRECT) {   // stage-loads 0 .. LEAD - 1 = 2; stage-load d fills register set d % 4
 #pragma unroll
         for (int c = 0; c < IDX_END; ++c) issue(0, c, std::integral_constant<int, 0>{});
 #pragma unroll
         for (int c = 0; c < IDX_END; ++c) issue(1, c, std::integral_constant<int, 1>{});
 #pragma unroll
         for (int c = 0; c < IDX_END; ++c) issue(2, c, std::integral_constant<int, 2>{});
-#pragma unroll
-        for (int c = 0; c < HEAD_IDX; ++c) issue(3, c, std::integral_constant<int, 3>{});
     } else {
 #pragma unroll
         for (int d = 0; d < DEPTH - 1; ++d)
@@ -435,7 +447,7 @@ void gemm_fp8_big_kernel(
 #pragma unroll
         for (int c = 0; c < HEAD_IDX; ++c) issue(DEPTH - 1, c, Slot0{});
     }
-    wait_copies<COPIES * (DEPTH - 2) + HEAD>();
+    wait_copies<COPIES * (LEAD - 2) + HEAD + (BDIRECT ? COPIES : 0)>();   // stage-load 0 has landed
     __syncthreads();
 #pragma unroll
     for (int j = 0; j < TN; ++j)
@@ -446,17 +458,23 @@ void gemm_fp8_big_kernel(
     if constexpr (BDIRECT) {
         // the register sets are named at compile time: four stage-loads per trip (the launcher sees to it
         // that their number is a multiple of four)
+        // at the barrier of stage d stage-load d + 2 may be in flight; behind it stage-load d + 3 is requested
         for (; d < n_loads - DEPTH; d += DEPTH) {
-            PHYAI_RUN_STAGE(d, 0, 1, DEPTH - 2, 1, 1)
-            PHYAI_RUN_STAGE(d + 1, 1, 1, DEPTH - 2, 1, 1)
-            PHYAI_RUN_STAGE(d + 2, 2, 1, DEPTH - 2, 1, 1)
-            PHYAI_RUN_STAGE(d + 3, 3, 1, DEPTH - 2, 1, 1)
+            PHYAI_RUN_STAGE(d, 0, 1, 1, 0, 1)
+            PHYAI_RUN_STAGE(d + 1, 1, 1, 1, 0, 1)
+            PHYAI_RUN_STAGE(d + 2, 2, 1, 1, 0, 1)
+            PHYAI_RUN_STAGE(d + 3, 3, 1, 1, 0, 1)
         }
     } else {
         for (; d < n_loads - DEPTH; ++d) { PHYAI_RUN_STAGE(d, 0, 1, DEPTH - 2, 1, 1) }
     }
     // d == n_loads - DEPTH: the last requests are still being spread, then the ring drains
-    if constexpr (DEPTH == 2) {
+    if constexpr (BDIRECT) {   // the last request goes out behind the barrier of stage n - 4
+        PHYAI_RUN_STAGE(d, 0, 1, 1, 0, 1)
+        PHYAI_RUN_STAGE(d + 1, 1, 1, 1, 0, 0)
+        PHYAI_RUN_STAGE(d + 2, 2, 1, 0, 0, 0)
+        PHYAI_RUN_STAGE(d + 3, 3, 0, 0, 0, 0)
+    } else if constexpr (DEPTH == 2) {
         PHYAI_RUN_STAGE(d, 0, 1, 0, 1, 0)
         PHYAI_RUN_STAGE(d + 1, 0, 0, 0, 0, 0)
     } else {
@@ -514,7 +532,7 @@ void gemm_fp8_big_kernel(
     constexpr int SLOTS = ROWB / 16;
     constexpr int ROWS_PER_PASS = 16 / SLOTS > 0 ? 16 / SLOTS : 1;   // rows per 256 bytes of banks
     constexpr int STG_BYTES = WM * ROWB;                 // per wavefront
-    static_assert(4 * STG_BYTES <= DEPTH * STAGE_BYTES, "staging fits in the operand LDS");
+    static_assert(4 * STG_BYTES <= LDS_BYTES, "staging fits in the operand LDS");
     const int n_lim = GATED ? half_n : p.N;
     const int nbase = n0 + wn * (GATED ? WN / 2 : WN);
     // column constants are read 4 at a time when the arrays allow it (N is a multiple of 16, so
@@ -746,8 +764,7 @@ BigPlan big_plan(int M, int N, int K, int epilogue) {
     }
     if (const char* e = tuning_env("PHYAI_FP8_BIG_SPLITS")) {
         const int s = atoi(e);
-        // (224-row tiles exist with a split K only for weights in operand order, see launch_gemm_big)
-        if (pl.tile != 192 && pl.cols != 64 && s >= 1 && K % (s * 128) == 0 && K / s >= 512 && tiles * s <= 4096) pl.splits = s;
+        if (pl.tile != 192 && pl.tile != 224 && pl.cols != 64 && s >= 1 && K % (s * 128) == 0 && K / s >= 512 && tiles * s <= 4096) pl.splits = s;
     }
     if (const char* e = tuning_env("PHYAI_FP8_BIG_DEPTH")) {
         const int d = atoi(e);
@@ -785,7 +802,7 @@ static void big_launch(BigArgs a, const GemmProblem& g, int splits, hipStream_t 
         // ... unless the busiest XCD then needs one more round of tiles than in the other order
         // (13056 x 2560 x 2048 in 256 x 256 tiles: 510 tiles are 64 per XCD by tile columns, two
         // rounds on 32 CUs, but 65 on some XCDs by tile rows: 92 against 75.5 us)
-        const int slots = 32 * ((DEPTH == 2 && TM < 4) ? 2 : 1);
+        const int slots = 32 * (big_two_per_cu(TM, TN, DEPTH, WMODE) ? 2 : 1);
         const int rounds_c = big_ceil_div(big_max_tiles_per_xcd(a.m_tiles, a.n_tiles, 4), slots);
         const int rounds_r = big_ceil_div(big_max_tiles_per_xcd(a.n_tiles, a.m_tiles, 4), slots);
         if (rounds_c != rounds_r) a.by_rows = rounds_r < rounds_c;
@@ -818,7 +835,7 @@ static void big_launch(BigArgs a, const GemmProblem& g, int splits, hipStream_t 
 #define PHYAI_BIG_ARGS a.a, a.b, a.K, a.M, a.N, a.m_tiles, a.n_tiles, a.band, a.by_rows | (a.operand_w << 4), a.k_per_split, a.a_scale, \
                        a.b_scale, a.bias, a.out, a.ldo, a.a_scale_scalar, a.partials, a.counters, a.res
     if (splits > 1) {
-        if constexpr ((TM == TN && (TM == 4 || DEPTH == 4)) || WMODE == 2)
+        if constexpr (TM == TN && (TM == 4 || DEPTH == 4))
             hipLaunchKernelGGL((gemm_fp8_big_kernel<TM, TN, DEPTH, EPI, true, WGM, WGN, WMODE>), grid, dim3(256), 0, st, PHYAI_BIG_ARGS);
     } else {
         hipLaunchKernelGGL((gemm_fp8_big_kernel<TM, TN, DEPTH, EPI, false, WGM, WGN, WMODE>), grid, dim3(256), 0, st, PHYAI_BIG_ARGS);
@@ -866,11 +883,11 @@ int launch_gemm_big(const GemmProblem& g, const BigPlan& pl, hipStream_t st) {
     if (pl.tile == 224) {
         // weights in operand order and a whole number of four-stage trips per K range: the wavefronts load
         // their own weight blocks straight into registers (PHYAI_FP8_BIG_DIRECT=0: stage them like the rest)
-        const bool direct = a.operand_w && (g.K / pl.splits) % 512 == 0 && g.K / pl.splits >= 512 &&
+        const bool direct = a.operand_w && g.K % 512 == 0 &&
                             !(tuning_env("PHYAI_FP8_BIG_DIRECT") && atoi(tuning_env("PHYAI_FP8_BIG_DIRECT")) == 0);
-        if (direct) return big_launch_epi<7, 2, 4, 1, 4, 2>(a, g, pl.splits, st);
-        if (pl.splits == 1) return big_launch_layout<7, 2, 2, 1, 4>(a, g, 1, st);
-        return -2;
+        if (pl.splits != 1) return -2;
+        if (direct) return big_launch_epi<7, 2, 4, 1, 4, 2>(a, g, 1, st);
+        return big_launch_layout<7, 2, 2, 1, 4>(a, g, 1, st);
     }
     if (pl.tile == 192 && pl.splits == 1) return big_launch_layout<3, 2, 2>(a, g, 1, st);
     if (pl.tile == 128 && pl.cols == 64) {

@@ -143,41 +143,6 @@ def test_operand_order_in_every_pipelined_tile_shape(dev, monkeypatch, mode, til
     assert torch.equal(_bits(lin_op), _bits(lin_rm))
 
 
-@pytest.mark.parametrize("splits", ["2", "4"])
-@pytest.mark.parametrize("M,N,K,epi", [(816, 512, 4096, None), (300, 544, 2048, "swiglu"), (816, 2048, 16384, None)])
-def test_split_k_of_the_224_row_tile_with_weights_in_registers(dev, monkeypatch, splits, M, N, K, epi):
-    """Only weights in operand order give the 224-row tile a split K; the result is held to the unsplit row-major
-    one (split-K changes the order of additions: close, not equal) and is the same from run to run."""
-    ops = _ops()
-    x, wq, ws, b = _problem(dev, M, N, K, seed=M + N + K + 5)
-    gated = epi in GATED
-    wo = ops.fp8_weight_to_operand_order(wq, gated=gated)
-    want = ops.fp8_linear(x, wq, ws, b, epilogue=epi).float()
-    monkeypatch.setenv("PHYAI_FP8_BIG", "224")
-    monkeypatch.setenv("PHYAI_FP8_BIG_SPLITS", splits)
-    outs = [ops.fp8_linear(x, wo, ws, b, epilogue=epi, weight_layout="operand_gated" if gated else "operand") for _ in range(3)]
-    torch.cuda.synchronize()
-    assert torch.equal(_bits(outs[0]), _bits(outs[1])) and torch.equal(_bits(outs[0]), _bits(outs[2]))
-    err = (outs[0].float() - want).abs().max().item()
-    assert err <= 1e-2 * want.abs().max().item(), err
-    for w in ops._workspaces.values():
-        assert int(w[: ops.WORKSPACE_HEADER_BYTES].max().item()) == 0
-
-
-@pytest.mark.parametrize("force", [("PHYAI_FP8_BIG_SPLITS", "2"), ("PHYAI_FP8_BIG_SPLITS", "4"), ("PHYAI_FP8_TILE", "128,128,1"),
-                                   ("PHYAI_FP8_TILE", "64,128,4"), ("PHYAI_FP8_SKINNY_STAGED", "0")])
-@pytest.mark.parametrize("M,N,K,epi", [(300, 384, 4096, None), (64, 512, 2048, "geglu_tanh"), (40, 256, 1024, None)])
-def test_operand_order_in_the_split_generic_and_unstaged_kernels(dev, monkeypatch, force, M, N, K, epi):
-    monkeypatch.setenv("PHYAI_FP8_FUSED", "0")
-    if force[0] == "PHYAI_FP8_BIG_SPLITS":
-        monkeypatch.setenv("PHYAI_FP8_BIG", "128")
-    if force[0] == "PHYAI_FP8_SKINNY_STAGED":
-        monkeypatch.setenv("PHYAI_FP8_BIG", "0")
-    monkeypatch.setenv(*force)
-    (lin_rm, gemm_rm), (lin_op, gemm_op) = _both_layouts(dev, M, N, K, epi, seed=M + N + K + 2)
-    assert torch.equal(_bits(lin_op), _bits(lin_rm)) and torch.equal(_bits(gemm_op), _bits(gemm_rm))
-
-
 def test_layout_and_epilogue_must_match(dev):
     ops = _ops()
     from phyai_amd import _lib
