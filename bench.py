@@ -712,6 +712,62 @@ def probe(dev, layers, M, shapes=EXPERT_SET):
     print("probe done")
 
 
+def stamps_report(dev):
+    """`--stamps`: the cycle budget of the GEMM kernels from inside (debug build of the library, whose kernels record the
+    shader clock at the ends of their phases; csrc/stamps.h).  Per workload one launch with fresh weights; per phase the
+    median over the wavefronts of the cycles between two stamps, the shader clock the launch ran at (against the 100 MHz
+    counter), and the span from the first wavefront's start to the last one's end.  Prints a markdown table."""
+    from phyai_amd import ops
+
+    big = ["start -> first stage published", "main loop", "split-K sums gathered", "epilogue arithmetic, tile staged",
+           "stores issued", "stores through"]
+    small = ["start -> rows landed", "row scales known", "codes written", "MFMAs done", "partial sums exchanged",
+             "epilogue, stores issued", "stores through"]
+    work = [("prefill gate_up + GeGLU", 816, 32768, 2048, "geglu_tanh"), ("prefill down", 816, 2048, 16384, None),
+            ("prefill qkv", 816, 2560, 2048, None), ("prefill o", 816, 2048, 2048, None),
+            ("batched gate_up + GeGLU (B = 8)", 6528, 32768, 2048, "geglu_tanh"),
+            ("expert qkv", 50, 2560, 1024, None), ("expert o", 50, 1024, 2048, None),
+            ("expert gate_up + GeGLU", 50, 8192, 1024, "geglu_tanh")]
+    only = os.environ.get("PHYAI_BENCH_STAMPS_ONLY")
+    if only:
+        work = [w for w in work if only in w[0]]
+    print("| workload | kernel | clock GHz | first start -> last end, us | phase: median cycles per wavefront (10 % .. 90 %) |")
+    print("|---|---|---|---|---|")
+    for label, M, N, K, epi in work:
+        lay = make_layers(dev, [("x", N, K, epi)], M, 2, seed0=4321)
+        for t in (lay[0]["x"], lay[1]["x"]):      # first a warm-up launch on other weights, stamps off
+            ops.debug_stamps(0)
+            linear(lay[0]["x"])
+            torch.cuda.synchronize()
+        t = lay[1]["x"]
+        small_m = one_launch(M, N, K, epi)
+        if not small_m:
+            xq, xs = ops.fp8_quant_rowwise(t["x"])
+        rec = ops.debug_stamps(8192)
+        if small_m:
+            linear(t)
+        else:
+            w, wl = weight_of(t)
+            ops.fp8_gemm(xq, xs, w, t["ws"], None, epilogue=t["epi"], out=t["out"], weight_layout=wl)
+        torch.cuda.synchronize()
+        ops.debug_stamps(0)
+        r = rec.cpu().double()
+        r = r[r[:, 0] > 0]
+        names = small if small_m else big
+        last = ops.STAMP_WORDS - 3
+        marks = [0] + [i for i in range(1, last) if bool((r[:, i] > 0).any())] + [last]
+        clock = ((r[:, last] - r[:, 0]) / ((r[:, -1] - r[:, -2]).clamp_min(1) / 100e6) / 1e9).median().item()
+        span = (r[:, -1].max() - r[:, -2].min()).item() / 100.0      # 100 MHz counter, common to the chip -> us
+        cells = []
+        for a, b in zip(marks[:-1], marks[1:]):
+            d = (r[:, b] - r[:, a]).sort().values
+            name = names[b - 1] if b != last else names[-1]
+            cells.append(f"{name}: {d[len(d) // 2].item():.0f} ({d[len(d) // 10].item():.0f} .. {d[(9 * len(d)) // 10].item():.0f})")
+        plan = ops_plan(M, N, K, epi) if small_m else ops.describe_plan(M, N, K, epi)
+        print(f"| {label} {M} x {N} x {K} | {plan}, {len(r)} wavefronts | {clock:.2f} | {span:.1f} | " + "; ".join(cells) + " |")
+        del lay, rec
+
+
 def cpu_info():
     """CPU model string and physical core count of the host (from /proc/cpuinfo)."""
     model, cores = "unknown", set()
@@ -837,6 +893,9 @@ def main() -> int:
                     help="the same for the prefill GEMM shapes (M = 816, 4 weight sets), for the MFMA / LDS counters")
     ap.add_argument("--probe-m", type=int, default=816,
                     help="token rows of --probe-prefill (816 x batch for the batched-serving shapes)")
+    ap.add_argument("--stamps", action="store_true",
+                    help="cycle budgets of the GEMM kernels from time stamps inside them: needs the debug build of the "
+                         "library (`make -C phyai_amd/csrc stamps`), prints a markdown table and exits")
     ap.add_argument("--row-major", action="store_true",
                     help="A/B: pass the weights row-major [N, K] instead of in MFMA operand order")
     ap.add_argument("--separate-linears", action="store_true",
@@ -844,6 +903,8 @@ def main() -> int:
     args = ap.parse_args()
     OPTS["operand"] = not args.row_major
     OPTS["mlp"] = not args.separate_linears
+    if args.stamps:
+        os.environ["PHYAI_FP8_LIBRARY"] = "stamps"   # before the library is opened
     if args.gpus != 1 or int(os.environ.get("WORLD_SIZE", "1")) != 1:
         print("bench.py: this path is built and measured on ONE GPU (TP=1, no collectives); "
               "run with --gpus 1", file=sys.stderr)
@@ -858,6 +919,9 @@ def main() -> int:
     torch.cuda.set_device(dev)
     M, n_layers, denoise_steps = 50, 18, 10
 
+    if args.stamps:
+        stamps_report(dev)
+        return 0
     if args.probe_prefill:
         probe(dev, make_layers(dev, PREFILL_SET, args.probe_m, 4, seed0=10_000), args.probe_m, PREFILL_SET)
         return 0

@@ -295,6 +295,19 @@ int phyai_fp8_describe_linear_plan(int64_t M, int64_t N, int64_t K, int epilogue
 int phyai_fp8_debug_cast_e4m3(const float *v, int64_t n, void *codes, void *stream);
 
 /*
+ * Time stamps of the kernels' phases, for the debug build of the library only (`make stamps` in
+ * phyai_amd/csrc builds lib/libphyai_fp8_stamps.so; the normal build returns PHYAI_FP8_EUNSUPPORTED).  From this
+ * call on every wavefront of the pipelined tile kernel and of the one-launch small-M kernel writes one record of
+ * PHYAI_FP8_STAMP_WORDS 64-bit words into `records` (device memory for n_records records, index = workgroup *
+ * wavefronts per workgroup + wavefront; records past the end are dropped): shader-clock stamps of its phases in
+ * words [0, 10), the 100 MHz counter at entry and at the end in the last two (csrc/stamps.h says what each
+ * marks).  n_records = 0 switches the recording off.  Synchronises the device.  Not part of the reference surface:
+ * this is how the cycle budgets of the kernels were measured.
+ */
+#define PHYAI_FP8_STAMP_WORDS 12
+int phyai_fp8_debug_stamps(uint64_t *records, int64_t n_records);
+
+/*
  * Hardware probe: `workgroups` workgroups of four wavefronts each issue iters x 16 independent
  * v_mfma_f32_32x32x64_f8f6f4 (32 x 32 x 64 x 2 flops each) and touch no memory.  counters (device,
  * 2 x workgroups 64-bit words) receives per workgroup the shader cycles and the 100 MHz ticks its

@@ -11,7 +11,10 @@ import os
 import subprocess
 
 _PKG = os.path.dirname(os.path.abspath(__file__))
-LIB_PATH = os.path.join(_PKG, "lib", "libphyai_fp8.so")
+# PHYAI_FP8_LIBRARY=stamps (set before the first call) makes the whole process use the debug build whose GEMM
+# kernels record time stamps of their phases (`make -C phyai_amd/csrc stamps`): same entry points, same results.
+STAMPS_LIB_PATH = os.path.join(_PKG, "lib", "libphyai_fp8_stamps.so")
+LIB_PATH = STAMPS_LIB_PATH if os.environ.get("PHYAI_FP8_LIBRARY") == "stamps" else os.path.join(_PKG, "lib", "libphyai_fp8.so")
 CSRC_DIR = os.path.join(_PKG, "csrc")
 ABI_VERSION = 8
 
@@ -42,6 +45,7 @@ SIGNATURES: dict[str, tuple[object, list[object]]] = {
     "phyai_fp8_describe_plan": (_int, [_i64, _i64, _i64, _int, ctypes.c_char_p, _sz]),
     "phyai_fp8_describe_linear_plan": (_int, [_i64, _i64, _i64, _int, ctypes.c_char_p, _sz]),
     "phyai_fp8_debug_cast_e4m3": (_int, [_vp, _i64, _vp, _vp]),
+    "phyai_fp8_debug_stamps": (_int, [_vp, _i64]),
     "phyai_fp8_debug_mfma_rate": (_int, [_int, _int, _vp, _vp, _vp]),
 }
 
@@ -60,28 +64,32 @@ def build(verbose: bool = False) -> str:
     return LIB_PATH
 
 
-def load() -> ctypes.CDLL:
-    global _lib
-    if _lib is not None:
-        return _lib
-    if not os.path.exists(LIB_PATH):
+def open_library(path: str) -> ctypes.CDLL:
+    """Open one build of the library and give its entry points their signatures."""
+    if not os.path.exists(path):
         raise Fp8LibraryError(
-            f"{LIB_PATH} not found: build it with `make -C {CSRC_DIR}` "
+            f"{path} not found: build it with `make -C {CSRC_DIR}` "
             "(or phyai_amd._lib.build()); there is no non-HIP fallback"
         )
-    lib = ctypes.CDLL(LIB_PATH)
+    lib = ctypes.CDLL(path)
     for name, (res, args) in SIGNATURES.items():
         try:
             fn = getattr(lib, name)
         except AttributeError as e:
-            raise Fp8LibraryError(f"{LIB_PATH} does not export {name}; rebuild it") from e
+            raise Fp8LibraryError(f"{path} does not export {name}; rebuild it") from e
         fn.restype = res
         fn.argtypes = args
     got = lib.phyai_fp8_abi_version()
     if got != ABI_VERSION:
-        raise Fp8LibraryError(f"{LIB_PATH} has ABI version {got}, expected {ABI_VERSION}; rebuild it")
-    _lib = lib
+        raise Fp8LibraryError(f"{path} has ABI version {got}, expected {ABI_VERSION}; rebuild it")
     return lib
+
+
+def load() -> ctypes.CDLL:
+    global _lib
+    if _lib is None:
+        _lib = open_library(LIB_PATH)
+    return _lib
 
 
 def check(rc: int, what: str) -> None:

@@ -589,6 +589,18 @@ int phyai_fp8_debug_mfma_rate(int workgroups, int iters, uint64_t* counters, flo
     return check_launch("phyai_fp8_debug_mfma_rate");
 }
 
+int phyai_fp8_debug_stamps(uint64_t* records, int64_t n_records) {
+    if (n_records < 0 || n_records > 0x7FFFFFFF || (n_records > 0 && !records))
+        return fail(PHYAI_FP8_EINVAL, "phyai_fp8_debug_stamps: bad arguments");
+    const int a = phyai::launch_set_stamp_sink_big(reinterpret_cast<unsigned long long*>(records), (unsigned int)n_records);
+    const int b = phyai::launch_set_stamp_sink_fused(reinterpret_cast<unsigned long long*>(records), (unsigned int)n_records);
+    if (a == -2 || b == -2)
+        return fail(PHYAI_FP8_EUNSUPPORTED, "phyai_fp8_debug_stamps: this library was built without time stamps "
+                    "(make stamps builds lib/libphyai_fp8_stamps.so)");
+    if (a != 0 || b != 0) return fail(PHYAI_FP8_ELAUNCH, "phyai_fp8_debug_stamps: hipMemcpyToSymbol failed");
+    return PHYAI_FP8_OK;
+}
+
 int phyai_fp8_debug_cast_e4m3(const float* v, int64_t n, void* codes, void* stream) {
     if (n < 0 || (n > 0 && (!v || !codes))) return fail(PHYAI_FP8_EINVAL, "phyai_fp8_debug_cast_e4m3: bad arguments");
     phyai::launch_debug_cast(v, n, codes, static_cast<hipStream_t>(stream));

@@ -129,16 +129,20 @@ def check_text(asm_text: str, min_kernels: int = 100) -> list[str]:
     return bad
 
 
-def check_file(make: bool = True) -> list[str]:
+def check_file(make: bool = True, stamps: bool = False) -> list[str]:
+    """stamps: the debug build with time stamps (make stamps), whose kernels must obey the same rules."""
+    target = "_obj/stamps_gemm_skinny_fused.s" if stamps else "_obj/gemm_skinny_fused.s"
     if make:
-        r = subprocess.run(["make", "-C", CSRC, "_obj/gemm_skinny_fused.s"], capture_output=True, text=True)
+        r = subprocess.run(["make", "-C", CSRC, target], capture_output=True, text=True)
         if r.returncode != 0:
-            return [f"make _obj/gemm_skinny_fused.s failed: {r.stderr[-2000:]}"]
-    return check_text(open(ASM, encoding="utf-8").read())
+            return [f"make {target} failed: {r.stderr[-2000:]}"]
+    return check_text(open(os.path.join(CSRC, target), encoding="utf-8").read())
 
 
 if __name__ == "__main__":
-    problems = check_file()
+    import sys
+
+    problems = check_file(stamps="--stamps" in sys.argv)
     for p in problems[:50]:
         print(p)
     print(f"{len(problems)} problem(s)")

@@ -46,6 +46,7 @@
 #include "launch.h"
 #include "tuning.h"
 #include "splitk.h"
+#include "stamps.h"
 #include "weight_layout.h"
 #include <stdlib.h>
 #include <type_traits>
@@ -53,6 +54,9 @@
 namespace phyai {
 
 constexpr int BIG_BK = 128;   // bytes of K per LDS row: one L2 cache line
+// (debug build only: where the kernels below leave their time stamps - 1 first stage published, 2 main loop done,
+// 3 split-K sums gathered, 4 epilogue arithmetic done and tile staged, 5 stores issued)
+PHYAI_STAMP_SINK(g_big_stamps)
 
 struct BigArgs {
     const uint8_t* __restrict__ a;   // xq [M, K]
@@ -195,6 +199,7 @@ void gemm_fp8_big_kernel(
     // a_by_rows = tile order | weights in operand order << 4
     p.m_tiles = a_m_tiles; p.n_tiles = a_n_tiles; p.band = a_band; p.by_rows = a_by_rows & 15; p.res = a_res;
     p.operand_w = __builtin_amdgcn_readfirstlane(a_by_rows >> 4);
+    PHYAI_STAMP_BEGIN
     constexpr bool GATED = epi_is_gated(EPI);
     constexpr bool OPW = WMODE != 0, BDIRECT = WMODE == 2;
     static_assert(WGM * WGN == 4, "four wavefronts per workgroup");
@@ -449,6 +454,7 @@ void gemm_fp8_big_kernel(
     }
     wait_copies<COPIES * (LEAD - 2) + HEAD + (BDIRECT ? COPIES : 0)>();   // stage-load 0 has landed
     __syncthreads();
+    PHYAI_STAMP(1)
 #pragma unroll
     for (int j = 0; j < TN; ++j)
         if constexpr (!BDIRECT) fb_cur[j] = read_b(lds + BM * BIG_BK, brow + j * 32, 0);
@@ -485,6 +491,7 @@ void gemm_fp8_big_kernel(
     }
 #undef PHYAI_RUN_STAGE
 #undef PHYAI_RUN_HALF
+    PHYAI_STAMP(2)
 
     // ---- split-K: publish partial sums; the last split to arrive adds them in split order --
     // Two blocks (32 floats per lane) at a time, so that the 4 x 4 variant never holds more than
@@ -519,6 +526,7 @@ void gemm_fp8_big_kernel(
         splitk_reset(p.counters, tile);
     }
 
+    PHYAI_STAMP(3)
     // ---- epilogue ------------------------------------------------------------------------
     // The weight block is the MFMA's first operand, so accumulator r of lane (l32, h) of block
     // (i, j) is the output at token row i*32 + l32, column j*32 + 8*(r/4) + 4*h + r%4: a lane
@@ -663,6 +671,7 @@ void gemm_fp8_big_kernel(
         }
     }
     }
+    PHYAI_STAMP(4)
     // write the staged tile out: 1 KB (whole rows) per instruction.  The output is written once
     // and never read here: non-temporal stores keep it from evicting the operands that the
     // neighbouring tiles still want from L2 (4800 x 8192 x 2048 + GELU: 113 -> 95 us;
@@ -677,6 +686,8 @@ void gemm_fp8_big_kernel(
         const int n = nbase + slot * 8;
         if (m < p.M && n < n_lim) __builtin_nontemporal_store(v, reinterpret_cast<v4i*>(p.out + (int64_t)m * p.ldo + n));
     }
+    PHYAI_STAMP(5)
+    PHYAI_STAMP_END(g_big_stamps, ((size_t)blockIdx.x + (size_t)gridDim.x * blockIdx.z) * 4 + wave, lane)
 }
 
 // ---- host side ---------------------------------------------------------------------------
@@ -862,6 +873,16 @@ template <int TM, int TN, int DEPTH, int WGM = 2, int WGN = 2>
 static int big_launch_layout(const BigArgs& a, const GemmProblem& g, int splits, hipStream_t st) {
     if (a.operand_w && !tuning_env("PHYAI_FP8_BIG_GATHER")) return big_launch_epi<TM, TN, DEPTH, WGM, WGN, 1>(a, g, splits, st);
     return big_launch_epi<TM, TN, DEPTH, WGM, WGN, 0>(a, g, splits, st);
+}
+
+int launch_set_stamp_sink_big(unsigned long long* buf, unsigned int records) {
+#ifdef PHYAI_FP8_STAMPS
+    const StampSink s = {buf, records};
+    return hipMemcpyToSymbol(HIP_SYMBOL(g_big_stamps), &s, sizeof(s)) == hipSuccess ? 0 : -4;
+#else
+    (void)buf; (void)records;
+    return -2;
+#endif
 }
 
 int launch_gemm_big(const GemmProblem& g, const BigPlan& pl, hipStream_t st) {

@@ -28,6 +28,7 @@
 #include <type_traits>
 
 #include "quant_device.h"
+#include "stamps.h"
 #include "tuning.h"
 #include "weight_layout.h"
 #include <stdio.h>
@@ -36,6 +37,9 @@ namespace phyai {
 
 constexpr int FQ_WAVES = 8;
 constexpr int FQ_THREADS = FQ_WAVES * kWave;
+// (debug build only: the kernel's time stamps - 1 rows landed, 2 row scales known, 3 codes written, 4 MFMAs done,
+// 5 partial sums exchanged, 6 stores issued)
+PHYAI_STAMP_SINK(g_fq_stamps)
 
 // A 16-byte load whose arrival the compiler does not track: the value may be used only after
 // landed() has waited for it.
@@ -140,6 +144,7 @@ __global__ __launch_bounds__(FQ_THREADS) void gemm_fp8_fusedq_kernel(
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     const int l16 = lane & 15, q = lane >> 4;
     const int M = a_M, N = a_N, K = a_K;
+    PHYAI_STAMP_BEGIN
     const int half_n = N / 2;
     const int n_out_total = GATED ? half_n : N;
     const int col0 = blockIdx.x * (COLS_PER_TILE * NT);
@@ -292,6 +297,7 @@ __global__ __launch_bounds__(FQ_THREADS) void gemm_fp8_fusedq_kernel(
             for (int i = 0; i < 4; ++i)
                 if (4 * i < rows_in_block(mb)) fq_landed<YOUNGER>(xv[j][mb][i]);
 
+    PHYAI_STAMP(1)
     // ---- row scales: lane l holds the scale of "its" row and the reciprocal ----------------------------
     // own maxima: lane l <-> row l, every wavefront derives all scales from the table; handed-over maxima:
     // lanes 8 r .. 8 r + 7 of register set a <-> row 8 a + r
@@ -407,6 +413,7 @@ __global__ __launch_bounds__(FQ_THREADS) void gemm_fp8_fusedq_kernel(
         }
     }
 
+    PHYAI_STAMP(2)
     // ---- 1d. codes into the staging slice, in the layout the copies would have produced -----------
     // (all reciprocals are fetched before the first conversion, and the choice between the two
     // division forms is made once for the workgroup's rows, not per block of four rows)
@@ -448,6 +455,7 @@ __global__ __launch_bounds__(FQ_THREADS) void gemm_fp8_fusedq_kernel(
                 if (4 * i < rows_in_block(mb)) s_of[mb][i] = of_row(s_row, 2 * mb + (i >> 1), 4 * (i & 1) + xr);
         write_codes(std::false_type{});
     }
+    PHYAI_STAMP(3)
     if constexpr (!DIRECT) wait_copies<0>();   // the weights (and everything else this wavefront asked for)
 
     // ---- 2. MFMA over this wavefront's K steps -------------------------------------------------------
@@ -485,6 +493,7 @@ __global__ __launch_bounds__(FQ_THREADS) void gemm_fp8_fusedq_kernel(
     }
     // the partial sums below overwrite this wavefront's own staging: its reads must be done
     asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
+    PHYAI_STAMP(4)
 
     // AmaxOut: |bf16| bit patterns order like the values.  The maximum of a lane's outputs (two packed
     // pairs), then over the four lane groups that share a token row, then over the workgroup's tiles in LDS.
@@ -504,6 +513,7 @@ __global__ __launch_bounds__(FQ_THREADS) void gemm_fp8_fusedq_kernel(
 #pragma unroll
         for (int mb = 0; mb < MB; ++mb) red(wave, nt, mb, lane) = acc[nt][mb];
     __syncthreads();
+    PHYAI_STAMP(5)
 #pragma unroll
     for (int rr = 0; rr < ROLE_ROUNDS; ++rr) {
         if (e_nt[rr] >= NT) continue;   // wavefront-uniform: no block for this wavefront in this round
@@ -549,6 +559,7 @@ __global__ __launch_bounds__(FQ_THREADS) void gemm_fp8_fusedq_kernel(
             }
         }
     }
+    PHYAI_STAMP(6)
     if constexpr (MAKES_AMAX) {
         if (a_amax_out.table != nullptr) {
             __syncthreads();
@@ -556,6 +567,7 @@ __global__ __launch_bounds__(FQ_THREADS) void gemm_fp8_fusedq_kernel(
                 a_amax_out.table[(size_t)(m_base + tid) * kAmaxSlots + blockIdx.x] = (uint16_t)amax_made[tid];
         }
     }
+    PHYAI_STAMP_END(g_fq_stamps, ((size_t)blockIdx.x + (size_t)gridDim.x * blockIdx.y) * FQ_WAVES + wave, lane)
 }
 
 // ---- host side -------------------------------------------------------------------------------------
@@ -702,6 +714,16 @@ static int fq_launch_epi(const GemmProblem& g, const FusedPlan& pl, hipStream_t 
     case 3204: return fq_launch_kpw<32, 4, EPI>(g, pl, st);
     default: return -2;
     }
+}
+
+int launch_set_stamp_sink_fused(unsigned long long* buf, unsigned int records) {
+#ifdef PHYAI_FP8_STAMPS
+    const StampSink s = {buf, records};
+    return hipMemcpyToSymbol(HIP_SYMBOL(g_fq_stamps), &s, sizeof(s)) == hipSuccess ? 0 : -4;
+#else
+    (void)buf; (void)records;
+    return -2;
+#endif
 }
 
 int launch_gemm_fused(const GemmProblem& g, const FusedPlan& pl, hipStream_t st) {

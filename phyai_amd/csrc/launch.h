@@ -151,6 +151,10 @@ BigPlan big_plan(int M, int N, int K, int epilogue);
 size_t big_partial_bytes(int M, int N, int epilogue, const BigPlan& pl);
 int launch_gemm_big(const GemmProblem& p, const BigPlan& pl, hipStream_t st);
 
+// Debug build (-DPHYAI_FP8_STAMPS) only: where the kernels of gemm_big.hip / gemm_skinny_fused.hip write their time
+// stamps (stamps.h); -2 in the normal build.
+int launch_set_stamp_sink_big(unsigned long long* buf, unsigned int records);
+int launch_set_stamp_sink_fused(unsigned long long* buf, unsigned int records);
 // Text form of what phyai_fp8_mlp launches for aligned, row-major operands.
 int describe_mlp_plan(int M, int H, int I, int O, int epilogue, char* buf, size_t n);
 // Text form of launch_gemm's choice for aligned operands and a dense output; returns its length.

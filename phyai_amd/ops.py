@@ -602,6 +602,24 @@ def fp8_mlp(x: torch.Tensor, weight1: torch.Tensor, weight1_scale: torch.Tensor,
     return out
 
 
+STAMP_WORDS = 12
+
+
+def debug_stamps(n_records: int, device: torch.device | None = None) -> torch.Tensor | None:
+    """Debug build only (``PHYAI_FP8_LIBRARY=stamps``): from now on every wavefront of the pipelined tile kernel and
+    of the one-launch small-M kernel writes its time stamps into the returned ``[n_records, 12]`` int64 tensor (keep
+    it alive while kernels run); ``n_records = 0`` switches the recording off and returns None.  Synchronises."""
+    lib = _lib.load()
+    if n_records <= 0:
+        _lib.check(lib.phyai_fp8_debug_stamps(None, 0), "debug_stamps")
+        return None
+    dev = torch.device("cuda", torch.cuda.current_device()) if device is None else torch.device(device)
+    buf = torch.zeros(n_records, STAMP_WORDS, dtype=torch.int64, device=dev)
+    torch.cuda.synchronize()
+    _lib.check(lib.phyai_fp8_debug_stamps(buf.data_ptr(), n_records), "debug_stamps")
+    return buf
+
+
 def debug_cast_e4m3(v: torch.Tensor) -> torch.Tensor:
     """Device fp32 -> e4m3fn cast used by the quantizers, exposed for exhaustive tests."""
     if not (v.is_cuda and v.dtype == torch.float32 and v.is_contiguous()):

@@ -60,6 +60,8 @@ PAIRS = [
     ((816, 2048, 16384, None, False), (50, 1024, 4096, None, True)),
     ((200, 512, 1040, None, True), (40, 256, 528, None, False)),
     ((816, 4096, 2048, "geglu_tanh", False), (50, 8192, 1024, "geglu_tanh", False)),
+    # the one-launch kernel (quantizes its own rows: the array is not touched at all), then a smaller one
+    ((50, 2560, 1024, None, True), (16, 1024, 2048, None, False)),
 ]
 
 
@@ -78,6 +80,46 @@ def test_static_scratch_linear_equals_workspace_linear(dev, first, second):
         # and once more on the array as that call left it
         again = _static(lib, x, wq, ws, b, epi, M, N, K, n_out)
         assert torch.equal(again.view(torch.int16), want.view(torch.int16)), f"call {i} repeated: {M}x{N}x{K}"
+
+
+def test_static_scratch_linear_recorded_into_a_graph(dev):
+    """The entry point is meant for code under graph capture (its first call on a device, which looks the array's
+    address up, made outside): two calls are recorded into one graph - a split-K shape, whose recording holds the
+    kernel that clears the arrival counters, the quantizer and the GEMM on the library's own array, and a shape that
+    the one-launch kernel serves - and every replay must give the bits of phyai_fp8_linear, with eager calls that
+    use the same array between the replays."""
+    from phyai_amd import _lib
+    from phyai_amd.runtime import HipGraph
+
+    lib = _lib.load()
+    shapes = [(816, 2048, 16384, 0), (50, 2560, 1024, 0)]
+    probs, wants, outs = [], [], []
+    for i, (M, N, K, epi) in enumerate(shapes):
+        x, wq, ws, b = _problem(dev, M, N, K, seed=1234 + i, bias=True)
+        probs.append((x, wq, ws, b))
+        wants.append(_with_workspace(lib, x, wq, ws, b, epi, M, N, K, N))
+        outs.append(torch.empty(M, N, dtype=torch.bfloat16, device=dev))
+        _static(lib, x, wq, ws, b, epi, M, N, K, N)      # the call that looks the address up, outside capture
+
+    def fn():
+        st = torch.cuda.current_stream().cuda_stream
+        for (M, N, K, epi), (x, wq, ws, b), out in zip(shapes, probs, outs):
+            _lib.check(lib.phyai_fp8_linear_static(x.data_ptr(), K, wq.data_ptr(), ws.data_ptr(), b.data_ptr(), out.data_ptr(),
+                                                   N, M, N, K, epi, st), "phyai_fp8_linear_static")
+
+    g = HipGraph()
+    g.capture(fn, {})
+    for r in range(3):
+        for out in outs:
+            out.fill_(float("nan"))
+        g.replay()
+        torch.cuda.synchronize()
+        for i, (out, want) in enumerate(zip(outs, wants)):
+            assert torch.equal(out.view(torch.int16), want.view(torch.int16)), f"replay {r}, call {i}"
+        # eager work on the same array between the replays: another split-K shape leaves other codes and partial sums
+        M, N, K = 300, 384, 4096
+        x, wq, ws, b = _problem(dev, M, N, K, seed=77 + r, bias=False)
+        _static(lib, x, wq, ws, b, 0, M, N, K, N)
 
 
 def test_static_scratch_linear_refuses_what_does_not_fit(dev):
