@@ -636,12 +636,18 @@ def sweep(dev):
             wq, ws = ops.fp8_weight_quant(w)
             b = (torch.randn(N, generator=g, device=dev) * 0.01).to(torch.bfloat16) if with_bias else None
             n_out = N // 2 if gated else N
-            items.append((x.to(torch.bfloat16), wq, ws, b, torch.empty(M, n_out, dtype=torch.bfloat16, device=dev)))
+            # the layout the layers install after loading (Fp8Spec(operand_order=True)); `wp`: plain operand order
+            # for the GEMM without the activation
+            wl, lay, wp, play = wq, None, wq, None
+            if OPTS["operand"] and K % 128 == 0:
+                wp, play = ops.fp8_weight_to_operand_order(wq), "operand"
+                wl, lay = (ops.fp8_weight_to_operand_order(wq, gated=True), "operand_gated") if gated else (wp, play)
+            items.append((x.to(torch.bfloat16), wq, ws, b, torch.empty(M, n_out, dtype=torch.bfloat16, device=dev), wl, lay, wp, play))
             del w
 
         def fn():
-            for x, wq, ws, b, o in items:
-                ops.fp8_linear(x, wq, ws, b, epilogue=epi, out=o)
+            for x, _, ws, b, o, wl, lay, _, _ in items:
+                ops.fp8_linear(x, wl, ws, b, epilogue=epi, out=o, weight_layout=lay)
 
         gr = HipGraph()
         gr.capture(fn, {})
@@ -656,15 +662,15 @@ def sweep(dev):
         del gr
         # the GEMM alone (codes ready, no activation) beside torch._scaled_mm - the call the
         # reference makes (layers/linear/backends/torch.py:168-175), hipBLASLt underneath
-        pre = [(ops.fp8_quant_rowwise(x), wq, ws, b, torch.empty(M, N, dtype=torch.bfloat16, device=dev))
-               for x, wq, ws, b, _ in items]
+        pre = [(ops.fp8_quant_rowwise(x), wq, ws, b, torch.empty(M, N, dtype=torch.bfloat16, device=dev), wp, play)
+               for x, wq, ws, b, _, _, _, wp, play in items]
 
         def ours():
-            for (xq, xs), wq, ws, b, o in pre:
-                ops.fp8_gemm(xq, xs, wq, ws, b, out=o)
+            for (xq, xs), _, ws, b, o, wp, play in pre:
+                ops.fp8_gemm(xq, xs, wp, ws, b, out=o, weight_layout=play)
 
         def blaslt():
-            for (xq, xs), wq, ws, b, o in pre:
+            for (xq, xs), wq, ws, b, o, _, _ in pre:
                 torch._scaled_mm(xq, wq.t(), scale_a=xs, scale_b=ws.reshape(1, -1), bias=b, out_dtype=torch.bfloat16, out=o)
 
         for key, f in (("gemm_us", ours), ("scaled_mm_us", blaslt)):
@@ -680,6 +686,67 @@ def sweep(dev):
                 row[key] = f"unavailable: {str(e)[:80]}"
         rows.append(row)
         del items, pre
+    rows += sweep_mlp(dev)
+    return rows
+
+
+def sweep_mlp(dev):
+    """The MLP of either set as ONE call per layer (phyai_fp8_mlp: gate_up + GeGLU, then down on its output) beside the
+    sum of its two GEMMs alone on ready codes, per batch size: what the second projection's quantizer costs when its
+    row maxima come from the first projection's epilogue (M <= 128) and when it is a launch of its own."""
+    from phyai_amd import ops
+    from phyai_amd.runtime import HipGraph
+
+    rows = []
+    for set_name, shapes, m1 in (("expert", EXPERT_SET, 50), ("prefill", PREFILL_SET, 816)):
+        (_, n1, H, epi), (_, O, I, _) = shapes[2], shapes[3]
+        for B in (1, 2, 4, 8, 16):
+            M = m1 * B
+            g = torch.Generator(device=dev).manual_seed(B * 77 + n1)
+            items = []
+            for _ in range(6):
+                x = torch.randn(M, H, generator=g, device=dev).to(torch.bfloat16)
+                q1, s1 = ops.fp8_weight_quant((torch.randn(n1, H, generator=g, device=dev) * 0.02).to(torch.bfloat16))
+                q2, s2 = ops.fp8_weight_quant((torch.randn(O, I, generator=g, device=dev) * 0.02).to(torch.bfloat16))
+                p1, p2 = ops.fp8_weight_to_operand_order(q1), ops.fp8_weight_to_operand_order(q2)
+                w1, l1, w2, l2 = q1, None, q2, None
+                if OPTS["operand"]:
+                    w1, l1, w2, l2 = ops.fp8_weight_to_operand_order(q1, gated=True), "operand_gated", p2, "operand"
+                items.append(dict(x=x, w1=w1, l1=l1, s1=s1, w2=w2, l2=l2, s2=s2, p1=p1, p2=p2,
+                                  out=torch.empty(M, O, dtype=torch.bfloat16, device=dev)))
+
+            def whole():
+                for t in items:
+                    ops.fp8_mlp(t["x"], t["w1"], t["s1"], None, t["w2"], t["s2"], None, epilogue=epi, out=t["out"],
+                                weight1_layout=t["l1"], weight2_layout=t["l2"])
+
+            whole()
+            for t in items:      # ready codes of both projections' inputs, outputs of the GEMMs alone
+                t["c1"] = ops.fp8_quant_rowwise(t["x"])
+                t["c2"] = ops.fp8_quant_rowwise(torch.randn(M, I, generator=g, device=dev).to(torch.bfloat16))
+                t["o1"] = torch.empty(M, n1, dtype=torch.bfloat16, device=dev)
+
+            def alone():
+                for t in items:
+                    ops.fp8_gemm(*t["c1"], t["p1"], t["s1"], None, out=t["o1"], weight_layout="operand")
+                    ops.fp8_gemm(*t["c2"], t["p2"], t["s2"], None, out=t["out"], weight_layout="operand")
+
+            us = {}
+            for key, f in (("us", whole), ("gemm_us", alone)):
+                f()
+                torch.cuda.synchronize()
+                gr = HipGraph()
+                gr.capture(f, {})
+                ts, _ = time_replays(gr, 15, 3)
+                us[key] = round(statistics.median(ts) * 1e3 / len(items), 2)
+                del gr
+            t_hbm = (algorithmic_bytes(M, n1, H, epi, False) + algorithmic_bytes(M, O, I, None, False)) / (HBM_PEAK_GBS * 1e9) * 1e6
+            t_mfma = 2.0 * M * (n1 * H + O * I) / (FP8_PEAK_TFLOPS * 1e12) * 1e6
+            rows.append({"set": set_name, "B": B, "M": M, "shape": "mlp (gate_up + GeGLU, down)", "us": us["us"],
+                         "bound": "hbm" if t_hbm >= t_mfma else "mfma", "roofline_us": round(max(t_hbm, t_mfma), 3),
+                         "frac": round(max(t_hbm, t_mfma) / us["us"], 4), "gemm_us": us["gemm_us"], "scaled_mm_us": "-",
+                         "plan": ops.describe_mlp_plan(M, H, I, O, epi)})
+            del items
     return rows
 
 
@@ -904,7 +971,8 @@ def main() -> int:
     OPTS["operand"] = not args.row_major
     OPTS["mlp"] = not args.separate_linears
     if args.stamps:
-        os.environ["PHYAI_FP8_LIBRARY"] = "stamps"   # before the library is opened
+        if os.environ.get("PHYAI_FP8_LIBRARY") != "ablate":   # (`make ablate ABLATE=n`: the same table with parts of a main loop left out)
+            os.environ["PHYAI_FP8_LIBRARY"] = "stamps"        # before the library is opened
     if args.gpus != 1 or int(os.environ.get("WORLD_SIZE", "1")) != 1:
         print("bench.py: this path is built and measured on ONE GPU (TP=1, no collectives); "
               "run with --gpus 1", file=sys.stderr)
@@ -1075,6 +1143,12 @@ def main() -> int:
                     "residuals, final norm, projection, Euler update; data chains through the 18 layers"}
     if args.sweep:
         extra["batched_sweep"] = sweep(dev)
+        # the same rows as a markdown table, on stderr (stdout carries the one JSON line)
+        print("| set | B | M | shape | us per linear | bound | roofline us | fraction | GEMM alone us | torch._scaled_mm us |", file=sys.stderr)
+        print("|---|---|---|---|---|---|---|---|---|---|", file=sys.stderr)
+        for r in extra["batched_sweep"]:
+            print(f"| {r['set']} | {r['B']} | {r['M']} | {r['shape']} | {r['us']} | {r['bound']} | {r['roofline_us']} | {r['frac']} | "
+                  f"{r.get('gemm_us', '-')} | {r.get('scaled_mm_us', '-')} |", file=sys.stderr)
 
     cpu = None
     if not args.no_cpu_baseline:

@@ -14,7 +14,10 @@ _PKG = os.path.dirname(os.path.abspath(__file__))
 # PHYAI_FP8_LIBRARY=stamps (set before the first call) makes the whole process use the debug build whose GEMM
 # kernels record time stamps of their phases (`make -C phyai_amd/csrc stamps`): same entry points, same results.
 STAMPS_LIB_PATH = os.path.join(_PKG, "lib", "libphyai_fp8_stamps.so")
-LIB_PATH = STAMPS_LIB_PATH if os.environ.get("PHYAI_FP8_LIBRARY") == "stamps" else os.path.join(_PKG, "lib", "libphyai_fp8.so")
+# PHYAI_FP8_LIBRARY=ablate: the time-stamp build with parts of a kernel's main loop left out (`make ablate ABLATE=n`),
+# for measurements only - its results are wrong by design.
+LIB_PATH = {"stamps": STAMPS_LIB_PATH, "ablate": os.path.join(_PKG, "lib", "libphyai_fp8_ablate.so")}.get(
+    os.environ.get("PHYAI_FP8_LIBRARY", ""), os.path.join(_PKG, "lib", "libphyai_fp8.so"))
 CSRC_DIR = os.path.join(_PKG, "csrc")
 ABI_VERSION = 8
 

@@ -54,6 +54,16 @@
 namespace phyai {
 
 constexpr int BIG_BK = 128;   // bytes of K per LDS row: one L2 cache line
+// Measurement only (make stamps ABLATE=n builds the time-stamp library with it; results are WRONG by design): parts
+// of the main loop left out, to see from the time stamps what each costs.  Bit 1: no copies / weight loads inside
+// the loop (the operands of the prologue are multiplied over and over); bit 2: the activation blocks of a K half
+// are not re-read from LDS; bit 4: no barrier in the loop of the variant that loads its weights into registers.
+#ifndef PHYAI_FP8_ABLATE
+#define PHYAI_FP8_ABLATE 0
+#endif
+#if PHYAI_FP8_ABLATE && !defined(PHYAI_FP8_STAMPS)
+#error "PHYAI_FP8_ABLATE is for the time-stamp build only"
+#endif
 // (debug build only: where the kernels below leave their time stamps - 1 first stage published, 2 main loop done,
 // 3 split-K sums gathered, 4 epilogue arithmetic done and tile staged, 5 stores issued)
 PHYAI_STAMP_SINK(g_big_stamps)
@@ -381,7 +391,7 @@ void gemm_fp8_big_kernel(
         _Pragma("unroll") for (int i_ = 0; i_ < TM; ++i_) {                                                    \
             if (!A_AHEAD && i_ == 0) {                                                                         \
                 _Pragma("unroll") for (int a_ = 1; a_ < TM; ++a_)                                              \
-                    fa_[a_] = big_frag(abuf_, arow + a_ * 32, h, KH);                                          \
+                    fa_[a_] = (PHYAI_FP8_ABLATE & 2) ? fa_[0] : big_frag(abuf_, arow + a_ * 32, h, KH);        \
             }                                                                                                  \
             if (i_ >= 1 && (NEXT)) {                                                                           \
                 /* item 0: B0; items 1..NA: the A blocks; then B1..: spread over row groups 1..TM-1 */         \
@@ -406,7 +416,7 @@ void gemm_fp8_big_kernel(
                 acc[i_][j_] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(fb_, fa_[i_], acc[i_][j_],       \
                                                                                0, 0, 0, 0, 0, 0);              \
                 _Pragma("unroll") for (int c_ = 0; c_ < CPS; ++c_)                                             \
-                    if (req_ && (slot0_ + j_) * CPS + c_ < IDX_END) {                                          \
+                    if (req_ && (slot0_ + j_) * CPS + c_ < IDX_END && !(PHYAI_FP8_ABLATE & 1)) {               \
                         /* (register set of the load: its number modulo DEPTH) */                              \
                         if (after_) issue(load_, (slot0_ + j_) * CPS + c_, std::integral_constant<int, ((SLOT) + LEAD) % DEPTH>{});     \
                         else issue(load_, (slot0_ + j_) * CPS + c_, std::integral_constant<int, ((SLOT) + LEAD - 1) % DEPTH>{}); \
@@ -416,7 +426,7 @@ void gemm_fp8_big_kernel(
             if ((KH) == 1 && i_ == 0 && (NEXT)) {                                                              \
                 if constexpr (BDIRECT) {                                                                       \
                     wait_copies<COPIES * (AHEAD)>();               /* my requests of D+1 have landed ... */    \
-                    __builtin_amdgcn_s_barrier();                  /* ... and so have everybody's */           \
+                    if (!(PHYAI_FP8_ABLATE & 4)) __builtin_amdgcn_s_barrier(); /* ... and so have everybody's */ \
                     asm volatile("" ::: "memory");                                                             \
                 } else {                                                                                       \
                     asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory"); /* my reads of stage-load D have landed */ \

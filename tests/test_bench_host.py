@@ -25,9 +25,10 @@ def test_reported_traffic_is_the_profiled_figure():
         cells = [c.strip() for c in ln.strip("|").split("|")]
         total_mb += float(cells[2]) + float(cells[4])       # fetched MB (calibrated) + written MB
     assert abs(got - total_mb * 1e6) <= 0.02e6, (got, total_mb)
-    # more than the algorithmic bytes of the layer (token rows are fetched once per XCD), but not by much
+    # more than the algorithmic bytes of the layer (bf16 token rows are fetched once per XCD, i.e. eight times:
+    # 0.8 - 3.3 MB per linear beside 2.6 - 8.4 MB of weights), but not by much
     algorithmic = sum(bench.algorithmic_bytes(50, N, K, epi) for _, N, K, epi in bench.EXPERT_SET)
-    assert algorithmic == 19_042_304 and algorithmic < got < 1.3 * algorithmic
+    assert algorithmic == 19_042_304 and algorithmic < got < 1.35 * algorithmic
 
 
 def test_cpu_description():
