@@ -154,8 +154,9 @@ int phyai_fp8_gemm(const void *xq, const float *x_scale, int x_scale_is_scalar,
  * GEMM above, as one call.  Replaces TorchKernel._fp8_per_channel
  * (layers/linear/backends/torch.py:155-176) end to end.
  *
- * Up to 128 token rows, K <= 2048 (a multiple of 128), with x and its row stride 16-byte
- * aligned and a grid that fits the chip at once, this is ONE kernel: every workgroup
+ * Up to 128 token rows, K <= 4096 (a multiple of 128), with x and its row stride 16-byte
+ * aligned and a workgroup shape whose grid fits the chip at once (beyond K = 2048: projections up to
+ * about 2048 wide), this is ONE kernel: every workgroup
  * quantizes the token rows it multiplies (same codes, same scales, same output bits as
  * the two launches) and the workspace is not touched: such a call may pass workspace = NULL.
  * Otherwise the quantizer writes codes and scales into the workspace and a GEMM kernel follows
@@ -214,7 +215,8 @@ int phyai_fp8_mlp(const void *x, int64_t ldx, const void *w1, const float *w1_sc
                   int64_t gate_rows, void *out, int64_t ldo, int64_t M, int64_t H, int64_t I,
                   int64_t O, int epilogue, void *workspace, size_t workspace_bytes, void *stream);
 /* "row maxima handed over: <first> | <second>" or "<first> | <second>", each part as
- * phyai_fp8_describe_linear_plan reports it (row-major weights; host only). */
+ * phyai_fp8_describe_linear_plan reports it.  Host only.  Row-major weights, or - with
+ * PHYAI_FP8_FLAG_W_OPERAND_ORDER or-ed into `epilogue` - both matrices in operand order. */
 int phyai_fp8_describe_mlp_plan(int64_t M, int64_t H, int64_t I, int64_t O, int epilogue, char *buf,
                                 size_t n);
 
@@ -283,7 +285,9 @@ int phyai_fp8_describe_plan(int64_t M, int64_t N, int64_t K, int epilogue, char 
 /*
  * The same for phyai_fp8_linear (bf16 activations in, dense rows): either
  *   "one launch: small-m rows=8 nt=5 kpw=1 grid=32x7"      the kernel that quantizes its own token rows
- * or "quantizer + " followed by what phyai_fp8_describe_plan reports.  Host only.
+ * or "quantizer + " followed by what phyai_fp8_describe_plan reports.  Host only.  The layout flag of
+ * the weight matrix (PHYAI_FP8_FLAG_W_OPERAND_ORDER / _GATED) may be or-ed into `epilogue` as in the
+ * calls: a few shapes are one launch only with weights in operand order (registers instead of LDS).
  */
 int phyai_fp8_describe_linear_plan(int64_t M, int64_t N, int64_t K, int epilogue, char *buf, size_t n);
 

@@ -556,11 +556,17 @@ int phyai_fp8_describe_linear_plan(int64_t M, int64_t N, int64_t K, int epilogue
     buf[0] = 0;
     if (M < 0 || N <= 0 || K <= 0 || M >= kMaxElems || N >= kMaxElems || K >= kMaxElems)
         return fail(PHYAI_FP8_EINVAL, "phyai_fp8_describe_linear_plan: bad shape M=%lld N=%lld K=%lld", (long long)M, (long long)N, (long long)K);
+    const int layout_bits = epilogue & PHYAI_FP8_FLAG_W_OPERAND_GATED;
     epilogue &= PHYAI_FP8_EPILOGUE_MASK;
     if (int rc = check_epilogue(epilogue, N)) return rc;
     if (K % 16 != 0 || N % 16 != 0)
         return fail(PHYAI_FP8_EUNSUPPORTED, "phyai_fp8_describe_linear_plan: K=%lld and N=%lld must be multiples of 16", (long long)K, (long long)N);
-    const int len = phyai::describe_linear_plan((int)M, (int)N, (int)K, epilogue, buf, n);
+    // (the layout flags of the weight matrix may ride in `epilogue` as in the calls; a layout that the calls would
+    // refuse for this shape or epilogue is described as row-major)
+    int layout = phyai::W_ROW_MAJOR;
+    if (layout_bits && K % 128 == 0 && N % (phyai::epi_is_gated(epilogue) ? 32 : 16) == 0)
+        layout = phyai::epi_is_gated(epilogue) ? phyai::W_OPERAND_GATED : phyai::W_OPERAND_PLAIN;
+    const int len = phyai::describe_linear_plan((int)M, (int)N, (int)K, epilogue, buf, n, layout);
     buf[n - 1] = 0;
     return len;
 }
@@ -571,13 +577,15 @@ int phyai_fp8_describe_mlp_plan(int64_t M, int64_t H, int64_t I, int64_t O, int 
     buf[0] = 0;
     if (M < 0 || H <= 0 || I <= 0 || O <= 0 || M >= kMaxElems || H >= kMaxElems || I >= kMaxElems || O >= kMaxElems)
         return fail(PHYAI_FP8_EINVAL, "%s: bad shape", fn);
+    const bool operand = (epilogue & PHYAI_FP8_FLAG_W_OPERAND_ORDER) != 0 && H % 128 == 0 && I % 128 == 0;
+    epilogue &= ~PHYAI_FP8_FLAG_W_OPERAND_GATED;
     if (epilogue <= PHYAI_FP8_EPI_NONE || epilogue > PHYAI_FP8_EPI_GELU_ERF)
         return fail(PHYAI_FP8_EINVAL, "%s: epilogue %d is not an activation", fn, epilogue);
     const int64_t n1 = phyai::epi_is_gated(epilogue) ? 2 * I : I;
     if (int rc = check_epilogue(epilogue, n1)) return rc;
     if (H % 16 != 0 || I % 16 != 0 || O % 16 != 0)
         return fail(PHYAI_FP8_EUNSUPPORTED, "%s: H, I and O must be multiples of 16", fn);
-    const int len = phyai::describe_mlp_plan((int)M, (int)H, (int)I, (int)O, epilogue, buf, n);
+    const int len = phyai::describe_mlp_plan((int)M, (int)H, (int)I, (int)O, epilogue, buf, n, operand);
     buf[n - 1] = 0;
     return len;
 }

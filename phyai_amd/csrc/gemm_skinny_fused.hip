@@ -193,8 +193,10 @@ __global__ __launch_bounds__(FQ_THREADS) void gemm_fp8_fusedq_kernel(
     // behind the 16 KB of weights of each earlier one - the rows, not the weights, are what the workgroup
     // waits for first.  (A bare barrier: nothing is awaited, only the order of issue is fixed.)  Measured:
     // o 2048 -> 1024 at M = 50 4.54 -> 4.32 us; with one K step per wavefront (K = 1024) the later start
-    // of the weight requests costs as much as the rows gain (gate_up 6.33 -> 6.41 us), so only K > 1024.
-    if constexpr (KPW >= 2) __builtin_amdgcn_s_barrier();
+    // of the weight requests costs as much as the rows gain when the weights are staged through LDS (gate_up
+    // 6.33 -> 6.41 us), so only K > 1024 there; with weights straight into registers it is level or 0.05 us
+    // ahead at K = 1024 too (qkv 3.62 -> 3.57 us, gate_up 5.71 -> 5.65 us).
+    if constexpr (KPW >= 2 || DIRECT) __builtin_amdgcn_s_barrier();
     // ---- 1b. the weights of the same K steps: into registers, or global -> LDS (as in gemm_skinny.hip) --
     const uint32_t lds_wave = __builtin_amdgcn_readfirstlane((uint32_t)(uintptr_t)smem + wave * PER_WAVE);
     uint8_t* my_stage = smem + wave * PER_WAVE;
@@ -592,12 +594,7 @@ static constexpr bool fq_regs_ok(int rows, int nt, int kpw, bool direct) {
     return !direct || kpw * nt * 8 + kpw * ((rows + 3) / 4) * 4 <= 160;
 }
 
-// Shapes that exist as kernels: (rows, nt) below, with kpw = 1, 2 or 4 as K asks.
-// Beyond K = 2048 only the 16 x 16 shape fits the LDS and every workgroup would pull eight times the
-// bf16 rows it has weights for: measured 7.7 us against 6.6 us for quantizer + GEMM at 50 x 1024 x 4096.
-// (The kernels with four K steps per wavefront stay compiled: the plan can be forced for tests, and with
-// handed-over row maxima they are what the down projection of an MLP runs.)
-static const int kFusedMaxK = 2048;
+// Shapes that exist as kernels: (rows, nt) below, with kpw = 1, 2 or 4 as K asks (K <= 4096).
 // Up to 128 token rows the kernel is level with or ahead of quantizer + GEMM as long as a workgroup
 // converts 16 rows or fewer (measured at M = 64 ... 256 on the expert shapes: 32-row workgroups lose).
 static const int kFusedMaxM = 128;
@@ -628,13 +625,16 @@ FusedPlan fused_plan(int M, int N, int K, int epilogue, int64_t ldo, int weight_
     double best = 1e30;
     int forced_rows = 0, forced_nt = 0;
     if (const char* e = tuning_env(amax_in ? "PHYAI_FP8_FUSED_PLAN_AMAX" : "PHYAI_FP8_FUSED_PLAN")) sscanf(e, "%d,%d", &forced_rows, &forced_nt);
-    // beyond K = 2048 the kernel pays only when the row maxima are handed over (no pass over the rows
-    // before the conversions) - or when a test forces it
-    if (K > kFusedMaxK && !forced_rows && !amax_in) return pl;
+    // Beyond K = 2048 (four K steps per wavefront) a kernel that finds its own row maxima is taken only in the
+    // 8 rows x 2 tiles shape.  Measured on whole linears against quantizer + GEMM over M = 1 ... 128,
+    // N = 256 ... 2048, K = 2560 / 3072 / 4096: that shape is 4 - 16 % ahead with weights in operand order
+    // (50 x 1024 x 4096: 6.8 -> 6.1 us) and 0 - 13 % ahead row-major; 8 rows x 4 tiles is level (0.96 - 1.05).
+    const bool long_k_alone = K > 2048 && !amax_in && !forced_rows;
     for (const auto& sh : kFusedShapes) {
         const int rows = sh[0], nt = sh[1];
         if (!fq_fits(rows, nt, kpw, direct, amax_in, epilogue != EPI_NONE) || !fq_regs_ok(rows, nt, kpw, direct)) continue;
         if (amax_in && !fq_amax_in_shape(rows, nt)) continue;
+        if (long_k_alone && (rows != 8 || nt != 2)) continue;
         if (forced_rows && (rows != forced_rows || nt != forced_nt)) continue;
         const int tiles = fq_ceil_div(cols, per_tile * nt), msplit = fq_ceil_div(M, rows);
         if (!forced_rows) {

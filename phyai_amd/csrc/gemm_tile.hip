@@ -464,9 +464,9 @@ int describe_gemm_plan(int M, int N, int K, int epilogue, char* buf, size_t n) {
     }
 }
 
-int describe_linear_plan(int M, int N, int K, int epilogue, char* buf, size_t n) {
+int describe_linear_plan(int M, int N, int K, int epilogue, char* buf, size_t n, int weight_layout) {
     const int64_t ldo = epi_is_gated(epilogue) ? N / 2 : N;
-    const GemmChoice c = choose_gemm(M, N, K, epilogue, ldo, true, ldo % 8 == 0, true);
+    const GemmChoice c = choose_gemm(M, N, K, epilogue, ldo, true, ldo % 8 == 0, true, weight_layout);
     if (c.kind == GemmChoice::FUSED)
         return snprintf(buf, n, "one launch: small-m rows=%d nt=%d kpw=%d grid=%dx%d", c.fq.rows, c.fq.nt, c.fq.kpw, c.fq.tiles, c.fq.msplit);
     const int len = snprintf(buf, n, "quantizer + ");
@@ -474,26 +474,28 @@ int describe_linear_plan(int M, int N, int K, int epilogue, char* buf, size_t n)
     return len + describe_gemm_plan(M, N, K, epilogue, buf + len, n - len);
 }
 
-int describe_mlp_plan(int M, int H, int I, int O, int epilogue, char* buf, size_t n) {
+int describe_mlp_plan(int M, int H, int I, int O, int epilogue, char* buf, size_t n, bool operand_order) {
     const int n1 = epi_is_gated(epilogue) ? 2 * I : I;
-    const GemmChoice a = choose_gemm(M, n1, H, epilogue, I, true, I % 8 == 0, true);
+    const int lay1 = !operand_order ? W_ROW_MAJOR : (epi_is_gated(epilogue) ? W_OPERAND_GATED : W_OPERAND_PLAIN);
+    const int lay2 = operand_order ? W_OPERAND_PLAIN : W_ROW_MAJOR;
+    const GemmChoice a = choose_gemm(M, n1, H, epilogue, I, true, I % 8 == 0, true, lay1);
     bool handed = false;
     if (a.kind == GemmChoice::FUSED && a.fq.tiles <= kRowAmaxSlots) {
-        const GemmChoice b = choose_gemm(M, O, I, EPI_NONE, O, true, O % 8 == 0, true, W_ROW_MAJOR, true);
+        const GemmChoice b = choose_gemm(M, O, I, EPI_NONE, O, true, O % 8 == 0, true, lay2, true);
         handed = b.kind == GemmChoice::FUSED && b.takes_amax;
     }
     int len = handed ? snprintf(buf, n, "row maxima handed over: ") : 0;
     if (len < 0 || (size_t)len >= n) return len;
-    len += describe_linear_plan(M, n1, H, epilogue, buf + len, n - len);
+    len += describe_linear_plan(M, n1, H, epilogue, buf + len, n - len, lay1);
     if ((size_t)len >= n) return len;
     len += snprintf(buf + len, n - len, " | ");
     if ((size_t)len >= n) return len;
     if (handed) {
-        const GemmChoice b = choose_gemm(M, O, I, EPI_NONE, O, true, O % 8 == 0, true, W_ROW_MAJOR, true);
+        const GemmChoice b = choose_gemm(M, O, I, EPI_NONE, O, true, O % 8 == 0, true, lay2, true);
         return len + snprintf(buf + len, n - len, "one launch: small-m rows=%d nt=%d kpw=%d grid=%dx%d", b.fq.rows, b.fq.nt,
                               b.fq.kpw, b.fq.tiles, b.fq.msplit);
     }
-    return len + describe_linear_plan(M, O, I, EPI_NONE, buf + len, n - len);
+    return len + describe_linear_plan(M, O, I, EPI_NONE, buf + len, n - len, lay2);
 }
 
 int launch_gemm(const GemmProblem& g, hipStream_t st) {

@@ -110,7 +110,7 @@ bool gemm_quantizes_itself(const GemmProblem& p);
 int gemm_row_maxima_slots(const GemmProblem& p);
 bool gemm_takes_row_maxima(const GemmProblem& p);
 // Text form of the whole-linear choice for aligned operands and dense activations / output.
-int describe_linear_plan(int M, int N, int K, int epilogue, char* buf, size_t n);
+int describe_linear_plan(int M, int N, int K, int epilogue, char* buf, size_t n, int weight_layout = 0);
 
 // Weight-streaming kernel for M <= 64 (gemm_skinny.hip).  It needs no workspace.
 struct SkinnyPlan {
@@ -156,7 +156,7 @@ int launch_gemm_big(const GemmProblem& p, const BigPlan& pl, hipStream_t st);
 int launch_set_stamp_sink_big(unsigned long long* buf, unsigned int records);
 int launch_set_stamp_sink_fused(unsigned long long* buf, unsigned int records);
 // Text form of what phyai_fp8_mlp launches for aligned, row-major operands.
-int describe_mlp_plan(int M, int H, int I, int O, int epilogue, char* buf, size_t n);
+int describe_mlp_plan(int M, int H, int I, int O, int epilogue, char* buf, size_t n, bool operand_order = false);
 // Text form of launch_gemm's choice for aligned operands and a dense output; returns its length.
 int describe_gemm_plan(int M, int N, int K, int epilogue, char* buf, size_t n);
 

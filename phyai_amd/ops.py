@@ -123,13 +123,15 @@ def describe_plan(M: int, N: int, K: int, epilogue=EPI_NONE) -> str:
     return buf.value.decode()
 
 
-def describe_linear_plan(M: int, N: int, K: int, epilogue=EPI_NONE) -> str:
+def describe_linear_plan(M: int, N: int, K: int, epilogue=EPI_NONE, weight_layout: str | None = None) -> str:
     """What the whole-linear entry point would launch (one kernel that quantizes its own rows, or the
-    quantizer followed by a GEMM); host only."""
+    quantizer followed by a GEMM) for a weight in the given layout; host only."""
     import ctypes
 
     buf = ctypes.create_string_buffer(160)
-    rc = _lib.load().phyai_fp8_describe_linear_plan(M, N, K, _epi("describe_linear_plan", epilogue), buf, len(buf))
+    epi = _epi("describe_linear_plan", epilogue)
+    flag = _layout_flag("describe_linear_plan", weight_layout, epi) if weight_layout else 0
+    rc = _lib.load().phyai_fp8_describe_linear_plan(M, N, K, epi | flag, buf, len(buf))
     if rc < 0:
         raise _err("describe_linear_plan", _lib.load().phyai_fp8_last_error().decode())
     return buf.value.decode()
@@ -548,12 +550,14 @@ def fp8_linear(x: torch.Tensor, weight: torch.Tensor, weight_scale: torch.Tensor
     return out
 
 
-def describe_mlp_plan(M: int, H: int, I: int, O: int, epilogue) -> str:
-    """What :func:`fp8_mlp` launches for this shape (row-major weights; host only)."""
+def describe_mlp_plan(M: int, H: int, I: int, O: int, epilogue, operand_order: bool = False) -> str:
+    """What :func:`fp8_mlp` launches for this shape, with row-major weights or with both matrices in operand
+    order; host only."""
     import ctypes
 
     buf = ctypes.create_string_buffer(256)
-    rc = _lib.load().phyai_fp8_describe_mlp_plan(M, H, I, O, _epi("describe_mlp_plan", epilogue), buf, len(buf))
+    epi = _epi("describe_mlp_plan", epilogue) | (FLAG_W_OPERAND_ORDER if operand_order else 0)
+    rc = _lib.load().phyai_fp8_describe_mlp_plan(M, H, I, O, epi, buf, len(buf))
     if rc < 0:
         raise _err("describe_mlp_plan", _lib.load().phyai_fp8_last_error().decode())
     return buf.value.decode()

@@ -130,7 +130,7 @@ def test_kernel_selection_for_the_benchmark_shapes(monkeypatch):
 
 def test_whole_linear_selection_one_launch_or_two(monkeypatch):
     """phyai_fp8_linear runs one kernel that quantizes its own token rows where that was measured
-    faster (up to 128 rows, K <= 2048, a grid of at most 256 workgroups), and quantizer + GEMM
+    faster (up to 128 rows, K <= 4096, a grid of at most 256 workgroups), and quantizer + GEMM
     elsewhere.  Host only."""
     from phyai_amd import ops
 
@@ -142,7 +142,10 @@ def test_whole_linear_selection_one_launch_or_two(monkeypatch):
     assert d(50, 8192, 1024, "geglu_tanh") == "one launch: small-m rows=16 nt=8 kpw=1 grid=64x4"
     assert d(50, 4096, 1024) == "one launch: small-m rows=16 nt=4 kpw=1 grid=64x4"
     assert d(1, 2048, 2048) == "one launch: small-m rows=8 nt=2 kpw=2 grid=64x1"
-    assert d(50, 1024, 4096) == "quantizer + small-m nt=1 mb=1 kpw=4 rounds=1"       # K too long for the LDS
+    assert d(50, 1024, 4096) == "one launch: small-m rows=8 nt=2 kpw=4 grid=32x7"      # four K steps per wavefront: 8 x 2 only
+    assert d(50, 2048, 4096).startswith("quantizer + small-m")                          # ... whose grid must fit one round
+    assert d(50, 2048, 4096, weight_layout="operand").startswith("quantizer + small-m")
+    assert d(50, 1024, 4224).startswith("quantizer + ")                                 # K beyond 4096
     assert d(50, 12288, 2048).startswith("quantizer + small-m")                       # more than one round of workgroups
     assert d(100, 2560, 1024) == "one launch: small-m rows=16 nt=8 kpw=1 grid=20x7"   # up to 128 rows, 16 per workgroup
     assert d(100, 8192, 1024, "geglu_tanh").startswith("quantizer + small-m")          # 16-row workgroups would need two rounds
