@@ -57,7 +57,8 @@ constexpr int BIG_BK = 128;   // bytes of K per LDS row: one L2 cache line
 // Measurement only (make stamps ABLATE=n builds the time-stamp library with it; results are WRONG by design): parts
 // of the main loop left out, to see from the time stamps what each costs.  Bit 1: no copies / weight loads inside
 // the loop (the operands of the prologue are multiplied over and over); bit 2: the activation blocks of a K half
-// are not re-read from LDS; bit 4: no barrier in the loop of the variant that loads its weights into registers.
+// are not re-read from LDS; bit 4: no barrier in the loop of the variant that loads its weights into registers;
+// bits 8 / 16 (that variant): only the weight loads / only the activation copies of the loop are left out.
 #ifndef PHYAI_FP8_ABLATE
 #define PHYAI_FP8_ABLATE 0
 #endif
@@ -338,9 +339,10 @@ void gemm_fp8_big_kernel(
         const int k = k_begin + d * BIG_BK;
         const uint32_t stage_off = (d % DEPTH) * STAGE_BYTES;
         if (c < CA) {
-            copy16_to_lds(p.a + k, aoff[c], wave_a + stage_off + c * 1024);
+            if (!(PHYAI_FP8_ABLATE & 16) || d < LEAD) copy16_to_lds(p.a + k, aoff[c], wave_a + stage_off + c * 1024);
         } else if constexpr (BDIRECT) {
             constexpr int S = decltype(slot)::value;
+            if ((PHYAI_FP8_ABLATE & 8) && d >= LEAD) return;
             const int e = c - CA, j = e >> 2, kh = (e >> 1) & 1, pr = e & 1;   // chunk 4 kh + 2 pr + h of block j
             bring[S][j][kh][pr] = *reinterpret_cast<const v4i*>(bsrc[j] + ((size_t)d << 11) + (4 * kh + 2 * pr) * 256);
         } else {
