@@ -146,6 +146,17 @@ def test_whole_linear_selection_one_launch_or_two(monkeypatch):
     assert d(50, 2048, 4096).startswith("quantizer + small-m")                          # ... whose grid must fit one round
     assert d(50, 2048, 4096, weight_layout="operand").startswith("quantizer + small-m")
     assert d(50, 1024, 4224).startswith("quantizer + ")                                 # K beyond 4096
+    # the layout of the weight matrix is part of the question: with weights straight into registers more shapes fit
+    assert d(50, 8192, 2048, "geglu_tanh").startswith("quantizer + ")
+    assert d(50, 8192, 2048, "geglu_tanh", weight_layout="operand_gated") == "one launch: small-m rows=16 nt=8 kpw=2 grid=64x4"
+    with pytest.raises(RuntimeError, match="does not go with"):
+        d(50, 8192, 2048, "geglu_tanh", weight_layout="operand")
+    m = ops.describe_mlp_plan
+    assert m(50, 1024, 4096, 1024, "geglu_tanh") == ("row maxima handed over: one launch: small-m rows=16 nt=8 kpw=1 grid=64x4 | "
+                                                     "one launch: small-m rows=8 nt=2 kpw=4 grid=32x7")
+    assert m(50, 1024, 4096, 1024, "geglu_tanh", operand_order=True) == m(50, 1024, 4096, 1024, "geglu_tanh")
+    assert not m(50, 2048, 8192, 2048, "geglu_tanh").startswith("row maxima")
+    assert m(200, 1024, 4096, 1024, "geglu_tanh").count("quantizer + ") == 2
     assert d(50, 12288, 2048).startswith("quantizer + small-m")                       # more than one round of workgroups
     assert d(100, 2560, 1024) == "one launch: small-m rows=16 nt=8 kpw=1 grid=20x7"   # up to 128 rows, 16 per workgroup
     assert d(100, 8192, 1024, "geglu_tanh").startswith("quantizer + small-m")          # 16-row workgroups would need two rounds
