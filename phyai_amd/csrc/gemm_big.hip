@@ -525,14 +525,27 @@ void gemm_fp8_big_kernel(
         if (!splitk_arrive(p.counters, tile, S, reinterpret_cast<int*>(lds))) return;
         // gather: as much of the fragment per round trip as the registers allow
         constexpr int GCH = FRAG <= 64 ? FRAG : 32;
+        if (S == 2) {   // (uniform) the own half is still in the accumulators: only the other one is read
 #pragma unroll
-        for (int c = 0; c < FRAG / GCH; ++c) {
-            float frag[GCH];
-            splitk_gather_part<FRAG, 256, GCH>(p.partials, tile, S, c * GCH, frag);
+            for (int c = 0; c < FRAG / GCH; ++c) {
+                float frag[GCH];
+                splitk_load_part<FRAG, 256, GCH>(p.partials, tile, 2, 1 - split_z, c * GCH, frag);
 #pragma unroll
-            for (int r = 0; r < GCH; ++r) {
-                const int blk = (c * GCH + r) / 16;
-                acc[blk / TN][blk % TN][r % 16] = frag[r];
+                for (int r = 0; r < GCH; ++r) {
+                    const int blk = (c * GCH + r) / 16;
+                    acc[blk / TN][blk % TN][r % 16] += frag[r];
+                }
+            }
+        } else {
+#pragma unroll
+            for (int c = 0; c < FRAG / GCH; ++c) {
+                float frag[GCH];
+                splitk_gather_part<FRAG, 256, GCH>(p.partials, tile, S, c * GCH, frag);
+#pragma unroll
+                for (int r = 0; r < GCH; ++r) {
+                    const int blk = (c * GCH + r) / 16;
+                    acc[blk / TN][blk % TN][r % 16] = frag[r];
+                }
             }
         }
         splitk_reset(p.counters, tile);

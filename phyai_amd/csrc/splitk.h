@@ -114,6 +114,17 @@ __device__ __forceinline__ void splitk_gather_part(const float* partials, int ti
     }
 }
 
+// Elements e0 .. e0+CHUNK-1 of ONE split's partial (for a tile split in two, whose last arriver still holds its
+// own half in registers: own + other is the sum in split order whichever half is its own, since a + b = b + a and
+// the sum of the general form starts from 0 + a = a).
+template <int FRAG, int THREADS, int CHUNK>
+__device__ __forceinline__ void splitk_load_part(const float* partials, int tile, int S, int z, int e0, float* frag) {
+    const float* one = partials + ((size_t)tile * S + z) * (size_t)(FRAG * THREADS);
+#pragma unroll
+    for (int e = 0; e < CHUNK; e += 2)
+        coherent_load2(one + (((e0 + e) / 2) * THREADS + threadIdx.x) * 2, frag[e], frag[e + 1]);
+}
+
 // The gathering workgroup puts the tile's counter back to zero for the next call.
 __device__ __forceinline__ void splitk_reset(int* counters, int tile) {
     if (threadIdx.x == 0)
