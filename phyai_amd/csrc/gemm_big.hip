@@ -235,8 +235,8 @@ void gemm_fp8_big_kernel(
     constexpr int LATE = (TM - 1) * TN * CPS;        // first request number that falls into the next stage
     constexpr int IDX_END = COPIES;
     static_assert(!BDIRECT || COPIES <= LATE, "with weights in registers every request goes out behind the barrier");
-    static_assert((TM == TN && TM % 2 == 0) || (TM == 3 && TN == 2) || (TM == 7 && TN == 2) || (TM == 2 && TN == 1 && !GATED),
-                  "supported wavefront tiles");
+    static_assert((TM == TN && TM % 2 == 0) || (TM == 3 && TN == 2) || (TM == 7 && TN == 2) || (TM == 2 && TN == 1 && !GATED) ||
+                  (TM == 3 && TN == 1 && !GATED), "supported wavefront tiles");
     static_assert(BM % 32 == 0 && BN % 32 == 0, "every wavefront copies whole groups of 8 rows");
     static_assert(DEPTH == 2 || DEPTH == 4, "ring depth");
     // (the epilogue stages the bf16 tile in the same LDS; where the ring is smaller than that, the ring grows)
@@ -743,8 +743,9 @@ BigPlan big_plan(int M, int N, int K, int epilogue) {
     int forced = -1;
     if (const char* e = tuning_env("PHYAI_FP8_BIG")) forced = atoi(e);   // "0": never; "256"/"192"/"128": force
     if (forced == 0) return pl;
-    if (forced == 256 || forced == 224 || forced == 192 || forced == 128) pl.tile = forced;
+    if (forced == 256 || forced == 224 || forced == 192 || forced == 128) pl.tile = forced;   // ("96": 96 x 128, below)
     else if (forced == 12864 && !epi_is_gated(epilogue)) { pl.tile = 128; pl.cols = 64; }   // "12864": 128 rows x 64 columns
+    else if (forced == 96 && !epi_is_gated(epilogue)) { pl.tile = 96; pl.cols = 128; }
     else if (M < 128) return pl;
     // 256 x 256 tiles need the fewest bytes from L2 per flop but run one workgroup per CU, so a
     // tile's prologue and epilogue leave the MFMA pipe idle; 192 x 128 tiles fit twice and overlap
@@ -784,9 +785,20 @@ BigPlan big_plan(int M, int N, int K, int epilogue) {
         pl.cols = 64;
         tiles = big_tiles(M, N, epilogue, 128, 64);
     }
+    // Between 129 and 255 tiles of 128 x 128 (and a plain epilogue) 96 x 128 tiles - wavefronts 1 x 4, three row
+    // blocks each - put up to 256 CUs to work in one round where the 128-row grid leaves a fifth to a half of them
+    // idle and 128 x 64 tiles would need a second round: 8 - 11 % faster on every shape measured (weights from HBM,
+    // 12 - 18 weight sets): 816 x 2560 x 2048 (140 -> 180 tiles) 11.2 -> 9.95 us, 816 x 3072 x 2048 11.2 -> 10.1,
+    // 700 x 4096 x 1024 8.4 -> 7.7, 1000 x 2304 x 2048 11.1 -> 10.1, 650 x 3584 x 4096 16.4 -> 14.9, 816 x 2560 x 4096
+    // 16.1 -> 14.9, 560 x 4096 x 2048 10.9 -> 9.9.  Where the 128-row grid already fills the chip, or 128 x 64 tiles
+    // fit one round, it loses (816 x 2048 x 2048: 9.6 against 8.2 us; 1632 x 2560 x 2048: 17.5 against 15.4).
+    if (forced < 0 && pl.tile == 128 && pl.cols == 128 && !epi_is_gated(epilogue) && tiles > 128 && tiles < 256 && K < 8192) {
+        const int t96 = big_tiles(M, N, epilogue, 96, 128);
+        if (t96 > tiles && t96 <= 256) { pl.tile = 96; tiles = t96; }
+    }
     pl.tiles = tiles;
-    pl.depth = pl.tile == 128 ? 4 : 2;
-    if (pl.tile == 128 && pl.cols == 64) {
+    pl.depth = (pl.tile == 128 || pl.tile == 96) ? 4 : 2;
+    if ((pl.tile == 128 && pl.cols == 64) || pl.tile == 96) {
         // always one round of at most 256 workgroups here, or forced: deep ring, no split
     } else if (pl.tile == 128) {
         // Measured at M = 816: splitting pays for K = 16384 (67 -> 49 us with two splits) and
@@ -800,7 +812,7 @@ BigPlan big_plan(int M, int N, int K, int epilogue) {
     }
     if (const char* e = tuning_env("PHYAI_FP8_BIG_SPLITS")) {
         const int s = atoi(e);
-        if (pl.tile != 192 && pl.tile != 224 && pl.cols != 64 && s >= 1 && K % (s * 128) == 0 && K / s >= 512 && tiles * s <= 4096) pl.splits = s;
+        if (pl.tile != 192 && pl.tile != 224 && pl.tile != 96 && pl.cols != 64 && s >= 1 && K % (s * 128) == 0 && K / s >= 512 && tiles * s <= 4096) pl.splits = s;
     }
     if (const char* e = tuning_env("PHYAI_FP8_BIG_DEPTH")) {
         const int d = atoi(e);
@@ -936,6 +948,15 @@ int launch_gemm_big(const GemmProblem& g, const BigPlan& pl, hipStream_t st) {
         return big_launch_layout<7, 2, 2, 1, 4>(a, g, 1, st);
     }
     if (pl.tile == 192 && pl.splits == 1) return big_launch_layout<3, 2, 2>(a, g, 1, st);
+    if (pl.tile == 96) {   // 96 rows x 128 columns: wavefronts 1 x 4, three row blocks each; plain epilogues
+        if (pl.splits != 1) return -2;
+        switch (g.epilogue) {
+        case EPI_NONE: a.operand_w ? big_launch<3, 1, 4, EPI_NONE, 1, 4, 1>(a, g, 1, st) : big_launch<3, 1, 4, EPI_NONE, 1, 4, 0>(a, g, 1, st); return 0;
+        case EPI_GELU_TANH: a.operand_w ? big_launch<3, 1, 4, EPI_GELU_TANH, 1, 4, 1>(a, g, 1, st) : big_launch<3, 1, 4, EPI_GELU_TANH, 1, 4, 0>(a, g, 1, st); return 0;
+        case EPI_GELU_ERF: a.operand_w ? big_launch<3, 1, 4, EPI_GELU_ERF, 1, 4, 1>(a, g, 1, st) : big_launch<3, 1, 4, EPI_GELU_ERF, 1, 4, 0>(a, g, 1, st); return 0;
+        default: return -2;
+        }
+    }
     if (pl.tile == 128 && pl.cols == 64) {
         if (pl.splits != 1) return -2;
         switch (g.epilogue) {   // plain epilogues only: one column block per wavefront cannot hold a gate / up pair

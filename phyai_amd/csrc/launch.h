@@ -141,7 +141,7 @@ int launch_gemm_fused(const GemmProblem& p, const FusedPlan& pl, hipStream_t st)
 // Pipelined tile kernel for large M (gemm_big.hip), 256 x 256 or 128 x 128 tiles; the small
 // tiles may be split along K (partials in the workspace, as for the generic tile kernel).
 struct BigPlan {
-    int tile;    // tile rows: 256 (x 256 columns), 224 (x 256), 192 (x 128), 128 (x 128 or x 64), or 0 if the kernel does not apply
+    int tile;    // tile rows: 256 (x 256 columns), 224 (x 256), 192 (x 128), 128 (x 128 or x 64), 96 (x 128), or 0 if the kernel does not apply
     int cols;    // tile columns
     int splits;
     int tiles;   // output tiles of that size

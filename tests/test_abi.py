@@ -96,7 +96,11 @@ def test_kernel_selection_for_the_benchmark_shapes(monkeypatch):
     assert d(50, 1024, 4096) == "small-m nt=1 mb=1 kpw=4 rounds=1"
     assert d(1, 12288, 2048).startswith("small-m nt=1 mb=1")
     # prefix prefill, M = 816
-    assert d(816, 2560, 2048) == "tile 128x128 depth=4 splits=1 tiles=140"
+    assert d(816, 2560, 2048) == "tile 96x128 depth=4 splits=1 tiles=180"      # 140 tiles of 128 x 128 idle 116 CUs, 280 of 128 x 64 need two rounds
+    assert d(816, 2560, 2048, "gelu") == "tile 96x128 depth=4 splits=1 tiles=180"
+    assert d(816, 2560, 2048, "geglu_tanh") == "tile 128x128 depth=4 splits=1 tiles=140"   # gated: no single-column-block tile
+    assert d(816, 2560, 8192).startswith("tile 128x128 depth=4 splits=2")             # long K: split form
+    assert d(1632, 2560, 2048) == "tile 128x128 depth=2 splits=1 tiles=260"             # the 128-row grid fills the chip
     assert d(816, 2048, 2048) == "tile 128x64 depth=4 splits=1 tiles=224"      # 112 tiles of 128 x 128 would idle half the CUs
     assert d(816, 32768, 2048, "geglu_tanh") == "tile 224x256 depth=2 splits=1 tiles=512"   # four tile rows either way: less padding
     assert d(816, 2048, 16384) == "tile 128x128 depth=4 splits=2 tiles=112"

@@ -129,7 +129,7 @@ def test_operand_order_with_the_gated_residual(dev, M, N, K):
 # 224-row tile with K a multiple of 512, straight into registers); the same without the register path; gathered
 # row by row into the row-major staging layout
 @pytest.mark.parametrize("mode", ["", "PHYAI_FP8_BIG_DIRECT=0", "PHYAI_FP8_BIG_GATHER=1"])
-@pytest.mark.parametrize("tile", ["256", "224", "192", "128", "128/2", "12864"])
+@pytest.mark.parametrize("tile", ["256", "224", "192", "128", "128/2", "12864", "96"])
 @pytest.mark.parametrize("M,N,K,epi", [(816, 768, 1024, None), (513, 400, 1536, "gelu"), (816, 1024, 1152, "geglu_tanh"),
                                        (260, 288, 1024, "swiglu"), (300, 544, 2048, "geglu_erf")])
 def test_operand_order_in_every_pipelined_tile_shape(dev, monkeypatch, mode, tile, M, N, K, epi):

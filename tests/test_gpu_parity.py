@@ -370,7 +370,7 @@ def test_linear_repeatable_and_workspace_stays_clean(dev):
 
 def _force_big(monkeypatch, spec):
     """spec = "rows" or "rows/ring depth": 256 (x 256 columns), 224 (x 256), 192 (x 128), 128 (x 128, ring of 4 or 2),
-    12864 (128 x 64; plain epilogues only, a gated one keeps the default choice)."""
+    12864 (128 x 64) and 96 (96 x 128): plain epilogues only, a gated one keeps the default choice."""
     tile, _, depth = spec.partition("/")
     monkeypatch.setenv("PHYAI_FP8_BIG", tile)
     if depth:
@@ -381,7 +381,7 @@ def _force_big(monkeypatch, spec):
     (256, 256, 1024, None, 0), (300, 512, 1280, None, 0), (816, 768, 1024, None, 0), (513, 400, 1536, "gelu", 5),
     (816, 1024, 1152, "geglu_tanh", 1), (260, 288, 1024, "swiglu", 3), (1000, 256, 2048, None, 0),
 ])
-@pytest.mark.parametrize("tile", ["256", "224", "192", "128", "128/2", "12864"])
+@pytest.mark.parametrize("tile", ["256", "224", "192", "128", "128/2", "12864", "96"])
 def test_big_tile_kernel_forced(dev, monkeypatch, tile, M, N, K, epi_name, epi):
     ops = _ops()
     _force_big(monkeypatch, tile)
@@ -393,7 +393,7 @@ def test_big_tile_kernel_forced(dev, monkeypatch, tile, M, N, K, epi_name, epi):
     assert_close_to_ref(got, want, f"big kernel {M}x{N}x{K} epi={epi_name}")
 
 
-@pytest.mark.parametrize("tile", ["256", "224", "192", "128", "128/2", "12864"])
+@pytest.mark.parametrize("tile", ["256", "224", "192", "128", "128/2", "12864", "96"])
 def test_big_tile_kernel_exact_integer(dev, monkeypatch, tile):
     ops = _ops()
     _force_big(monkeypatch, tile)
@@ -424,7 +424,7 @@ def test_tile_variants_agree_bit_for_bit_on_random_shapes(dev, monkeypatch):
         xq, xs = ops.fp8_quant_rowwise(x.to(dev))
         wd, sd, bd = wq.to(dev), ws.to(dev), b.to(dev)
         outs = {}
-        for spec in ("256", "224", "192", "128", "128/2", "12864", "256/rows", "224/rows", "128/rows", "12864/rows", "generic"):
+        for spec in ("256", "224", "192", "128", "128/2", "12864", "96", "256/rows", "224/rows", "128/rows", "12864/rows", "96/rows", "generic"):
             monkeypatch.delenv("PHYAI_FP8_BIG", raising=False)
             monkeypatch.delenv("PHYAI_FP8_BIG_DEPTH", raising=False)
             monkeypatch.delenv("PHYAI_FP8_TILE", raising=False)
@@ -684,7 +684,8 @@ def test_quant_rowwise_exhaustive_all_values_all_scales(dev):
 @pytest.mark.parametrize("M,N,K,force,gate_rows", [
     (50, 1024, 2048, "", 1), (50, 1024, 4096, "", 50), (200, 1024, 4096, "", 4), (70, 192, 272, "", 70),
     (816, 2048, 2048, "128", 816), (816, 2048, 2048, "256", 1), (300, 384, 4096, "128", 3), (9, 64, 128, "", 9),
-    (816, 2048, 2048, "192", 816), (500, 640, 1024, "192", 5), (816, 2048, 2048, "224", 816), (500, 640, 1024, "224", 4), (816, 2048, 2048, "12864", 816), (500, 640, 1024, "12864", 1)])
+    (816, 2048, 2048, "192", 816), (500, 640, 1024, "192", 5), (816, 2048, 2048, "224", 816), (500, 640, 1024, "224", 4), (816, 2048, 2048, "12864", 816), (500, 640, 1024, "12864", 1),
+    (816, 2560, 2048, "", 816), (500, 640, 1024, "96", 1)])
 def test_linear_gated_residual(dev, monkeypatch, M, N, K, force, gate_rows):
     """out = addcmul(residual, linear(x), gate) inside the GEMM epilogue, every kernel family; the result
     must equal torch.addcmul applied to the device's own plain linear output bit for bit."""
