@@ -58,7 +58,8 @@ constexpr int BIG_BK = 128;   // bytes of K per LDS row: one L2 cache line
 // of the main loop left out, to see from the time stamps what each costs.  Bit 1: no copies / weight loads inside
 // the loop (the operands of the prologue are multiplied over and over); bit 2: the activation blocks of a K half
 // are not re-read from LDS; bit 4: no barrier in the loop of the variant that loads its weights into registers;
-// bits 8 / 16 (that variant): only the weight loads / only the activation copies of the loop are left out.
+// bit 8 (that variant): only the weight loads of the loop are left out; bit 16 (either variant): only the
+// activation copies.
 #ifndef PHYAI_FP8_ABLATE
 #define PHYAI_FP8_ABLATE 0
 #endif
