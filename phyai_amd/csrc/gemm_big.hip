@@ -243,7 +243,8 @@ void gemm_fp8_big_kernel(
     // (the epilogue stages the bf16 tile in the same LDS; where the ring is smaller than that, the ring grows)
     constexpr int EPI_STAGING = 4 * WM * ((GATED ? TN / 2 : TN) * 64);
     constexpr int LDS_BYTES = DEPTH * STAGE_BYTES > EPI_STAGING ? DEPTH * STAGE_BYTES : EPI_STAGING;
-    __shared__ __attribute__((aligned(1024))) uint8_t lds[LDS_BYTES];
+    // (weights in registers: 16 more bytes for the four wavefronts' progress words, see the main loop)
+    __shared__ __attribute__((aligned(1024))) uint8_t lds[LDS_BYTES + (BDIRECT ? 16 : 0)];
 
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     const int wm = wave / WGN, wn = wave % WGN;
@@ -361,6 +362,38 @@ void gemm_fp8_big_kernel(
         else return big_frag(bbuf, row, h, kh);
     };
 
+    // Weights in registers: LDS carries the activations only, and the wavefronts hand its stages to each other
+    // through one progress word each instead of meeting at a barrier.  Word w = d says: wavefront w has issued all its
+    // LDS reads of stage-loads <= d, and its own copies of stage-loads <= d + 2 have landed.  At its hand-over point
+    // of stage d a wavefront publishes d and goes on once every word is >= d - 1: then stage-load d + 1 is complete
+    // in LDS and the stage of d - 1 may be refilled (with d + 3).  A wavefront may so run up to one stage ahead of
+    // the slowest instead of waiting for it at every stage: each stalls now and then on its own memory requests, and a
+    // barrier per stage makes all four pay for every such stall (main loop at K = 2048: 40.2 k cycles with the
+    // barrier, 32.7 k with none at all).  The slowest wavefront never waits, so the scheme cannot lock up; the spin is
+    // bounded all the same (a wavefront that gave up would read a stage early: wrong numbers, never a hang).
+    // The words are read BEFORE the stage's last batch of operand reads and looked at behind the MFMAs that follow it
+    // (LDS answers in order: read at the hand-over point they would queue behind that batch, several hundred cycles
+    // with two MFMAs in the pipe); a value that old can only be too small, and then the words are read again.
+    // (pointers that say "LDS": through a generic pointer the accesses would be flat ones, counted with the copies)
+    typedef __attribute__((address_space(3))) int lds_int_t;
+    typedef __attribute__((address_space(3))) v4i lds_v4i_t;
+    volatile lds_int_t* const progress = (volatile lds_int_t*)(lds + LDS_BYTES);
+    auto progress_words = [&]() -> v4i { return *(const volatile lds_v4i_t*)(lds + LDS_BYTES); };
+    auto hand_over = [&](int d, v4i seen) {
+        if (lane == 0) progress[wave] = d;
+        auto behind = [&](const v4i& w) {
+            return __builtin_amdgcn_readfirstlane(min(min(w[0], w[1]), min(w[2], w[3]))) < d - 1;
+        };
+        if (__builtin_expect(behind(seen), 0)) {   // (its own block: the wait for `seen` above stays a counted one)
+#pragma nounroll
+            for (int spin = 0; spin < (1 << 18); ++spin) {
+                __builtin_amdgcn_s_sleep(1);
+                const v4i now = progress_words();
+                if (!behind(now)) break;
+            }
+        }
+    };
+
     // Operand blocks read one K half ahead: those of the current half (cur) and of the next one
     // (nxt); the two sets swap roles every half.  All B blocks and the first A block - or all A
     // blocks when there are only two row groups, which are too short to hide an LDS read.
@@ -390,6 +423,8 @@ void gemm_fp8_big_kernel(
         const uint8_t* abuf_ = stage_ptr(d_);                                                                  \
         const uint8_t* nbuf_ = (KH) == 0 ? abuf_ : stage_ptr(d_ + 1);                                          \
         v8i fa_[TM];                                                                                           \
+        v4i seen_ = {0, 0, 0, 0};                                                                              \
+        if constexpr (BDIRECT) if ((KH) == 1 && (NEXT)) seen_ = progress_words();                              \
         _Pragma("unroll") for (int i_ = 0; i_ < TM; ++i_) fa_[i_] = FA0[A_AHEAD ? i_ : 0];                     \
         _Pragma("unroll") for (int i_ = 0; i_ < TM; ++i_) {                                                    \
             if (!A_AHEAD && i_ == 0) {                                                                         \
@@ -428,8 +463,10 @@ void gemm_fp8_big_kernel(
             }                                                                                                  \
             if ((KH) == 1 && i_ == 0 && (NEXT)) {                                                              \
                 if constexpr (BDIRECT) {                                                                       \
-                    wait_copies<COPIES * (AHEAD)>();               /* my requests of D+1 have landed ... */    \
-                    if (!(PHYAI_FP8_ABLATE & 4)) __builtin_amdgcn_s_barrier(); /* ... and so have everybody's */ \
+                    /* my activation copies of D+2 have landed (its weight loads, requested after them, may  */ \
+                    /* be in flight); published, and everybody's of D+1 awaited                              */ \
+                    wait_copies<(COPIES - CA) * (AHEAD)>();                                                    \
+                    if (!(PHYAI_FP8_ABLATE & 4)) hand_over(d_, seen_);                                                \
                     asm volatile("" ::: "memory");                                                             \
                 } else {                                                                                       \
                     asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory"); /* my reads of stage-load D have landed */ \
@@ -465,7 +502,13 @@ void gemm_fp8_big_kernel(
 #pragma unroll
         for (int c = 0; c < HEAD_IDX; ++c) issue(DEPTH - 1, c, Slot0{});
     }
-    wait_copies<COPIES * (LEAD - 2) + HEAD + (BDIRECT ? COPIES : 0)>();   // stage-load 0 has landed
+    if constexpr (BDIRECT) {
+        // stage-load 0 and the activations of stage-load 1 have landed (what progress word -1 stands for)
+        wait_copies<COPIES + (COPIES - CA)>();
+        if (lane == 0) progress[wave] = -1;
+    } else {
+        wait_copies<COPIES * (LEAD - 2) + HEAD>();   // stage-load 0 has landed
+    }
     __syncthreads();
     PHYAI_STAMP(1)
 #pragma unroll
