@@ -215,7 +215,7 @@ void gemm_fp8_big_kernel(
     constexpr bool GATED = epi_is_gated(EPI);
     constexpr bool OPW = WMODE != 0, BDIRECT = WMODE == 2;
     static_assert(WGM * WGN == 4, "four wavefronts per workgroup");
-    static_assert(!BDIRECT || (WGM == 1 && DEPTH == 4), "weights go straight to registers only where a wavefront owns them");
+    static_assert(!BDIRECT || (WGM == 1 && (DEPTH == 4 || DEPTH == 8)), "weights go straight to registers only where a wavefront owns them");
     constexpr int BM = WGM * 32 * TM, BN = WGN * 32 * TN;   // workgroup tile
     constexpr int WM = 32 * TM, WN = 32 * TN;        // wavefront tile
     constexpr int STAGE_BYTES = (BM + (BDIRECT ? 0 : BN)) * BIG_BK;  // one stage: A rows, then B rows (if staged)
@@ -231,15 +231,22 @@ void gemm_fp8_big_kernel(
     // every wavefront has issued before it reaches the barrier of stage d, so the barrier need not wait for the
     // LDS reads in flight (the activation blocks of the second K half, requested just before it), and no register
     // set is written while MFMAs of its stage are still to come.
-    constexpr int CPS = (COPIES * 2 + SLOTS_PER_STAGE - 1) / SLOTS_PER_STAGE;
-    constexpr int LEAD = BDIRECT ? DEPTH - 1 : DEPTH;
+    // Weights in registers, ring of eight (one column block per wavefront, stages of 8 MFMAs or fewer): LEAD = 6, so
+    // that a wavefront may run two stages ahead of the slowest (see the hand-over below) with its weight loads six
+    // stages and its activation copies three stages old when they are needed.
+    constexpr int CPS = BDIRECT ? (COPIES + (TM - 1) * TN - 1) / ((TM - 1) * TN) : (COPIES * 2 + SLOTS_PER_STAGE - 1) / SLOTS_PER_STAGE;
+    constexpr int LEAD = BDIRECT ? (DEPTH == 8 ? 6 : DEPTH - 1) : DEPTH;
+    // (weights in registers) progress word d of a wavefront vouches for its activation copies up to stage-load
+    // d + CLAIM; SLACK: how many stages a wavefront may be ahead of the slowest one
+    constexpr int CLAIM = DEPTH == 8 ? 3 : 2;
+    constexpr int SLACK = CLAIM - 1 < DEPTH - LEAD ? CLAIM - 1 : DEPTH - LEAD;
     constexpr int LATE = (TM - 1) * TN * CPS;        // first request number that falls into the next stage
     constexpr int IDX_END = COPIES;
     static_assert(!BDIRECT || COPIES <= LATE, "with weights in registers every request goes out behind the barrier");
     static_assert((TM == TN && TM % 2 == 0) || (TM == 3 && TN == 2) || (TM == 7 && TN == 2) || (TM == 2 && TN == 1 && !GATED) ||
-                  (TM == 3 && TN == 1 && !GATED), "supported wavefront tiles");
+                  (TM == 3 && TN == 1 && !GATED) || (TM == 4 && TN == 1 && !GATED && BDIRECT), "supported wavefront tiles");
     static_assert(BM % 32 == 0 && BN % 32 == 0, "every wavefront copies whole groups of 8 rows");
-    static_assert(DEPTH == 2 || DEPTH == 4, "ring depth");
+    static_assert(DEPTH == 2 || DEPTH == 4 || (DEPTH == 8 && BDIRECT), "ring depth");
     // (the epilogue stages the bf16 tile in the same LDS; where the ring is smaller than that, the ring grows)
     constexpr int EPI_STAGING = 4 * WM * ((GATED ? TN / 2 : TN) * 64);
     constexpr int LDS_BYTES = DEPTH * STAGE_BYTES > EPI_STAGING ? DEPTH * STAGE_BYTES : EPI_STAGING;
@@ -364,13 +371,15 @@ void gemm_fp8_big_kernel(
 
     // Weights in registers: LDS carries the activations only, and the wavefronts hand its stages to each other
     // through one progress word each instead of meeting at a barrier.  Word w = d says: wavefront w has issued all its
-    // LDS reads of stage-loads <= d, and its own copies of stage-loads <= d + 2 have landed.  At its hand-over point
-    // of stage d a wavefront publishes d and goes on once every word is >= d - 1: then stage-load d + 1 is complete
-    // in LDS and the stage of d - 1 may be refilled (with d + 3).  A wavefront may so run up to one stage ahead of
-    // the slowest instead of waiting for it at every stage: each stalls now and then on its own memory requests, and a
-    // barrier per stage makes all four pay for every such stall (main loop at K = 2048: 40.2 k cycles with the
-    // barrier, 32.7 k with none at all).  The slowest wavefront never waits, so the scheme cannot lock up; the spin is
-    // bounded all the same (a wavefront that gave up would read a stage early: wrong numbers, never a hang).
+    // LDS reads of stage-loads <= d, and its own copies of stage-loads <= d + CLAIM have landed.  At its hand-over
+    // point of stage d a wavefront publishes d and goes on once every word is >= d - SLACK: then stage-load d + 1 is
+    // complete in LDS (SLACK <= CLAIM - 1) and the stage that stage-load d + LEAD refills has been read by everyone
+    // (it held stage-load d + LEAD - DEPTH <= d - SLACK).  A wavefront may so run up to SLACK stages ahead of the
+    // slowest instead of waiting for it at every stage: each stalls now and then on its own memory requests, and a
+    // barrier per stage makes all four pay for every such stall (224 x 256 main loop at K = 2048: 40.2 k cycles with
+    // the barrier, 32.7 k with none at all and with this).  The slowest wavefront never waits, so the scheme cannot
+    // lock up; the spin is bounded all the same (a wavefront that gave up would read a stage early: wrong numbers,
+    // never a hang).
     // The words are read BEFORE the stage's last batch of operand reads and looked at behind the MFMAs that follow it
     // (LDS answers in order: read at the hand-over point they would queue behind that batch, several hundred cycles
     // with two MFMAs in the pipe); a value that old can only be too small, and then the words are read again.
@@ -382,7 +391,7 @@ void gemm_fp8_big_kernel(
     auto hand_over = [&](int d, v4i seen) {
         if (lane == 0) progress[wave] = d;
         auto behind = [&](const v4i& w) {
-            return __builtin_amdgcn_readfirstlane(min(min(w[0], w[1]), min(w[2], w[3]))) < d - 1;
+            return __builtin_amdgcn_readfirstlane(min(min(w[0], w[1]), min(w[2], w[3]))) < d - SLACK;
         };
         if (__builtin_expect(behind(seen), 0)) {   // (its own block: the wait for `seen` above stays a counted one)
 #pragma nounroll
@@ -463,15 +472,16 @@ void gemm_fp8_big_kernel(
             }                                                                                                  \
             if ((KH) == 1 && i_ == 0 && (NEXT)) {                                                              \
                 if constexpr (BDIRECT) {                                                                       \
-                    /* my activation copies of D+2 have landed (its weight loads, requested after them, may  */ \
-                    /* be in flight); published, and everybody's of D+1 awaited                              */ \
-                    wait_copies<(COPIES - CA) * (AHEAD)>();                                                    \
+                    /* my activation copies of D+CLAIM have landed (AHEAD: the stage-loads from that one on  */ \
+                    /* that have been requested: its weight loads, which follow its copies, and all of the   */ \
+                    /* later ones may be in flight); published, and everybody's of D+1 awaited               */ \
+                    wait_copies<(AHEAD) == 0 ? 0 : ((AHEAD) - 1) * COPIES + (COPIES - CA)>();                  \
                     if (!(PHYAI_FP8_ABLATE & 4)) hand_over(d_, seen_);                                                \
                     asm volatile("" ::: "memory");                                                             \
                 } else {                                                                                       \
                     asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory"); /* my reads of stage-load D have landed */ \
                     wait_copies<COPIES * (AHEAD)>();               /* ... my copies of D+1 too ... */          \
-                    __syncthreads();                               /* ... and so have everybody's */           \
+                    if (!(PHYAI_FP8_ABLATE & 4)) __syncthreads();  /* ... and so have everybody's */           \
                 }                                                                                              \
             }                                                                                                  \
         }                                                                                                      \
@@ -487,13 +497,28 @@ void gemm_fp8_big_kernel(
     // (as request numbers up to LATE, and as the instructions they are)
     constexpr int HEAD_IDX = LATE < IDX_END ? LATE : IDX_END;
     constexpr int HEAD = BDIRECT ? 0 : HEAD_IDX;
-    if constexpr (BDIRECT) {   // stage-loads 0 .. LEAD - 1 = 2; stage-load d fills register set d % 4
+    if constexpr (BDIRECT) {   // stage-loads 0 .. LEAD - 1; stage-load d fills register set d % DEPTH
+        // First what the first stage waits for: the activations of the stage-loads that progress word -1 vouches
+        // for (0 .. CLAIM - 1; they come from L2) and the weights of stage-load 0; then the other weights of those
+        // stage-loads and the later stage-loads whole, in the order the waits of the main loop count on.
+        auto part = [&](auto slot, int c0, int c1) {
 #pragma unroll
-        for (int c = 0; c < IDX_END; ++c) issue(0, c, std::integral_constant<int, 0>{});
-#pragma unroll
-        for (int c = 0; c < IDX_END; ++c) issue(1, c, std::integral_constant<int, 1>{});
-#pragma unroll
-        for (int c = 0; c < IDX_END; ++c) issue(2, c, std::integral_constant<int, 2>{});
+            for (int c = c0; c < c1; ++c) issue(decltype(slot)::value, c, slot);
+        };
+        using S0 = std::integral_constant<int, 0>; using S1 = std::integral_constant<int, 1>;
+        using S2 = std::integral_constant<int, 2>;
+        part(S0{}, 0, CA);
+        part(S1{}, 0, CA);
+        if constexpr (CLAIM == 3) part(S2{}, 0, CA);
+        part(S0{}, CA, IDX_END);
+        part(S1{}, CA, IDX_END);
+        if constexpr (CLAIM == 3) part(S2{}, CA, IDX_END);
+        if constexpr (CLAIM == 2) part(S2{}, 0, IDX_END);
+        if constexpr (LEAD == 6) {
+            part(std::integral_constant<int, 3>{}, 0, IDX_END);
+            part(std::integral_constant<int, 4>{}, 0, IDX_END);
+            part(std::integral_constant<int, 5>{}, 0, IDX_END);
+        }
     } else {
 #pragma unroll
         for (int d = 0; d < DEPTH - 1; ++d)
@@ -503,8 +528,8 @@ void gemm_fp8_big_kernel(
         for (int c = 0; c < HEAD_IDX; ++c) issue(DEPTH - 1, c, Slot0{});
     }
     if constexpr (BDIRECT) {
-        // stage-load 0 and the activations of stage-load 1 have landed (what progress word -1 stands for)
-        wait_copies<COPIES + (COPIES - CA)>();
+        // stage-load 0 and the activations up to stage-load CLAIM - 1 have landed (what progress word -1 stands for)
+        wait_copies<(LEAD - CLAIM) * COPIES + (CLAIM - 1) * (COPIES - CA)>();
         if (lane == 0) progress[wave] = -1;
     } else {
         wait_copies<COPIES * (LEAD - 2) + HEAD>();   // stage-load 0 has landed
@@ -518,20 +543,40 @@ void gemm_fp8_big_kernel(
     for (int i = 0; i < (A_AHEAD ? TM : 1); ++i) fa_cur[i] = big_frag(lds, arow + i * 32, h, 0);
     int d = 0;
     if constexpr (BDIRECT) {
-        // the register sets are named at compile time: four stage-loads per trip (the launcher sees to it
-        // that their number is a multiple of four)
-        // at the barrier of stage d stage-load d + 2 may be in flight; behind it stage-load d + 3 is requested
+        // the register sets are named at compile time: DEPTH stage-loads per trip (the launcher sees to it
+        // that their number is a multiple of DEPTH)
+        // ring of four: at the hand-over of stage d stage-load d + 2 may be in flight; behind it d + 3 is requested
         for (; d < n_loads - DEPTH; d += DEPTH) {
-            PHYAI_RUN_STAGE(d, 0, 1, 1, 0, 1)
-            PHYAI_RUN_STAGE(d + 1, 1, 1, 1, 0, 1)
-            PHYAI_RUN_STAGE(d + 2, 2, 1, 1, 0, 1)
-            PHYAI_RUN_STAGE(d + 3, 3, 1, 1, 0, 1)
+            if constexpr (DEPTH == 4) {
+                PHYAI_RUN_STAGE(d, 0, 1, 1, 0, 1)
+                PHYAI_RUN_STAGE(d + 1, 1, 1, 1, 0, 1)
+                PHYAI_RUN_STAGE(d + 2, 2, 1, 1, 0, 1)
+                PHYAI_RUN_STAGE(d + 3, 3, 1, 1, 0, 1)
+            } else {   // at the hand-over of stage d stage-loads d + 3 .. d + 5 may be in flight; d + 6 is requested behind it
+                PHYAI_RUN_STAGE(d, 0, 1, 3, 0, 1)
+                PHYAI_RUN_STAGE(d + 1, 1, 1, 3, 0, 1)
+                PHYAI_RUN_STAGE(d + 2, 2, 1, 3, 0, 1)
+                PHYAI_RUN_STAGE(d + 3, 3, 1, 3, 0, 1)
+                PHYAI_RUN_STAGE(d + 4, 4, 1, 3, 0, 1)
+                PHYAI_RUN_STAGE(d + 5, 5, 1, 3, 0, 1)
+                PHYAI_RUN_STAGE(d + 6, 6, 1, 3, 0, 1)
+                PHYAI_RUN_STAGE(d + 7, 7, 1, 3, 0, 1)
+            }
         }
     } else {
         for (; d < n_loads - DEPTH; ++d) { PHYAI_RUN_STAGE(d, 0, 1, DEPTH - 2, 1, 1) }
     }
     // d == n_loads - DEPTH: the last requests are still being spread, then the ring drains
-    if constexpr (BDIRECT) {   // the last request goes out behind the barrier of stage n - 4
+    if constexpr (BDIRECT && DEPTH == 8) {   // the last request goes out behind the hand-over of stage n - 7
+        PHYAI_RUN_STAGE(d, 0, 1, 3, 0, 1)
+        PHYAI_RUN_STAGE(d + 1, 1, 1, 3, 0, 1)
+        PHYAI_RUN_STAGE(d + 2, 2, 1, 3, 0, 0)
+        PHYAI_RUN_STAGE(d + 3, 3, 1, 2, 0, 0)
+        PHYAI_RUN_STAGE(d + 4, 4, 1, 1, 0, 0)
+        PHYAI_RUN_STAGE(d + 5, 5, 1, 0, 0, 0)
+        PHYAI_RUN_STAGE(d + 6, 6, 1, 0, 0, 0)
+        PHYAI_RUN_STAGE(d + 7, 7, 0, 0, 0, 0)
+    } else if constexpr (BDIRECT) {   // the last request goes out behind the hand-over of stage n - 4
         PHYAI_RUN_STAGE(d, 0, 1, 1, 0, 1)
         PHYAI_RUN_STAGE(d + 1, 1, 1, 1, 0, 0)
         PHYAI_RUN_STAGE(d + 2, 2, 1, 0, 0, 0)
@@ -927,7 +972,7 @@ static void big_launch(BigArgs a, const GemmProblem& g, int splits, hipStream_t 
 #define PHYAI_BIG_ARGS a.a, a.b, a.K, a.M, a.N, a.m_tiles, a.n_tiles, a.band, a.by_rows | (a.operand_w << 4), a.k_per_split, a.a_scale, \
                        a.b_scale, a.bias, a.out, a.ldo, a.a_scale_scalar, a.partials, a.counters, a.res
     if (splits > 1) {
-        if constexpr (TM == TN && (TM == 4 || DEPTH == 4))
+        if constexpr ((TM == TN && (TM == 4 || DEPTH == 4)) || (WMODE == 2 && TN == 1))
             hipLaunchKernelGGL((gemm_fp8_big_kernel<TM, TN, DEPTH, EPI, true, WGM, WGN, WMODE>), grid, dim3(256), 0, st, PHYAI_BIG_ARGS);
     } else {
         hipLaunchKernelGGL((gemm_fp8_big_kernel<TM, TN, DEPTH, EPI, false, WGM, WGN, WMODE>), grid, dim3(256), 0, st, PHYAI_BIG_ARGS);
@@ -942,6 +987,17 @@ static int big_launch_epi(const BigArgs& a, const GemmProblem& g, int splits, hi
     case EPI_GEGLU_TANH: big_launch<TM, TN, DEPTH, EPI_GEGLU_TANH, WGM, WGN, WMODE>(a, g, splits, st); return 0;
     case EPI_GEGLU_ERF: big_launch<TM, TN, DEPTH, EPI_GEGLU_ERF, WGM, WGN, WMODE>(a, g, splits, st); return 0;
     case EPI_SWIGLU: big_launch<TM, TN, DEPTH, EPI_SWIGLU, WGM, WGN, WMODE>(a, g, splits, st); return 0;
+    case EPI_GELU_TANH: big_launch<TM, TN, DEPTH, EPI_GELU_TANH, WGM, WGN, WMODE>(a, g, splits, st); return 0;
+    case EPI_GELU_ERF: big_launch<TM, TN, DEPTH, EPI_GELU_ERF, WGM, WGN, WMODE>(a, g, splits, st); return 0;
+    default: return -2;
+    }
+}
+
+// (tiles with one column block per wavefront cannot hold a gate / up pair: plain epilogues only)
+template <int TM, int TN, int DEPTH, int WGM = 2, int WGN = 2, int WMODE = 0>
+static int big_launch_plain(const BigArgs& a, const GemmProblem& g, int splits, hipStream_t st) {
+    switch (g.epilogue) {
+    case EPI_NONE: big_launch<TM, TN, DEPTH, EPI_NONE, WGM, WGN, WMODE>(a, g, splits, st); return 0;
     case EPI_GELU_TANH: big_launch<TM, TN, DEPTH, EPI_GELU_TANH, WGM, WGN, WMODE>(a, g, splits, st); return 0;
     case EPI_GELU_ERF: big_launch<TM, TN, DEPTH, EPI_GELU_ERF, WGM, WGN, WMODE>(a, g, splits, st); return 0;
     default: return -2;
@@ -982,11 +1038,15 @@ int launch_gemm_big(const GemmProblem& g, const BigPlan& pl, hipStream_t st) {
                           g.workspace_bytes < kGemmHeaderBytes + big_partial_bytes(g.M, g.N, g.epilogue, pl)))
         return -3;
     if (pl.tile == 256) return big_launch_layout<4, 4, 2>(a, g, pl.splits, st);
+    // weights in operand order and a whole number of trips round the ring per K range: the wavefronts load
+    // their own weight blocks straight into registers (PHYAI_FP8_BIG_DIRECT=0: stage them like the rest)
+    const bool may_direct = a.operand_w && !(tuning_env("PHYAI_FP8_BIG_DIRECT") && atoi(tuning_env("PHYAI_FP8_BIG_DIRECT")) == 0);
+    // (ring of eight for 128 x 128 tiles, wavefronts 1 x 4 with one column block each; plain epilogues only.  Not for
+    // the 96 x 128 tile: its main loop gains what its longer prologue - six stage-loads requested up front, at
+    // what the CU's vector-memory path passes - loses: 816 x 2560 x 2048 10.0 -> 10.1 us)
+    const bool direct8 = may_direct && a.k_per_split % 1024 == 0 && !epi_is_gated(g.epilogue);
     if (pl.tile == 224) {
-        // weights in operand order and a whole number of four-stage trips per K range: the wavefronts load
-        // their own weight blocks straight into registers (PHYAI_FP8_BIG_DIRECT=0: stage them like the rest)
-        const bool direct = a.operand_w && g.K % 512 == 0 &&
-                            !(tuning_env("PHYAI_FP8_BIG_DIRECT") && atoi(tuning_env("PHYAI_FP8_BIG_DIRECT")) == 0);
+        const bool direct = may_direct && g.K % 512 == 0;
         if (pl.splits != 1) return -2;
         if (direct) return big_launch_epi<7, 2, 4, 1, 4, 2>(a, g, 1, st);
         return big_launch_layout<7, 2, 2, 1, 4>(a, g, 1, st);
@@ -994,22 +1054,13 @@ int launch_gemm_big(const GemmProblem& g, const BigPlan& pl, hipStream_t st) {
     if (pl.tile == 192 && pl.splits == 1) return big_launch_layout<3, 2, 2>(a, g, 1, st);
     if (pl.tile == 96) {   // 96 rows x 128 columns: wavefronts 1 x 4, three row blocks each; plain epilogues
         if (pl.splits != 1) return -2;
-        switch (g.epilogue) {
-        case EPI_NONE: a.operand_w ? big_launch<3, 1, 4, EPI_NONE, 1, 4, 1>(a, g, 1, st) : big_launch<3, 1, 4, EPI_NONE, 1, 4, 0>(a, g, 1, st); return 0;
-        case EPI_GELU_TANH: a.operand_w ? big_launch<3, 1, 4, EPI_GELU_TANH, 1, 4, 1>(a, g, 1, st) : big_launch<3, 1, 4, EPI_GELU_TANH, 1, 4, 0>(a, g, 1, st); return 0;
-        case EPI_GELU_ERF: a.operand_w ? big_launch<3, 1, 4, EPI_GELU_ERF, 1, 4, 1>(a, g, 1, st) : big_launch<3, 1, 4, EPI_GELU_ERF, 1, 4, 0>(a, g, 1, st); return 0;
-        default: return -2;
-        }
+        return a.operand_w ? big_launch_plain<3, 1, 4, 1, 4, 1>(a, g, 1, st) : big_launch_plain<3, 1, 4, 1, 4, 0>(a, g, 1, st);
     }
     if (pl.tile == 128 && pl.cols == 64) {
         if (pl.splits != 1) return -2;
-        switch (g.epilogue) {   // plain epilogues only: one column block per wavefront cannot hold a gate / up pair
-        case EPI_NONE: a.operand_w ? big_launch<2, 1, 4, EPI_NONE, 2, 2, 1>(a, g, 1, st) : big_launch<2, 1, 4, EPI_NONE>(a, g, 1, st); return 0;
-        case EPI_GELU_TANH: a.operand_w ? big_launch<2, 1, 4, EPI_GELU_TANH, 2, 2, 1>(a, g, 1, st) : big_launch<2, 1, 4, EPI_GELU_TANH>(a, g, 1, st); return 0;
-        case EPI_GELU_ERF: a.operand_w ? big_launch<2, 1, 4, EPI_GELU_ERF, 2, 2, 1>(a, g, 1, st) : big_launch<2, 1, 4, EPI_GELU_ERF>(a, g, 1, st); return 0;
-        default: return -2;
-        }
+        return a.operand_w ? big_launch_plain<2, 1, 4, 2, 2, 1>(a, g, 1, st) : big_launch_plain<2, 1, 4, 2, 2, 0>(a, g, 1, st);
     }
+    if (pl.tile == 128 && pl.depth == 4 && direct8) return big_launch_plain<4, 1, 8, 1, 4, 2>(a, g, pl.splits, st);
     if (pl.tile == 128 && pl.depth == 4) return big_launch_layout<2, 2, 4>(a, g, pl.splits, st);
     if (pl.tile == 128 && pl.splits == 1) return big_launch_layout<2, 2, 2>(a, g, 1, st);
     return -2;

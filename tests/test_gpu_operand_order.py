@@ -143,6 +143,25 @@ def test_operand_order_in_every_pipelined_tile_shape(dev, monkeypatch, mode, til
     assert torch.equal(_bits(lin_op), _bits(lin_rm))
 
 
+# 128 x 128 tiles with weights in operand order, a plain epilogue and K (per split) a multiple of 1024:
+# wavefronts 1 x 4, weights straight into registers through a ring of eight, activation stages handed over through
+# progress words.  One trip round the ring (tail only), several, K split 2 and 4, ragged M and N.
+@pytest.mark.parametrize("tile,splits,M,N,K,epi", [
+    ("128", "1", 816, 768, 1024, None), ("128", "1", 816, 768, 2048, "gelu"), ("128", "2", 816, 768, 2048, None),
+    ("128", "1", 513, 400, 3072, "gelu_tanh"), ("128", "1", 300, 272, 8192, None), ("128", "2", 300, 272, 8192, "gelu"),
+    ("128", "4", 300, 272, 8192, None), ("128", "2", 130, 2048, 16384, None), ("128", "1", 129, 144, 5120, None),
+    ("128", "1", 97, 144, 1024, "gelu_erf"), ("128", "1", 480, 1024, 7168, None),
+])
+def test_register_weights_ring_of_eight(dev, monkeypatch, tile, splits, M, N, K, epi):
+    monkeypatch.setenv("PHYAI_FP8_BIG", tile)
+    monkeypatch.setenv("PHYAI_FP8_BIG_SPLITS", splits)
+    (lin_rm, gemm_rm), (lin_op, gemm_op) = _both_layouts(dev, M, N, K, epi, seed=M + N + K + 5)
+    assert torch.equal(_bits(lin_op), _bits(lin_rm)) and torch.equal(_bits(gemm_op), _bits(gemm_rm))
+    monkeypatch.setenv("PHYAI_FP8_BIG_DIRECT", "0")      # the same tiles with the weights staged through LDS
+    (_, _), (lin_st, _) = _both_layouts(dev, M, N, K, epi, seed=M + N + K + 5)
+    assert torch.equal(_bits(lin_st), _bits(lin_op))
+
+
 def test_layout_and_epilogue_must_match(dev):
     ops = _ops()
     from phyai_amd import _lib
