@@ -456,9 +456,13 @@ def launch_floor_us(dev, nodes=2000):
 
 
 def ops_plan(M, N, K, epi):
+    """What the whole linear is launched as, for weights in the layout the benchmark passes."""
     from phyai_amd import ops
 
-    return ops.describe_linear_plan(M, N, K, epi)
+    lay = None
+    if OPTS["operand"] and K % 128 == 0:
+        lay = "operand_gated" if (epi is not None and "glu" in str(epi)) else "operand"
+    return ops.describe_linear_plan(M, N, K, epi, weight_layout=lay)
 
 
 def layer_plans(layer, shapes, M):
@@ -830,7 +834,7 @@ def stamps_report(dev):
             d = (r[:, b] - r[:, a]).sort().values
             name = names[b - 1] if b != last else names[-1]
             cells.append(f"{name}: {d[len(d) // 2].item():.0f} ({d[len(d) // 10].item():.0f} .. {d[(9 * len(d)) // 10].item():.0f})")
-        plan = ops_plan(M, N, K, epi) if small_m else ops.describe_plan(M, N, K, epi)
+        plan = ops_plan(M, N, K, epi) if small_m else ops.describe_plan(M, N, K, epi, weight_layout=wl)
         print(f"| {label} {M} x {N} x {K} | {plan}, {len(r)} wavefronts | {clock:.2f} | {span:.1f} | " + "; ".join(cells) + " |")
         del lay, rec
 

@@ -276,7 +276,9 @@ int phyai_fp8_adarmsnorm_quant(const void *x, int64_t ldx, const void *modulatio
  *   "tile 192x128 depth=2 splits=1 tiles=2304"   pipelined tile kernel
  *   "generic 128x128 splits=2"               fallback tile kernel
  * written to buf (at most n bytes, always terminated).  Host only: nothing is launched, no GPU is
- * needed.  Returns the length of the text, or a negative status for bad arguments.  The
+ * needed.  The layout flag of the weight matrix (PHYAI_FP8_FLAG_W_OPERAND_ORDER / _GATED) may be
+ * OR-ed into `epilogue` as in the calls: the choice of tile can depend on it.  Returns the length
+ * of the text, or a negative status for bad arguments.  The
  * reference has no counterpart (its dispatcher only picks between whole backends,
  * layers/linear/dispatch.py:28-95); this is for logs and for tests of the selection rules.
  */

@@ -542,11 +542,15 @@ int phyai_fp8_describe_plan(int64_t M, int64_t N, int64_t K, int epilogue, char*
     buf[0] = 0;
     if (M < 0 || N <= 0 || K <= 0 || M >= kMaxElems || N >= kMaxElems || K >= kMaxElems)
         return fail(PHYAI_FP8_EINVAL, "phyai_fp8_describe_plan: bad shape M=%lld N=%lld K=%lld", (long long)M, (long long)N, (long long)K);
-    epilogue &= PHYAI_FP8_EPILOGUE_MASK;   // flags do not change the choice of kernel
+    const int layout_bits = epilogue & PHYAI_FP8_FLAG_W_OPERAND_GATED;
+    epilogue &= PHYAI_FP8_EPILOGUE_MASK;   // of the flags only the layout of the weights bears on the choice of kernel
     if (int rc = check_epilogue(epilogue, N)) return rc;
     if (K % 16 != 0 || N % 16 != 0)
         return fail(PHYAI_FP8_EUNSUPPORTED, "phyai_fp8_describe_plan: K=%lld and N=%lld must be multiples of 16", (long long)K, (long long)N);
-    const int len = phyai::describe_gemm_plan((int)M, (int)N, (int)K, epilogue, buf, n);
+    int layout = phyai::W_ROW_MAJOR;
+    if (layout_bits && K % 128 == 0 && N % (phyai::epi_is_gated(epilogue) ? 32 : 16) == 0)
+        layout = phyai::epi_is_gated(epilogue) ? phyai::W_OPERAND_GATED : phyai::W_OPERAND_PLAIN;
+    const int len = phyai::describe_gemm_plan((int)M, (int)N, (int)K, epilogue, buf, n, layout);
     buf[n - 1] = 0;
     return len;
 }

@@ -57,9 +57,8 @@ constexpr int BIG_BK = 128;   // bytes of K per LDS row: one L2 cache line
 // Measurement only (make stamps ABLATE=n builds the time-stamp library with it; results are WRONG by design): parts
 // of the main loop left out, to see from the time stamps what each costs.  Bit 1: no copies / weight loads inside
 // the loop (the operands of the prologue are multiplied over and over); bit 2: the activation blocks of a K half
-// are not re-read from LDS; bit 4: no barrier in the loop of the variant that loads its weights into registers;
-// bit 8 (that variant): only the weight loads of the loop are left out; bit 16 (either variant): only the
-// activation copies.
+// are not re-read from LDS; bit 4: no barrier / no hand-over between the wavefronts in the loop; bit 8 (weights in
+// registers): only the weight loads of the loop are left out; bit 16 (either variant): only the activation copies.
 #ifndef PHYAI_FP8_ABLATE
 #define PHYAI_FP8_ABLATE 0
 #endif
@@ -826,7 +825,7 @@ static double big_fill(int tiles, int slots) {
     return rounds > 0 ? (double)tiles / ((double)rounds * slots) : 1.0;
 }
 
-BigPlan big_plan(int M, int N, int K, int epilogue) {
+BigPlan big_plan(int M, int N, int K, int epilogue, bool operand_w) {
     BigPlan pl = {0, 0, 1, 0, 0};
     if (K % 128 != 0 || K < 512) return pl;   // slabs come in pairs and must fill the ring
     int forced = -1;
@@ -887,6 +886,29 @@ BigPlan big_plan(int M, int N, int K, int epilogue) {
     }
     pl.tiles = tiles;
     pl.depth = (pl.tile == 128 || pl.tile == 96) ? 4 : 2;
+    bool to_224 = false;
+    if (operand_w && forced < 0 && pl.tile != 224 && K >= 4096 && K % 512 == 0) {
+        // Weights in operand order: the 224 x 256 tile loads them straight into registers and hands its activation
+        // stages over without barriers - its main loop runs at 0.88 of the MFMA rate where the other shapes reach
+        // 0.7 - 0.85 - and from K = 4096 on the prologue and epilogue that nothing overlaps in it weigh less than
+        // that.  Taken when it has at least 160 tiles and fills its rounds of 256 workgroups with useful rows and
+        // columns at least 0.8 times as well as the shape chosen above fills its own (weights from HBM, 4 - 6 weight
+        // sets, us: 6528 x 2048 x 16384 185 -> 166, 13056 x 2048 x 16384 366 -> 317, 6528 x 2048 x 8192 96 -> 86,
+        // 1632 x 8192 x 8192 96 -> 88, 4800 x 2048 x 8192 81 -> 74, 6528 x 4096 x 4096 106 -> 96, 13056 x 2048 x 4096
+        // 107 -> 98, 3264 x 16384 x 4096 + GeGLU 202 -> 189; level: 4800 x 8192 x 4096, 3264 x 8192 x 4096; not taken,
+        // and slower when forced: 2048 x 8192 x 8192 (320 tiles, two rounds: 150 against 103), 8000 x 1024 x 8192 (144
+        // tiles: 74 against 69), 3264 x 2048 x 16384 (120 tiles: 129 against 125).  At K = 2048 the shapes that run
+        // two workgroups per CU keep their lead.
+        const int t224 = big_tiles(M, N, epilogue, 224, 256);
+        const int slots = big_two_per_cu(pl.tile == 192 ? 3 : pl.tile == 256 ? 4 : 2, 2, pl.depth, 0) ? 512 : 256;
+        const double area_now = (double)big_ceil_div(tiles * pl.splits, slots) * slots * pl.tile * pl.cols;
+        const double area_224 = (double)big_ceil_div(t224, 256) * 256 * 224 * 256;
+        if (t224 >= 160 && pl.splits == 1 && area_now >= 0.8 * area_224) to_224 = true;
+    }
+    if (to_224) {
+        pl.tile = 224; pl.cols = 256; pl.depth = 2;
+        pl.tiles = tiles = big_tiles(M, N, epilogue, 224, 256);
+    }
     if ((pl.tile == 128 && pl.cols == 64) || pl.tile == 96) {
         // always one round of at most 256 workgroups here, or forced: deep ring, no split
     } else if (pl.tile == 128) {

@@ -321,8 +321,11 @@ size_t gemm_workspace_bytes(int64_t M, int64_t N, int64_t K, int epilogue, int64
     if (M <= 64 && skinny_applicable((int)M, (int)N, (int)K, epilogue, ldo)) return kHeaderBytes;
     size_t big = 0;
     {
-        const BigPlan bp = big_plan((int)M, (int)N, (int)K, epilogue);
-        if (bp.tile) big = big_partial_bytes((int)M, (int)N, epilogue, bp);
+        for (int operand_w = 0; operand_w < 2; ++operand_w) {   // (the plan may depend on the weight layout)
+            const BigPlan bp = big_plan((int)M, (int)N, (int)K, epilogue, operand_w != 0);
+            const size_t b = bp.tile ? big_partial_bytes((int)M, (int)N, epilogue, bp) : 0;
+            big = b > big ? b : big;
+        }
     }
     const TileConfig c = pick_config((int)M, (int)N, (int)K, epilogue);
     const size_t own = partial_bytes(c, (int)M, (int)N, epilogue);
@@ -398,7 +401,7 @@ static GemmChoice choose_gemm(int M, int N, int K, int epilogue, int64_t ldo, bo
     };
     if (skinny_ok && M <= 64) return small();
     if (!tuning_env("PHYAI_FP8_TILE")) {
-        const BigPlan bp = big_plan(M, N, K, epilogue);
+        const BigPlan bp = big_plan(M, N, K, epilogue, layout != W_ROW_MAJOR);
         const bool few_small_tiles = bp.tile == 128 && bp.cols == 128 && bp.tiles <= 64 && !tuning_env("PHYAI_FP8_BIG");
         if (bp.tile && out16 && !(few_small_tiles && skinny_ok)) {
             c.kind = GemmChoice::BIG;
@@ -449,10 +452,10 @@ size_t gemm_scratch_need(const GemmProblem& g) {
     return choose_gemm(g).need;
 }
 
-int describe_gemm_plan(int M, int N, int K, int epilogue, char* buf, size_t n) {
+int describe_gemm_plan(int M, int N, int K, int epilogue, char* buf, size_t n, int weight_layout) {
     // operands that satisfy every alignment requirement, dense output
     const int64_t ldo = epi_is_gated(epilogue) ? N / 2 : N;
-    const GemmChoice c = choose_gemm(M, N, K, epilogue, ldo, true, ldo % 8 == 0, false);
+    const GemmChoice c = choose_gemm(M, N, K, epilogue, ldo, true, ldo % 8 == 0, false, weight_layout);
     switch (c.kind) {
     case GemmChoice::SKINNY:
         return snprintf(buf, n, "small-m nt=%d mb=%d kpw=%d rounds=%d", c.sk.nt, c.sk.mb, c.sk.kpw, c.sk.rounds);
@@ -471,7 +474,7 @@ int describe_linear_plan(int M, int N, int K, int epilogue, char* buf, size_t n,
         return snprintf(buf, n, "one launch: small-m rows=%d nt=%d kpw=%d grid=%dx%d", c.fq.rows, c.fq.nt, c.fq.kpw, c.fq.tiles, c.fq.msplit);
     const int len = snprintf(buf, n, "quantizer + ");
     if (len < 0 || (size_t)len >= n) return len;
-    return len + describe_gemm_plan(M, N, K, epilogue, buf + len, n - len);
+    return len + describe_gemm_plan(M, N, K, epilogue, buf + len, n - len, weight_layout);
 }
 
 int describe_mlp_plan(int M, int H, int I, int O, int epilogue, char* buf, size_t n, bool operand_order) {

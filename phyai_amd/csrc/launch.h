@@ -147,7 +147,7 @@ struct BigPlan {
     int tiles;   // output tiles of that size
     int depth;   // stages of the LDS ring
 };
-BigPlan big_plan(int M, int N, int K, int epilogue);
+BigPlan big_plan(int M, int N, int K, int epilogue, bool operand_w = false);
 size_t big_partial_bytes(int M, int N, int epilogue, const BigPlan& pl);
 int launch_gemm_big(const GemmProblem& p, const BigPlan& pl, hipStream_t st);
 
@@ -158,6 +158,6 @@ int launch_set_stamp_sink_fused(unsigned long long* buf, unsigned int records);
 // Text form of what phyai_fp8_mlp launches for aligned, row-major operands.
 int describe_mlp_plan(int M, int H, int I, int O, int epilogue, char* buf, size_t n, bool operand_order = false);
 // Text form of launch_gemm's choice for aligned operands and a dense output; returns its length.
-int describe_gemm_plan(int M, int N, int K, int epilogue, char* buf, size_t n);
+int describe_gemm_plan(int M, int N, int K, int epilogue, char* buf, size_t n, int weight_layout = 0);
 
 }  // namespace phyai

@@ -112,12 +112,15 @@ def workspace_bytes(M: int, N: int, K: int, epilogue=EPI_NONE) -> int:
     return int(_lib.load().phyai_fp8_linear_workspace_bytes(M, N, K, _epi("workspace_bytes", epilogue)))
 
 
-def describe_plan(M: int, N: int, K: int, epilogue=EPI_NONE) -> str:
-    """Which kernel the GEMM entry point would launch for this problem (host only, no GPU needed)."""
+def describe_plan(M: int, N: int, K: int, epilogue=EPI_NONE, weight_layout: str | None = None) -> str:
+    """Which kernel the GEMM entry point would launch for this problem and a weight in the given layout (host only,
+    no GPU needed)."""
     import ctypes
 
     buf = ctypes.create_string_buffer(128)
-    rc = _lib.load().phyai_fp8_describe_plan(M, N, K, _epi("describe_plan", epilogue), buf, len(buf))
+    epi = _epi("describe_plan", epilogue)
+    flag = _layout_flag("describe_plan", weight_layout, epi) if weight_layout else 0
+    rc = _lib.load().phyai_fp8_describe_plan(M, N, K, epi | flag, buf, len(buf))
     if rc < 0:
         raise _err("describe_plan", _lib.load().phyai_fp8_last_error().decode())
     return buf.value.decode()
