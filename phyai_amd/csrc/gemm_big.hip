@@ -600,20 +600,26 @@ void gemm_fp8_big_kernel(
         constexpr int FRAG = TM * TN * 16, CHUNK = 32;
         const int S = n_splits;
         const int tile = tile_id.m * p.n_tiles + tile_id.n;
+        auto publish = [&]() {
 #pragma unroll
-        for (int c = 0; c < TM * TN / 2; ++c) {
-            float frag[CHUNK];
+            for (int c = 0; c < TM * TN / 2; ++c) {
+                float frag[CHUNK];
 #pragma unroll
-            for (int r = 0; r < 32; ++r) frag[r] = acc[(2 * c) / TN][(2 * c) % TN + r / 16][r % 16];
-            splitk_publish_part<FRAG, 256, CHUNK>(p.partials, tile, S, split_z, c * CHUNK, frag);
-        }
-        wait_own_stores();
-        // splitk_arrive opens with a barrier, after which nobody reads operands any more: a word
-        // of the ring serves as its flag
-        if (!splitk_arrive(p.counters, tile, S, reinterpret_cast<int*>(lds))) return;
+                for (int r = 0; r < 32; ++r) frag[r] = acc[(2 * c) / TN][(2 * c) % TN + r / 16][r % 16];
+                splitk_publish_part<FRAG, 256, CHUNK>(p.partials, tile, S, split_z, c * CHUNK, frag);
+            }
+            wait_own_stores();
+        };
         // gather: as much of the fragment per round trip as the registers allow
         constexpr int GCH = FRAG <= 64 ? FRAG : 32;
-        if (S == 2) {   // (uniform) the own half is still in the accumulators: only the other one is read
+        if (S == 2) {   // (uniform) two splits: the first to arrive writes its half, the second adds it to its own
+            const int found = splitk_arrive_early(p.counters, tile, reinterpret_cast<int*>(lds));
+            if (found == 0) {
+                publish();
+                splitk_published(p.counters, tile);
+                return;
+            }
+            splitk_await_published(p.counters, tile, found);
 #pragma unroll
             for (int c = 0; c < FRAG / GCH; ++c) {
                 float frag[GCH];
@@ -625,6 +631,10 @@ void gemm_fp8_big_kernel(
                 }
             }
         } else {
+            publish();
+            // splitk_arrive opens with a barrier, after which nobody reads operands any more: a word
+            // of the ring serves as its flag
+            if (!splitk_arrive(p.counters, tile, S, reinterpret_cast<int*>(lds))) return;
 #pragma unroll
             for (int c = 0; c < FRAG / GCH; ++c) {
                 float frag[GCH];

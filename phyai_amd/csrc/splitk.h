@@ -87,6 +87,40 @@ __device__ __forceinline__ bool splitk_arrive(int* counters, int tile, int S, in
     return *s_flag != 0;
 }
 
+// A tile split in two, the other way round: arrive first, publish only if nobody was there.  The first of the two
+// workgroups to arrive (it finds 0) writes its partial sums, waits for its stores (wait_own_stores) and then tells so
+// with splitk_published(); the second (it finds 1, or 3 if the first has told already) writes nothing: it waits
+// until the first has told, reads that half and adds it to the accumulators it still holds.  Half of the partial
+// sums are never written.  The first workgroup runs to its end without waiting for anyone, so the second cannot
+// wait for ever; its spin is bounded all the same (giving up would add a half that is not there yet: wrong
+// numbers, never a hang).  The argument above carries over: the first workgroup's stores are acknowledged by the
+// memory side before its second add to the counter, and the second workgroup's loads are issued after it has read
+// a counter value that contains that add.
+__device__ __forceinline__ int splitk_arrive_early(int* counters, int tile, int* s_flag) {
+    __syncthreads();   // (nobody reads operands from LDS any more: a word of it serves as the flag)
+    if (threadIdx.x == 0)
+        *s_flag = __hip_atomic_fetch_add(counters + tile, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    __syncthreads();
+    return *s_flag;
+}
+
+// All threads of the first workgroup, each after wait_own_stores().
+__device__ __forceinline__ void splitk_published(int* counters, int tile) {
+    __syncthreads();
+    if (threadIdx.x == 0) __hip_atomic_fetch_add(counters + tile, 2, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+}
+
+// All threads of the second workgroup; `found` is what splitk_arrive_early returned.
+__device__ __forceinline__ void splitk_await_published(int* counters, int tile, int found) {
+    if (found == 1 && threadIdx.x == 0) {
+        for (int spin = 0; spin < (1 << 22); ++spin) {
+            if (__hip_atomic_load(counters + tile, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) >= 4) break;
+            __builtin_amdgcn_s_sleep(8);
+        }
+    }
+    __syncthreads();
+}
+
 // Sum of elements e0 .. e0+CHUNK-1 over the S partials of a tile, in split order.  The loads of
 // two partials are in flight together: every batch of loads is a round trip to memory, and the
 // round trips, not the bytes, are what the gathering workgroup waits for.
