@@ -25,6 +25,12 @@
 //    with its MFMA pipe empty.  One barrier per stage-load, placed in its second K half: it
 //    publishes the next stage and tells everyone that the stage about to be refilled is no
 //    longer read.  All wavefronts reach it at about the same time, with MFMAs queued.
+//    Where the weights are in MFMA operand order and a wavefront owns its column blocks
+//    (wavefronts 1 x 4: the 224 x 256 tile, and 128 x 128 tiles as 4 x 1 blocks per wavefront)
+//    they do not go through LDS at all - each wavefront loads its own weight blocks straight into
+//    a ring of register sets - and the barrier gives way to a hand-over through one progress word
+//    per wavefront in LDS, which lets a wavefront run a stage or two ahead of the slowest
+//    (see `hand_over` in the kernel).
 //  * the operand blocks that open the next K half are read from LDS during the later row groups
 //    of the current one into a second register set, and inside a half the A blocks of the later
 //    row groups are read before the first group's MFMAs are issued, so ds_read latency overlaps
