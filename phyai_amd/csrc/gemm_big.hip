@@ -512,10 +512,10 @@ void gemm_fp8_big_kernel(
         };
         using S0 = std::integral_constant<int, 0>; using S1 = std::integral_constant<int, 1>;
         using S2 = std::integral_constant<int, 2>;
+        part(S0{}, CA, IDX_END);   // (the weights of stage-load 0 come from HBM: out first)
         part(S0{}, 0, CA);
         part(S1{}, 0, CA);
         if constexpr (CLAIM == 3) part(S2{}, 0, CA);
-        part(S0{}, CA, IDX_END);
         part(S1{}, CA, IDX_END);
         if constexpr (CLAIM == 3) part(S2{}, CA, IDX_END);
         if constexpr (CLAIM == 2) part(S2{}, 0, IDX_END);
@@ -531,6 +531,14 @@ void gemm_fp8_big_kernel(
             for (int c = 0; c < COPIES; ++c) issue(d, c, Slot0{});
 #pragma unroll
         for (int c = 0; c < HEAD_IDX; ++c) issue(DEPTH - 1, c, Slot0{});
+    }
+    // (the large tiles' 224 - 256 accumulators are zeroed here, under the first stage-load's latency: left to the
+    // compiler they are zeroed behind the wait, 1 - 2 k cycles in which nothing else happens)
+    if constexpr (TM * TN >= 14) {
+#pragma unroll
+        for (int i = 0; i < TM; ++i)
+#pragma unroll
+            for (int j = 0; j < TN; ++j) asm volatile("" : "+a"(acc[i][j]));
     }
     if constexpr (BDIRECT) {
         // stage-load 0 and the activations up to stage-load CLAIM - 1 have landed (what progress word -1 stands for)
