@@ -16,6 +16,12 @@ returns a list of violations over every instantiation of the kernel:
 * the number of vector-memory instructions between the last invisible load and that wait differs from the
   wait's ``N``;
 * the kernel uses scratch memory (a spilled register in that stretch could be one of the loads').
+
+``check_tile_usage`` is the guard of gemm_big.hip, whose global -> LDS copies are inline assembly too and whose
+``s_waitcnt vmcnt(N)`` count, by hand, the vector-memory instructions of a wavefront in issue order: a kernel of that
+file that spills has scratch loads and stores of the compiler's among them, and a wait would then let a stage be
+read before it has landed.  It reads the compiler's resource-usage remarks that the Makefile keeps beside every
+object (``_obj/gemm_big.o.usage``) and reports every instantiation with a scratch size other than zero.
 """
 
 from __future__ import annotations
@@ -139,10 +145,35 @@ def check_file(make: bool = True, stamps: bool = False) -> list[str]:
     return check_text(open(os.path.join(CSRC, target), encoding="utf-8").read())
 
 
+def usage_problems(text: str, kernel: str = "gemm_fp8_big_kernel", min_kernels: int = 50) -> list[str]:
+    """Kernels named `kernel` whose resource-usage remarks (-Rpass-analysis=kernel-resource-usage) show scratch."""
+    bad, seen, name = [], 0, None
+    for line in text.split("\n"):
+        m = re.search(r"remark: Function Name: (\S+)", line)
+        if m:
+            name = m.group(1) if kernel in m.group(1) else None
+            seen += name is not None
+            continue
+        m = re.search(r"remark:\s+ScratchSize \[bytes/lane\]: (\d+)", line)
+        if m and name is not None and int(m.group(1)) != 0:
+            bad.append(f"{name}: {m.group(1)} bytes of scratch per lane")
+    if seen < min_kernels:
+        bad.append(f"only {seen} instantiations of {kernel} found in the resource-usage remarks")
+    return bad
+
+
+def check_tile_usage(stamps: bool = False) -> list[str]:
+    """The pipelined tile kernels of the built library (or of the time-stamp build) use no scratch memory."""
+    path = os.path.join(CSRC, "_obj", ("stamps_" if stamps else "") + "gemm_big.o.usage")
+    if not os.path.exists(path):
+        return [f"{path} is missing (make -C {CSRC} all stamps writes it)"]
+    return usage_problems(open(path, encoding="utf-8", errors="replace").read())
+
+
 if __name__ == "__main__":
     import sys
 
-    problems = check_file(stamps="--stamps" in sys.argv)
+    problems = check_file(stamps="--stamps" in sys.argv) + check_tile_usage(stamps="--stamps" in sys.argv)
     for p in problems[:50]:
         print(p)
     print(f"{len(problems)} problem(s)")

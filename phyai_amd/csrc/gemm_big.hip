@@ -947,7 +947,7 @@ BigPlan big_plan(int M, int N, int K, int epilogue, bool operand_w) {
     }
     if (const char* e = tuning_env("PHYAI_FP8_BIG_SPLITS")) {
         const int s = atoi(e);
-        if (pl.tile != 192 && pl.tile != 224 && pl.tile != 96 && pl.cols != 64 && s >= 1 && K % (s * 128) == 0 && K / s >= 512 && tiles * s <= 4096) pl.splits = s;
+        if (pl.tile == 128 && pl.cols == 128 && s >= 1 && K % (s * 128) == 0 && K / s >= 512 && tiles * s <= 4096) pl.splits = s;
     }
     if (const char* e = tuning_env("PHYAI_FP8_BIG_DEPTH")) {
         const int d = atoi(e);
@@ -1018,7 +1018,10 @@ static void big_launch(BigArgs a, const GemmProblem& g, int splits, hipStream_t 
 #define PHYAI_BIG_ARGS a.a, a.b, a.K, a.M, a.N, a.m_tiles, a.n_tiles, a.band, a.by_rows | (a.operand_w << 4), a.k_per_split, a.a_scale, \
                        a.b_scale, a.bias, a.out, a.ldo, a.a_scale_scalar, a.partials, a.counters, a.res
     if (splits > 1) {
-        if constexpr ((TM == TN && (TM == 4 || DEPTH == 4)) || (WMODE == 2 && TN == 1))
+        // (K splits: 128 x 128 tiles with a ring of four, staged or with weights in registers.  The 256 x 256 tile is
+        // not built with them: its 256 accumulators leave the gather no registers, and a kernel that spills has
+        // vector-memory instructions of the compiler's among the copies that the waits count by hand.)
+        if constexpr ((TM == TN && TM == 2 && DEPTH == 4) || (WMODE == 2 && TN == 1))
             hipLaunchKernelGGL((gemm_fp8_big_kernel<TM, TN, DEPTH, EPI, true, WGM, WGN, WMODE>), grid, dim3(256), 0, st, PHYAI_BIG_ARGS);
     } else {
         hipLaunchKernelGGL((gemm_fp8_big_kernel<TM, TN, DEPTH, EPI, false, WGM, WGN, WMODE>), grid, dim3(256), 0, st, PHYAI_BIG_ARGS);

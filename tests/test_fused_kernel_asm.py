@@ -62,3 +62,20 @@ def test_planted_violations_are_caught(guard, asm):
     # scratch
     planted = k + "\n\tscratch_store_dword off, v1, s0\n"
     assert any("scratch" in p for p in guard.check_kernel(planted, rows))
+
+
+def test_tile_kernels_use_no_scratch(guard):
+    """The pipelined tile kernels count their global -> LDS copies by hand (s_waitcnt vmcnt(N)): a spill would put
+    scratch loads and stores of the compiler's among them.  The Makefile keeps the compiler's resource-usage remarks
+    beside every object; the guard reads them (the library's build runs the same check)."""
+    usage = os.path.join(ROOT, "phyai_amd", "csrc", "_obj", "gemm_big.o.usage")
+    if not os.path.exists(usage):
+        pytest.skip("no resource-usage remarks here (the library was built elsewhere)")
+    assert not guard.check_tile_usage(), "\n".join(guard.check_tile_usage()[:20])
+    planted = ("x.hip:1:1: remark: Function Name: _ZN5phyai19gemm_fp8_big_kernelILi2ELi2EEEvv [-Rpass-analysis=kernel-resource-usage]\n"
+               "x.hip:1:1: remark:     ScratchSize [bytes/lane]: 268 [-Rpass-analysis=kernel-resource-usage]\n"
+               "x.hip:1:1: remark: Function Name: _ZN5phyai5otherEv [-Rpass-analysis=kernel-resource-usage]\n"
+               "x.hip:1:1: remark:     ScratchSize [bytes/lane]: 16 [-Rpass-analysis=kernel-resource-usage]\n")
+    bad = guard.usage_problems(planted, min_kernels=1)
+    assert len(bad) == 1 and "268 bytes" in bad[0]
+    assert any("only 1" in p for p in guard.usage_problems(planted, min_kernels=2))

@@ -507,9 +507,9 @@ def test_weight_streaming_kernel_workgroup_shapes_agree_bit_for_bit(dev, monkeyp
             assert_close_to_ref(outs[None], want, f"case {case} {(M, N, K, epi_name)}")
 
 
-@pytest.mark.parametrize("tile", ["128", "256"])
+@pytest.mark.parametrize("tile", ["128"])
 def test_big_tile_kernel_split_k(dev, monkeypatch, tile):
-    """Both tile sizes with the K range split over two and four workgroups (partials in the workspace)."""
+    """The K range split over two and four workgroups (partials in the workspace)."""
     ops = _ops()
     monkeypatch.setenv("PHYAI_FP8_BIG", tile)
     x, wq, ws, b = _problem(300, 384, 4096, seed=77)
@@ -571,7 +571,7 @@ def _as_bits(t):
     return t.contiguous().view(torch.int16)
 
 
-@pytest.mark.parametrize("force,shape", [(("PHYAI_FP8_BIG", "128"), (300, 384, 4096)), (("PHYAI_FP8_BIG", "256"), (300, 384, 4096)),
+@pytest.mark.parametrize("force,shape", [(("PHYAI_FP8_BIG", "128"), (300, 384, 4096)), (("PHYAI_FP8_BIG", "128"), (816, 2048, 8192)),
                                          (("PHYAI_FP8_TILE", "128,128,4"), (200, 512, 1040))])
 def test_split_k_many_runs_one_result(dev, monkeypatch, force, shape):
     """The split-K hand-over (write-through partial sums, own-store wait, barrier, arrival counter,
@@ -595,7 +595,7 @@ def test_split_k_many_runs_one_result(dev, monkeypatch, force, shape):
 
 
 @pytest.mark.parametrize("M,N,K,tile,splits", [(816, 2048, 16384, "", ""), (816, 2048, 8192, "128", "2"), (300, 1024, 4096, "128", "4"),
-                                               (300, 2048, 4096, "128", "8"), (520, 2048, 4096, "256", "2"), (300, 768, 4096, "128", "4")])
+                                               (300, 2048, 4096, "128", "8"), (520, 2048, 4096, "128", "2"), (300, 768, 4096, "128", "4")])
 def test_split_k_with_an_xcd_per_k_range_gives_the_same_bits(dev, monkeypatch, M, N, K, tile, splits):
     """Split-K launches can hand every XCD one K range (its L2 then fetches that range of the activation
     codes once) instead of whole tile columns; the tiles, the K ranges and the order in which the partial
