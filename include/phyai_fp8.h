@@ -274,6 +274,8 @@ int phyai_fp8_adarmsnorm_quant(const void *x, int64_t ldx, const void *modulatio
  * dense output (ldo = output width): a short text such as
  *   "small-m nt=2 mb=4 kpw=1 rounds=1"      weight-streaming kernel
  *   "tile 192x128 depth=2 splits=1 tiles=2304"   pipelined tile kernel
+ *   "tile 224x256 depth=2 splits=1 tiles=512 weights in registers, ring of 4"   the same with weights in
+ *       operand order loaded straight into registers and no barrier in the main loop
  *   "generic 128x128 splits=2"               fallback tile kernel
  * written to buf (at most n bytes, always terminated).  Host only: nothing is launched, no GPU is
  * needed.  The layout flag of the weight matrix (PHYAI_FP8_FLAG_W_OPERAND_ORDER / _GATED) may be

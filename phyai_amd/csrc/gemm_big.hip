@@ -850,7 +850,7 @@ static double big_fill(int tiles, int slots) {
 }
 
 BigPlan big_plan(int M, int N, int K, int epilogue, bool operand_w) {
-    BigPlan pl = {0, 0, 1, 0, 0};
+    BigPlan pl = {0, 0, 1, 0, 0, 0};
     if (K % 128 != 0 || K < 512) return pl;   // slabs come in pairs and must fill the ring
     int forced = -1;
     if (const char* e = tuning_env("PHYAI_FP8_BIG")) forced = atoi(e);   // "0": never; "256"/"192"/"128": force
@@ -952,6 +952,16 @@ BigPlan big_plan(int M, int N, int K, int epilogue, bool operand_w) {
     if (const char* e = tuning_env("PHYAI_FP8_BIG_DEPTH")) {
         const int d = atoi(e);
         if (pl.tile == 128 && pl.cols == 128 && pl.splits == 1 && (d == 2 || d == 4)) pl.depth = d;
+    }
+    // Weights in operand order and a whole number of trips round the ring per K range: the wavefronts load their own
+    // weight blocks straight into registers (PHYAI_FP8_BIG_DIRECT=0: stage them like the rest).  224 x 256 tiles: ring
+    // of four.  128 x 128 tiles with a ring of four LDS stages and a plain epilogue: wavefronts 1 x 4 with one column
+    // block each and a ring of eight.  (Not the 96 x 128 tile: its main loop gains what its longer prologue - six
+    // stage-loads requested up front, at what the CU's vector-memory path passes - loses: 816 x 2560 x 2048 10.0 ->
+    // 10.1 us.)
+    if (operand_w && !(tuning_env("PHYAI_FP8_BIG_DIRECT") && atoi(tuning_env("PHYAI_FP8_BIG_DIRECT")) == 0)) {
+        if (pl.tile == 224 && pl.splits == 1 && K % 512 == 0) pl.regs = 4;
+        else if (pl.tile == 128 && pl.cols == 128 && pl.depth == 4 && (K / pl.splits) % 1024 == 0 && !epi_is_gated(epilogue)) pl.regs = 8;
     }
     return pl;
 }
@@ -1086,18 +1096,11 @@ int launch_gemm_big(const GemmProblem& g, const BigPlan& pl, hipStream_t st) {
     if (pl.splits > 1 && (g.workspace == nullptr ||
                           g.workspace_bytes < kGemmHeaderBytes + big_partial_bytes(g.M, g.N, g.epilogue, pl)))
         return -3;
-    if (pl.tile == 256) return big_launch_layout<4, 4, 2>(a, g, pl.splits, st);
-    // weights in operand order and a whole number of trips round the ring per K range: the wavefronts load
-    // their own weight blocks straight into registers (PHYAI_FP8_BIG_DIRECT=0: stage them like the rest)
-    const bool may_direct = a.operand_w && !(tuning_env("PHYAI_FP8_BIG_DIRECT") && atoi(tuning_env("PHYAI_FP8_BIG_DIRECT")) == 0);
-    // (ring of eight for 128 x 128 tiles, wavefronts 1 x 4 with one column block each; plain epilogues only.  Not for
-    // the 96 x 128 tile: its main loop gains what its longer prologue - six stage-loads requested up front, at
-    // what the CU's vector-memory path passes - loses: 816 x 2560 x 2048 10.0 -> 10.1 us)
-    const bool direct8 = may_direct && a.k_per_split % 1024 == 0 && !epi_is_gated(g.epilogue);
+    if (pl.tile == 256) return pl.splits == 1 ? big_launch_layout<4, 4, 2>(a, g, 1, st) : -2;
+    if (pl.regs != 0 && !a.operand_w) return -2;
     if (pl.tile == 224) {
-        const bool direct = may_direct && g.K % 512 == 0;
         if (pl.splits != 1) return -2;
-        if (direct) return big_launch_epi<7, 2, 4, 1, 4, 2>(a, g, 1, st);
+        if (pl.regs == 4) return big_launch_epi<7, 2, 4, 1, 4, 2>(a, g, 1, st);
         return big_launch_layout<7, 2, 2, 1, 4>(a, g, 1, st);
     }
     if (pl.tile == 192 && pl.splits == 1) return big_launch_layout<3, 2, 2>(a, g, 1, st);
@@ -1109,7 +1112,7 @@ int launch_gemm_big(const GemmProblem& g, const BigPlan& pl, hipStream_t st) {
         if (pl.splits != 1) return -2;
         return a.operand_w ? big_launch_plain<2, 1, 4, 2, 2, 1>(a, g, 1, st) : big_launch_plain<2, 1, 4, 2, 2, 0>(a, g, 1, st);
     }
-    if (pl.tile == 128 && pl.depth == 4 && direct8) return big_launch_plain<4, 1, 8, 1, 4, 2>(a, g, pl.splits, st);
+    if (pl.tile == 128 && pl.depth == 4 && pl.regs == 8) return big_launch_plain<4, 1, 8, 1, 4, 2>(a, g, pl.splits, st);
     if (pl.tile == 128 && pl.depth == 4) return big_launch_layout<2, 2, 4>(a, g, pl.splits, st);
     if (pl.tile == 128 && pl.splits == 1) return big_launch_layout<2, 2, 2>(a, g, 1, st);
     return -2;

@@ -460,6 +460,9 @@ int describe_gemm_plan(int M, int N, int K, int epilogue, char* buf, size_t n, i
     case GemmChoice::SKINNY:
         return snprintf(buf, n, "small-m nt=%d mb=%d kpw=%d rounds=%d", c.sk.nt, c.sk.mb, c.sk.kpw, c.sk.rounds);
     case GemmChoice::BIG:
+        if (c.big.regs)
+            return snprintf(buf, n, "tile %dx%d depth=%d splits=%d tiles=%d weights in registers, ring of %d", c.big.tile,
+                            c.big.cols, c.big.depth, c.big.splits, c.big.tiles, c.big.regs);
         return snprintf(buf, n, "tile %dx%d depth=%d splits=%d tiles=%d", c.big.tile, c.big.cols,
                         c.big.depth, c.big.splits, c.big.tiles);
     default:

@@ -146,6 +146,8 @@ struct BigPlan {
     int splits;
     int tiles;   // output tiles of that size
     int depth;   // stages of the LDS ring
+    int regs;    // weights in operand order loaded straight into a ring of this many register sets (4 or 8) by the
+                 // wavefront that owns the columns, the activation stages handed over without barriers; 0: staged through LDS
 };
 BigPlan big_plan(int M, int N, int K, int epilogue, bool operand_w = false);
 size_t big_partial_bytes(int M, int N, int epilogue, const BigPlan& pl);
