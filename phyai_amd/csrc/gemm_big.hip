@@ -610,10 +610,14 @@ void gemm_fp8_big_kernel(
     // ---- split-K: publish partial sums; the last split to arrive adds them in split order --
     // Two blocks (32 floats per lane) at a time, so that the 4 x 4 variant never holds more than
     // that outside its accumulators.
+    // (K split in two) this workgroup arrived second: the half that the first one wrote is added where the epilogue
+    // reads the accumulators, block by block, the loads of the next block under the arithmetic of the current one
+    bool add_other = false;
+    const int sp_tile = tile_id.m * p.n_tiles + tile_id.n;
     if constexpr (SPLIT) {
         constexpr int FRAG = TM * TN * 16, CHUNK = 32;
         const int S = n_splits;
-        const int tile = tile_id.m * p.n_tiles + tile_id.n;
+        const int tile = sp_tile;
         auto publish = [&]() {
 #pragma unroll
             for (int c = 0; c < TM * TN / 2; ++c) {
@@ -634,16 +638,7 @@ void gemm_fp8_big_kernel(
                 return;
             }
             splitk_await_published(p.counters, tile, found);
-#pragma unroll
-            for (int c = 0; c < FRAG / GCH; ++c) {
-                float frag[GCH];
-                splitk_load_part<FRAG, 256, GCH>(p.partials, tile, 2, 1 - split_z, c * GCH, frag);
-#pragma unroll
-                for (int r = 0; r < GCH; ++r) {
-                    const int blk = (c * GCH + r) / 16;
-                    acc[blk / TN][blk % TN][r % 16] += frag[r];
-                }
-            }
+            add_other = true;
         } else {
             publish();
             // splitk_arrive opens with a barrier, after which nobody reads operands any more: a word
@@ -710,6 +705,14 @@ void gemm_fp8_big_kernel(
     }
     __syncthreads();  // every wavefront is done reading operands from LDS
     uint8_t* stg = lds + wave * STG_BYTES;
+    // the other workgroup's 16 partial sums of block (i, j) (element (i TN + j) 16 + r of its fragment, splitk.h)
+    auto other_half = [&](int i, int j, float* po) {
+        if constexpr (SPLIT) {
+            if (add_other) splitk_load_part<TM * TN * 16, 256, 16>(p.partials, sp_tile, 2, 1 - split_z, (i * TN + j) * 16, po);
+        }
+    };
+    // accumulator r of a block, with the other half where there is one (a + b: the sum in split order either way)
+    auto summed = [&](float a, const float* po, int r) { return SPLIT && add_other ? a + po[r] : a; };
     if constexpr (OPW && GATED) {
         // Weights in the gated operand order: rows 4p .. 4p+3 of a 16-row unit are gate columns 2p, 2p+1 and up
         // columns 2p, 2p+1.  Accumulator 4k + e of lane (l32, h) of block j is block row 8k + 4h + e, i.e. with
@@ -731,16 +734,22 @@ void gemm_fp8_big_kernel(
                     buk[k][b] = p.bias ? bf16_bits_to_f32(p.bias[half_n + n_safe + b]) : 0.f;
                 }
             }
+            float pn[16] = {};
+            other_half(0, j, pn);
 #pragma unroll
             for (int i = 0; i < TM; ++i) {
                 const int row = i * 32 + l32;
                 const int sw = (row / ROWS_PER_PASS) & (SLOTS - 1);
+                float po[16];
+#pragma unroll
+                for (int r = 0; r < 16; ++r) po[r] = pn[r];
+                if (i + 1 < TM) other_half(i + 1, j, pn);
 #pragma unroll
                 for (int k = 0; k < 4; ++k) {
-                    const float g0 = __builtin_fmaf(acc[i][j][4 * k + 0], sa[i] * sgk[k][0], bgk[k][0]);
-                    const float g1 = __builtin_fmaf(acc[i][j][4 * k + 1], sa[i] * sgk[k][1], bgk[k][1]);
-                    const float u0 = __builtin_fmaf(acc[i][j][4 * k + 2], sa[i] * suk[k][0], buk[k][0]);
-                    const float u1 = __builtin_fmaf(acc[i][j][4 * k + 3], sa[i] * suk[k][1], buk[k][1]);
+                    const float g0 = __builtin_fmaf(summed(acc[i][j][4 * k + 0], po, 4 * k + 0), sa[i] * sgk[k][0], bgk[k][0]);
+                    const float g1 = __builtin_fmaf(summed(acc[i][j][4 * k + 1], po, 4 * k + 1), sa[i] * sgk[k][1], bgk[k][1]);
+                    const float u0 = __builtin_fmaf(summed(acc[i][j][4 * k + 2], po, 4 * k + 2), sa[i] * suk[k][0], buk[k][0]);
+                    const float u1 = __builtin_fmaf(summed(acc[i][j][4 * k + 3], po, 4 * k + 3), sa[i] * suk[k][1], buk[k][1]);
                     // gate and up pass through bf16 first, as the two-launch form materialises them
                     const uint32_t g01 = pack_bf16x2(g0, g1), u01 = pack_bf16x2(u0, u1);
                     const float o0 = apply_act<EPI>(__uint_as_float(g01 << 16)) * __uint_as_float(u01 << 16);
@@ -761,19 +770,29 @@ void gemm_fp8_big_kernel(
             load_cols(n_safe, sg[g], bg[g]);
             if constexpr (GATED) load_cols(half_n + n_safe, su[g], bu[g]);
         }
+        float pn[16] = {}, un[16] = {};
+        other_half(0, j, pn);
+        if constexpr (GATED) other_half(0, j + TN / 2, un);
 #pragma unroll
         for (int i = 0; i < TM; ++i) {
             const int row = i * 32 + l32;
             const int sw = (row / ROWS_PER_PASS) & (SLOTS - 1);
+            float po[16], pu[16];
+#pragma unroll
+            for (int r = 0; r < 16; ++r) { po[r] = pn[r]; pu[r] = un[r]; }
+            if (i + 1 < TM) {
+                other_half(i + 1, j, pn);
+                if constexpr (GATED) other_half(i + 1, j + TN / 2, un);
+            }
 #pragma unroll
             for (int g = 0; g < 4; ++g) {
                 float o[4];
 #pragma unroll
-                for (int e = 0; e < 4; ++e) o[e] = __builtin_fmaf(acc[i][j][4 * g + e], sa[i] * sg[g][e], bg[g][e]);
+                for (int e = 0; e < 4; ++e) o[e] = __builtin_fmaf(summed(acc[i][j][4 * g + e], po, 4 * g + e), sa[i] * sg[g][e], bg[g][e]);
                 if constexpr (GATED) {
                     float u[4];
 #pragma unroll
-                    for (int e = 0; e < 4; ++e) u[e] = __builtin_fmaf(acc[i][j + TN / 2][4 * g + e], sa[i] * su[g][e], bu[g][e]);
+                    for (int e = 0; e < 4; ++e) u[e] = __builtin_fmaf(summed(acc[i][j + TN / 2][4 * g + e], pu, 4 * g + e), sa[i] * su[g][e], bu[g][e]);
                     // gate and up pass through bf16 first, as the two-launch form materialises them
                     const uint32_t g01 = pack_bf16x2(o[0], o[1]), g23 = pack_bf16x2(o[2], o[3]);
                     const uint32_t u01 = pack_bf16x2(u[0], u[1]), u23 = pack_bf16x2(u[2], u[3]);
