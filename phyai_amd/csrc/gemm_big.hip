@@ -182,7 +182,9 @@ __device__ __forceinline__ v8i big_frag_operand(const uint8_t* buf, int row, int
 
 // Variants held to the register and LDS budget of two workgroups per CU (two wavefronts per SIMD).
 __host__ __device__ constexpr bool big_two_per_cu(int tm, int tn, int depth, int wmode) {
-    return depth == 2 && tm < 4;
+    // (... and the 128 x 128 tile as 4 x 1 blocks per wavefront with weights in registers and a ring of four: 64 KB of
+    // LDS, 64 accumulators)
+    return (depth == 2 && tm < 4) || (wmode == 2 && tm == 4 && tn == 1 && depth == 4);
 }
 
 // DEPTH: stages of the LDS ring, each holding BIG_BK bytes of K for the whole tile.
@@ -981,6 +983,8 @@ BigPlan big_plan(int M, int N, int K, int epilogue, bool operand_w) {
     if (operand_w && !(tuning_env("PHYAI_FP8_BIG_DIRECT") && atoi(tuning_env("PHYAI_FP8_BIG_DIRECT")) == 0)) {
         if (pl.tile == 224 && pl.splits == 1 && K % 512 == 0) pl.regs = 4;
         else if (pl.tile == 128 && pl.cols == 128 && pl.depth == 4 && (K / pl.splits) % 1024 == 0 && !epi_is_gated(epilogue)) pl.regs = 8;
+        // (more tiles than CUs: two workgroups per CU, each with a ring of four)
+        else if (pl.tile == 128 && pl.cols == 128 && pl.depth == 2 && pl.splits == 1 && K % 512 == 0 && !epi_is_gated(epilogue)) pl.regs = 4;
     }
     return pl;
 }
@@ -1050,7 +1054,7 @@ static void big_launch(BigArgs a, const GemmProblem& g, int splits, hipStream_t 
         // (K splits: 128 x 128 tiles with a ring of four, staged or with weights in registers.  The 256 x 256 tile is
         // not built with them: its 256 accumulators leave the gather no registers, and a kernel that spills has
         // vector-memory instructions of the compiler's among the copies that the waits count by hand.)
-        if constexpr ((TM == TN && TM == 2 && DEPTH == 4) || (WMODE == 2 && TN == 1))
+        if constexpr ((TM == TN && TM == 2 && DEPTH == 4) || (WMODE == 2 && TN == 1 && !big_two_per_cu(TM, TN, DEPTH, WMODE)))
             hipLaunchKernelGGL((gemm_fp8_big_kernel<TM, TN, DEPTH, EPI, true, WGM, WGN, WMODE>), grid, dim3(256), 0, st, PHYAI_BIG_ARGS);
     } else {
         hipLaunchKernelGGL((gemm_fp8_big_kernel<TM, TN, DEPTH, EPI, false, WGM, WGN, WMODE>), grid, dim3(256), 0, st, PHYAI_BIG_ARGS);
@@ -1132,6 +1136,7 @@ int launch_gemm_big(const GemmProblem& g, const BigPlan& pl, hipStream_t st) {
         return a.operand_w ? big_launch_plain<2, 1, 4, 2, 2, 1>(a, g, 1, st) : big_launch_plain<2, 1, 4, 2, 2, 0>(a, g, 1, st);
     }
     if (pl.tile == 128 && pl.depth == 4 && pl.regs == 8) return big_launch_plain<4, 1, 8, 1, 4, 2>(a, g, pl.splits, st);
+    if (pl.tile == 128 && pl.depth == 2 && pl.regs == 4 && pl.splits == 1) return big_launch_plain<4, 1, 4, 1, 4, 2>(a, g, 1, st);
     if (pl.tile == 128 && pl.depth == 4) return big_launch_layout<2, 2, 4>(a, g, pl.splits, st);
     if (pl.tile == 128 && pl.splits == 1) return big_launch_layout<2, 2, 2>(a, g, 1, st);
     return -2;

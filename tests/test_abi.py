@@ -135,14 +135,17 @@ def test_kernel_selection_for_the_benchmark_shapes(monkeypatch):
     assert d(1632, 2048, 2048, None, op) == "tile 128x128 depth=4 splits=1 tiles=208" + R8
     assert d(1632, 2048, 2048 + 512, None, op) == "tile 128x128 depth=4 splits=1 tiles=208"  # K not a multiple of 1024
     assert d(816, 4096, 2048, "geglu_tanh", og) == "tile 128x128 depth=4 splits=1 tiles=224" # gated: staged
+    assert d(1632, 2560, 2048, None, op) == "tile 128x128 depth=2 splits=1 tiles=260" + R4
+    assert d(1632, 2560, 2048 + 128, None, op) == "tile 128x128 depth=2 splits=1 tiles=260"  # K not a multiple of 512
+    assert d(800, 8192, 1024, "geglu_tanh", og) == "tile 128x128 depth=2 splits=1 tiles=448" # gated: staged
     assert d(6528, 2048, 16384, None, op) == "tile 224x256 depth=2 splits=1 tiles=240" + R4
     assert d(13056, 2048, 16384, None, op) == "tile 224x256 depth=2 splits=1 tiles=472" + R4
     assert d(4800, 2048, 8192, None, op) == "tile 224x256 depth=2 splits=1 tiles=176" + R4
     assert d(6528, 4096, 4096, "gelu", op) == "tile 224x256 depth=2 splits=1 tiles=480" + R4
     assert d(3264, 16384, 4096, "geglu_tanh", og) == "tile 224x256 depth=2 splits=1 tiles=960" + R4
     assert d(2048, 8192, 8192, None, op) == "tile 256x256 depth=2 splits=1 tiles=256"      # 320 tiles of 224 rows: a second round, mostly empty
-    assert d(8000, 1024, 8192, None, op) == "tile 128x128 depth=2 splits=1 tiles=504"      # 144 tiles of 224 x 256: too few
-    assert d(3264, 2048, 16384, None, op) == "tile 128x128 depth=2 splits=1 tiles=416"
+    assert d(8000, 1024, 8192, None, op) == "tile 128x128 depth=2 splits=1 tiles=504" + R4  # 144 tiles of 224 x 256: too few
+    assert d(3264, 2048, 16384, None, op) == "tile 128x128 depth=2 splits=1 tiles=416" + R4   # two workgroups per CU, each with its ring
     assert d(816, 2048, 16384, None, op) == "tile 128x128 depth=4 splits=2 tiles=112" + R8      # split launches stay
     assert d(6528, 32768, 2048, "geglu_tanh", og) == "tile 192x128 depth=2 splits=1 tiles=8704"   # K = 2048: two workgroups per CU keep their lead
     assert d(4800, 2048, 8192 + 128, None, op) == d(4800, 2048, 8192 + 128)                # K not a multiple of 512: no register path

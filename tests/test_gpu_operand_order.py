@@ -105,6 +105,8 @@ def _both_layouts(dev, M, N, K, epi, seed, *, residual=False):
 # kernel (on ready codes), every pipelined tile shape by automatic choice
 SHAPES = [
     (4800, 2048, 8192, None), (1632, 8192, 8192, "gelu"), (3264, 2048, 4096, "geglu_tanh"),   # 224 x 256 by the layout-aware rule
+    # more 128 x 128 tiles than CUs: 4 x 1 blocks per wavefront, weights in registers, ring of four, two workgroups per CU
+    (1632, 2560, 2048, None), (3264, 2048, 1536, "gelu"), (2100, 2048, 512, None), (2305, 2064, 1024, "gelu_tanh"),
     (50, 2560, 1024, None), (50, 1024, 2048, None), (50, 8192, 1024, "geglu_tanh"), (50, 1024, 4096, None),
     (1, 256, 128, None), (7, 272, 512, "gelu"), (33, 528, 2048, "gelu_tanh"), (64, 2048, 4096, "geglu_erf"),
     (100, 2560, 1024, None), (200, 1024, 4096, None), (400, 8192, 1024, "geglu_tanh"), (800, 1024, 2048, None),
